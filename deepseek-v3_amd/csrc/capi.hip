@@ -1,0 +1,81 @@
+// C ABI of libdsv3fp8.so: host-side argument validation and dispatch.
+// Everything is checked before the first HIP call so that the error paths are
+// usable (and tested) on a machine without a GPU.
+#include "common.hpp"
+
+using namespace dsv3;
+
+namespace {
+inline bool aligned(const void* p, uintptr_t a) { return ((uintptr_t)p % a) == 0; }
+inline bool valid_dtype(int d) { return d == DSV3_BF16 || d == DSV3_F16 || d == DSV3_F32; }
+}
+
+extern "C" {
+
+int dsv3_version(void) { return 100; }
+
+const char* dsv3_status_string(int status) {
+    switch (status) {
+        case DSV3_OK: return "ok";
+        case DSV3_ERR_NULL_POINTER: return "null pointer";
+        case DSV3_ERR_BAD_SHAPE: return "bad shape (negative size, or last dimension not a multiple of the block size)";
+        case DSV3_ERR_BAD_BLOCK: return "unsupported block size";
+        case DSV3_ERR_MISALIGNED: return "pointer not aligned as required";
+        case DSV3_ERR_BAD_DTYPE: return "unsupported dtype code";
+        case DSV3_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+        case DSV3_ERR_LAUNCH: return "HIP launch failed";
+        default: return "unknown status";
+    }
+}
+
+int dsv3_act_quant(const void* x, int x_dtype, void* y, float* s,
+                   int64_t numel, int64_t last_dim, int block_size,
+                   int scale_fmt, void* stream) {
+    if (!valid_dtype(x_dtype)) return DSV3_ERR_BAD_DTYPE;
+    if (scale_fmt != DSV3_SCALE_FMT_NONE && scale_fmt != DSV3_SCALE_FMT_UE8M0) return DSV3_ERR_BAD_DTYPE;
+    if (block_size != 32 && block_size != 64 && block_size != 128 && block_size != 256 && block_size != 512)
+        return DSV3_ERR_BAD_BLOCK;
+    if (numel < 0 || last_dim < 0) return DSV3_ERR_BAD_SHAPE;
+    if (last_dim % block_size != 0) return DSV3_ERR_BAD_SHAPE;
+    if (numel == 0) return DSV3_OK;
+    if (last_dim == 0 || numel % last_dim != 0) return DSV3_ERR_BAD_SHAPE;
+    if (!x || !y || !s) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(x, 16) || !aligned(y, 8) || !aligned(s, 4)) return DSV3_ERR_MISALIGNED;
+    return launch_act_quant(x, x_dtype, y, s, numel, block_size, scale_fmt, (hipStream_t)stream);
+}
+
+int dsv3_weight_dequant(const void* x, const float* s, void* y, int y_dtype,
+                        int64_t m, int64_t n, int block_size, void* stream) {
+    if (!valid_dtype(y_dtype)) return DSV3_ERR_BAD_DTYPE;
+    if (block_size < 1) return DSV3_ERR_BAD_BLOCK;
+    if (m < 0 || n < 0) return DSV3_ERR_BAD_SHAPE;
+    if (m == 0 || n == 0) return DSV3_OK;
+    if (!x || !s || !y) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(s, 4) || !aligned(y, y_dtype == DSV3_F32 ? 4 : 2)) return DSV3_ERR_MISALIGNED;
+    return launch_weight_dequant(x, s, y, y_dtype, m, n, block_size, (hipStream_t)stream);
+}
+
+size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+    if (m <= 0 || n <= 0 || k <= 0 || k % 128 != 0) return 0;
+    return fp8_gemm_workspace_bytes(m, n, k);
+}
+
+int dsv3_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
+                  void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                  void* workspace, size_t workspace_bytes, void* stream) {
+    if (!valid_dtype(c_dtype)) return DSV3_ERR_BAD_DTYPE;
+    if (m < 0 || n < 0 || k < 0) return DSV3_ERR_BAD_SHAPE;
+    if (k % 128 != 0) return DSV3_ERR_BAD_SHAPE;
+    if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (m == 0 || n == 0) return DSV3_OK;
+    if (!c) return DSV3_ERR_NULL_POINTER;
+    if (k > 0 && (!a || !a_s || !b || !b_s)) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(a, 16) || !aligned(b, 16) || !aligned(a_s, 4) || !aligned(b_s, 4) ||
+        !aligned(c, c_dtype == DSV3_F32 ? 16 : 8))
+        return DSV3_ERR_MISALIGNED;
+    const size_t need = dsv3_fp8_gemm_workspace_bytes(m, n, k);
+    if (need > 0 && (!workspace || workspace_bytes < need || !aligned(workspace, 256))) return DSV3_ERR_WORKSPACE;
+    return launch_fp8_gemm(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

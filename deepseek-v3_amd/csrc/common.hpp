@@ -1,0 +1,75 @@
+// Shared device helpers for the gfx950 kernels: vector types, bf16/fp16/fp8
+// conversions that map to single CDNA4 instructions, and launch plumbing.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include "../../include/dsv3_fp8.h"
+
+namespace dsv3 {
+
+typedef int      v2i  __attribute__((ext_vector_type(2)));
+typedef int      v4i  __attribute__((ext_vector_type(4)));
+typedef int      v8i  __attribute__((ext_vector_type(8)));
+typedef unsigned v2u  __attribute__((ext_vector_type(2)));
+typedef unsigned v4u  __attribute__((ext_vector_type(4)));
+typedef float    v2f  __attribute__((ext_vector_type(2)));
+typedef float    v4f  __attribute__((ext_vector_type(4)));
+typedef float    v16f __attribute__((ext_vector_type(16)));
+typedef __bf16   v2bf __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float u32_as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// Two bf16 packed in a dword -> two binary32 (exact widening).
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t p) { return u32_as_f32(p << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t p) { return u32_as_f32(p & 0xffff0000u); }
+
+// Two binary32 -> packed bf16, round-to-nearest-even (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    v2bf r = { (__bf16)lo, (__bf16)hi };
+    return __builtin_bit_cast(uint32_t, r);
+}
+// Two binary32 -> packed fp16, round-to-nearest-even.
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+    __half2 r = __floats2half2_rn(lo, hi);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// Four binary32 -> four OCP e4m3 bytes (v_cvt_pk_fp8_f32, RNE).
+__device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float d) {
+    int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+    return (uint32_t)r;
+}
+
+// e4m3 bytes of a dword -> binary32 (v_cvt_pk_f32_fp8 on the low / high half).
+__device__ __forceinline__ v2f fp8x2_lo_to_f32(uint32_t p) { return __builtin_amdgcn_cvt_pk_f32_fp8((int)p, false); }
+__device__ __forceinline__ v2f fp8x2_hi_to_f32(uint32_t p) { return __builtin_amdgcn_cvt_pk_f32_fp8((int)p, true); }
+
+// Output element writers: one binary32 -> C element of dsv3_dtype T.
+template <int DT> struct OutT;
+template <> struct OutT<DSV3_BF16> { typedef uint16_t type; static constexpr int bytes = 2; };
+template <> struct OutT<DSV3_F16>  { typedef uint16_t type; static constexpr int bytes = 2; };
+template <> struct OutT<DSV3_F32>  { typedef float    type; static constexpr int bytes = 4; };
+
+template <int DT> __device__ __forceinline__ typename OutT<DT>::type cvt_out(float v);
+template <> __device__ __forceinline__ uint16_t cvt_out<DSV3_BF16>(float v) { return (uint16_t)(pack_bf16(v, 0.f) & 0xffffu); }
+template <> __device__ __forceinline__ uint16_t cvt_out<DSV3_F16>(float v)  { return (uint16_t)(pack_f16(v, 0.f) & 0xffffu); }
+template <> __device__ __forceinline__ float    cvt_out<DSV3_F32>(float v)  { return v; }
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? DSV3_OK : DSV3_ERR_LAUNCH; }
+
+// Entry points of the individual kernel families (defined in the .hip files).
+int launch_act_quant(const void* x, int x_dtype, void* y, float* s, int64_t numel,
+                     int block_size, int scale_fmt, hipStream_t stream);
+int launch_weight_dequant(const void* x, const float* s, void* y, int y_dtype,
+                          int64_t m, int64_t n, int block_size, hipStream_t stream);
+int launch_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
+                    void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                    void* workspace, size_t workspace_bytes, hipStream_t stream);
+size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
+
+}  // namespace dsv3

@@ -1,0 +1,308 @@
+// fp8_gemm, large-M kernel for gfx950 (reference: inference/kernel.py:118-172).
+//
+//   c[m,n] = sum_kb ( sum_{t<128} a[m,128kb+t] * b[n,128kb+t] ) * a_s[m,kb] * b_s[n/128,kb]
+//
+// A workgroup owns a BM x BN tile of C and walks K in blocks of 128 -- exactly
+// one scale block -- staging the A rows and the B rows (both K-contiguous) in
+// LDS, double buffered.  Each wavefront computes a WM x WN sub-tile out of
+// 16x16 MFMA tiles with v_mfma_f32_16x16x128_f8f6f4: one instruction consumes a
+// whole scale block of K and returns its raw dot products, which are folded into
+// the binary32 accumulators with one FMA each by the block's scale.
+//
+// The MFMA is issued "transposed": the weight rows (n) are the instruction's A
+// operand and the activation rows (m) its B operand, so a lane's four results
+// share one m.  That makes the scale a single value per lane and 16-row
+// sub-tile ( a_s[m,kb] * b_s[n/128,kb] with the b_s factor uniform over the
+// workgroup because BN divides 128-aligned tiles ), and it makes a lane's four
+// results consecutive in n for the store.
+//
+// Both operands take their 32 bytes per lane from the same K offsets, so the
+// result does not depend on how the instruction numbers K internally.
+#include "common.hpp"
+
+namespace dsv3 {
+namespace {
+
+constexpr int kRowBytes = 128;           // one K block of fp8 per tile row
+constexpr int kRowStride = 128 + 16;     // padded: consecutive rows land in different banks
+
+__device__ __forceinline__ v8i join(v4i lo, v4i hi) {
+    v8i r = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+    return r;
+}
+
+template <int BM, int BN, int WM, int WN, int CD>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave, 2) void fp8_gemm_tile_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c,
+        int M, int N, int K, int tiles_m, int tiles_n, int kb_per_split) {
+    constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;
+    constexpr int THREADS = WAVES_M * WAVES_N * kWave;
+    constexpr int SM = WM / 16, SN = WN / 16;             // 16x16 sub-tiles per wave
+    constexpr int A_CHUNKS = BM * 8 / THREADS;            // 16-byte chunks a thread stages per K block
+    constexpr int B_CHUNKS = BN * 8 / THREADS;
+    constexpr int STAGE = (BM + BN) * kRowStride;
+    static_assert(BM * 8 % THREADS == 0 && BN * 8 % THREADS == 0, "tile/threads mismatch");
+    static_assert(BN <= 128 && 128 % BN == 0, "b_s must be uniform over the tile");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    // ---- workgroup -> tile: give each XCD (workgroups are dealt round-robin to the 8 XCDs)
+    // a contiguous run of tiles, and walk tiles in bands of GROUP_M tile-rows for L2 reuse.
+    const int T = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int q = T / 8, r = T % 8, x = pid % 8;
+        pid = x * q + (x < r ? x : r) + pid / 8;
+    }
+    constexpr int GROUP_M = 8;
+    const int band = pid / (GROUP_M * tiles_n);
+    const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+    const int in_band = pid - band * GROUP_M * tiles_n;
+    const int tm = band * GROUP_M + in_band % band_rows;
+    const int tn = in_band / band_rows;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    const int KB = K / 128;                       // row stride of both scale tensors
+    // split-K: blockIdx.y owns K blocks [kb0, kb0 + nkb) and writes its own [M,N] slab of c
+    const int kb0 = blockIdx.y * kb_per_split;
+    const int nkb = min(kb_per_split, KB - kb0);
+    c += (size_t)blockIdx.y * M * N;
+
+    // ---- global -> register staging: chunk id = i*THREADS + tid -> (row = id/8, chunk = id%8)
+    const uint8_t* a_src[A_CHUNKS];
+    const uint8_t* b_src[B_CHUNKS];
+    int a_dst[A_CHUNKS], b_dst[B_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+        const int id = i * THREADS + tid, row = id >> 3, ch = id & 7;
+        a_src[i] = a + (size_t)min(m0 + row, M - 1) * K + kb0 * 128 + ch * 16;
+        a_dst[i] = row * kRowStride + ch * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+        const int id = i * THREADS + tid, row = id >> 3, ch = id & 7;
+        b_src[i] = b + (size_t)min(n0 + row, N - 1) * K + kb0 * 128 + ch * 16;
+        b_dst[i] = BM * kRowStride + row * kRowStride + ch * 16;
+    }
+
+    // ---- per-lane scale sources: a_s[m, kb] for the lane's row of each 16-row sub-tile
+    const float* as_src[SM];
+#pragma unroll
+    for (int j = 0; j < SM; ++j)
+        as_src[j] = a_s + (size_t)min(m0 + wm * WM + j * 16 + (lane & 15), M - 1) * KB + kb0;
+    const float* bs_src = b_s + (size_t)(n0 / 128) * KB + kb0;
+
+    // ---- LDS read offsets of the lane's 32 bytes inside a tile row
+    const int frag_off = (lane & 15) * kRowStride + (lane >> 4) * 32;
+    const int a_rd = wm * WM * kRowStride + frag_off;
+    const int b_rd = BM * kRowStride + wn * WN * kRowStride + frag_off;
+
+    v4f acc[SN][SM];
+#pragma unroll
+    for (int i = 0; i < SN; ++i)
+#pragma unroll
+        for (int j = 0; j < SM; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    v4i a_st[A_CHUNKS], b_st[B_CHUNKS];
+    float as_cur[SM], as_nxt[SM];
+    float bs_cur, bs_nxt = 0.f;
+
+    // prologue: K block 0 -> LDS stage 0
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) a_st[i] = *(const v4i*)(a_src[i]);
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) b_st[i] = *(const v4i*)(b_src[i]);
+#pragma unroll
+    for (int j = 0; j < SM; ++j) as_cur[j] = as_src[j][0];
+    bs_cur = bs_src[0];
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) *(v4i*)(lds + a_dst[i]) = a_st[i];
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) *(v4i*)(lds + b_dst[i]) = b_st[i];
+    __syncthreads();
+
+    for (int kb = 0; kb < nkb; ++kb) {
+        const uint8_t* cur = lds + (kb & 1) * STAGE;
+        uint8_t* nxt = lds + ((kb + 1) & 1) * STAGE;
+        const bool more = kb + 1 < nkb;
+        if (more) {
+            const int ko = (kb + 1) * 128;
+#pragma unroll
+            for (int i = 0; i < A_CHUNKS; ++i) a_st[i] = *(const v4i*)(a_src[i] + ko);
+#pragma unroll
+            for (int i = 0; i < B_CHUNKS; ++i) b_st[i] = *(const v4i*)(b_src[i] + ko);
+#pragma unroll
+            for (int j = 0; j < SM; ++j) as_nxt[j] = as_src[j][kb + 1];
+            bs_nxt = bs_src[kb + 1];
+        }
+
+        v8i af[SM];
+#pragma unroll
+        for (int j = 0; j < SM; ++j) {
+            const uint8_t* p = cur + a_rd + j * 16 * kRowStride;
+            af[j] = join(*(const v4i*)p, *(const v4i*)(p + 16));
+        }
+        float sc[SM];
+#pragma unroll
+        for (int j = 0; j < SM; ++j) sc[j] = as_cur[j] * bs_cur;
+#pragma unroll
+        for (int i = 0; i < SN; ++i) {
+            const uint8_t* p = cur + b_rd + i * 16 * kRowStride;
+            const v8i bf = join(*(const v4i*)p, *(const v4i*)(p + 16));
+#pragma unroll
+            for (int j = 0; j < SM; ++j) {
+                const v4f z = {0.f, 0.f, 0.f, 0.f};
+                const v4f p4 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af[j], z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(p4[e], sc[j], acc[i][j][e]);
+            }
+        }
+
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < A_CHUNKS; ++i) *(v4i*)(nxt + a_dst[i]) = a_st[i];
+#pragma unroll
+            for (int i = 0; i < B_CHUNKS; ++i) *(v4i*)(nxt + b_dst[i]) = b_st[i];
+#pragma unroll
+            for (int j = 0; j < SM; ++j) as_cur[j] = as_nxt[j];
+            bs_cur = bs_nxt;
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds c[m][n .. n+3] per sub-tile
+    const bool vec_ok = (N % 4) == 0;
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        const int m = m0 + wm * WM + j * 16 + (lane & 15);
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < SN; ++i) {
+            const int n = n0 + wn * WN + i * 16 + (lane >> 4) * 4;
+            typename OutT<CD>::type* dst = c + (size_t)m * N + n;
+            if (vec_ok && n + 3 < N) {
+                if (CD == DSV3_F32) {
+                    *(v4f*)dst = acc[i][j];
+                } else if (CD == DSV3_BF16) {
+                    v2u o = { pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3]) };
+                    *(v2u*)dst = o;
+                } else {
+                    v2u o = { pack_f16(acc[i][j][0], acc[i][j][1]), pack_f16(acc[i][j][2], acc[i][j][3]) };
+                    *(v2u*)dst = o;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) dst[e] = cvt_out<CD>(acc[i][j][e]);
+            }
+        }
+    }
+}
+
+// Sums the split-K slabs in a fixed order and converts to the output type.
+template <int CD>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(
+        const float* __restrict__ ws, typename OutT<CD>::type* __restrict__ c, int64_t mn, int splits) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= mn) return;
+    float v = 0.f;
+    for (int s = 0; s < splits; ++s) v += ws[(int64_t)s * mn + i];
+    c[i] = cvt_out<CD>(v);
+}
+
+template <int BM, int BN, int WM, int WN, int CD>
+int launch_cfg(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+               int64_t m, int64_t n, int64_t k, int splits, int kb_per_split, hipStream_t stream) {
+    const int64_t tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
+    if (tm * tn > 0x7fffffff || splits > 65535) return DSV3_ERR_BAD_SHAPE;
+    auto kern = fp8_gemm_tile_kernel<BM, BN, WM, WN, CD>;
+    constexpr int lds_bytes = 2 * (BM + BN) * kRowStride;
+    // more than the default 64 KiB of dynamic LDS has to be granted once per device;
+    // the flag is idempotent, so a race between threads only repeats the same call
+    static bool granted[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
+    if (!granted[dev]) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+            return DSV3_ERR_LAUNCH;
+        granted[dev] = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn), (unsigned)splits), dim3((BM / WM) * (BN / WN) * kWave), lds_bytes, stream,
+                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c,
+                       (int)m, (int)n, (int)k, (int)tm, (int)tn, kb_per_split);
+    return launch_status();
+}
+
+// Split-K plan for skinny problems: enough workgroups to cover the chip a few times over,
+// but at least 4 K blocks per split.
+struct Plan { int bm; int splits; int kb_per_split; };
+
+Plan make_plan(int64_t m, int64_t n, int64_t k) {
+    Plan p;
+    p.bm = m <= 32 ? 32 : (m <= 64 ? 64 : 128);
+    const int64_t kb = k / 128;
+    p.splits = 1;
+    p.kb_per_split = (int)kb;
+    if (m <= 64 && kb > 0) {
+        const int64_t tiles = (n + 127) / 128;
+        const int64_t target = 1024;                       // workgroups wanted (256 CUs x 4)
+        int64_t s = (target + tiles - 1) / tiles;
+        int64_t max_s = kb / 4 > 0 ? kb / 4 : 1;
+        if (s > max_s) s = max_s;
+        if (s < 1) s = 1;
+        p.kb_per_split = (int)((kb + s - 1) / s);
+        p.splits = (int)((kb + p.kb_per_split - 1) / p.kb_per_split);
+    }
+    return p;
+}
+
+template <int CD>
+int launch_typed(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+                 int64_t m, int64_t n, int64_t k, void* ws, hipStream_t st) {
+    if (k == 0) {   // empty sum: c = 0
+        const int64_t mn0 = m * n;
+        hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn0 + 255) / 256)), dim3(256), 0, st,
+                           (const float*)nullptr, (typename OutT<CD>::type*)c, mn0, 0);
+        return launch_status();
+    }
+    const Plan p = make_plan(m, n, k);
+    if (p.splits == 1) {
+        if (p.bm == 32) return launch_cfg<32, 128, 32, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
+        if (p.bm == 64) return launch_cfg<64, 128, 64, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
+        return launch_cfg<128, 128, 64, 64, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
+    }
+    int rc;
+    if (p.bm == 32) rc = launch_cfg<32, 128, 32, 32, DSV3_F32>(a, a_s, b, b_s, ws, m, n, k, p.splits, p.kb_per_split, st);
+    else            rc = launch_cfg<64, 128, 64, 32, DSV3_F32>(a, a_s, b, b_s, ws, m, n, k, p.splits, p.kb_per_split, st);
+    if (rc != DSV3_OK) return rc;
+    const int64_t mn = m * n;
+    hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
+                       (const float*)ws, (typename OutT<CD>::type*)c, mn, p.splits);
+    return launch_status();
+}
+
+}  // namespace
+
+size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    const Plan p = make_plan(m, n, k);
+    return p.splits > 1 ? (size_t)p.splits * (size_t)m * (size_t)n * sizeof(float) : 0;
+}
+
+int launch_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
+                    void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                    void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    (void)workspace_bytes;
+    switch (c_dtype) {
+        case DSV3_BF16: return launch_typed<DSV3_BF16>(a, a_s, b, b_s, c, m, n, k, workspace, stream);
+        case DSV3_F16:  return launch_typed<DSV3_F16>(a, a_s, b, b_s, c, m, n, k, workspace, stream);
+        case DSV3_F32:  return launch_typed<DSV3_F32>(a, a_s, b, b_s, c, m, n, k, workspace, stream);
+        default: return DSV3_ERR_BAD_DTYPE;
+    }
+}
+
+}  // namespace dsv3

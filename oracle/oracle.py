@@ -1,0 +1,182 @@
+"""TEST INFRASTRUCTURE ONLY.
+
+torch-CPU restatement of the arithmetic of DeepSeek-V3's block-scaled FP8 path.
+Nothing in the shipped package imports this module; only ``tests/``, the smoke
+check and the bench's ``cpu_baseline`` leg do, and only as the checker.
+
+Each function cites the reference lines it restates (paths relative to the
+reference checkout).  All arithmetic is IEEE binary32 on the CPU:
+
+* ``act_quant``      inference/kernel.py:23-35, 51-57
+* ``weight_dequant`` inference/kernel.py:76-86, 104-110
+* ``fp8_gemm``       inference/kernel.py:145-172, 188-196
+* ``linear``         inference/model.py:131-163
+* ``gate``           inference/model.py:566-598
+* ``mlp`` / ``moe``  inference/model.py:532, 633, 669-693
+* ``block_quant_weight`` README_WEIGHTS.md:83-92 (zero padding of ragged blocks)
+
+Pinning (see tests/test_oracle_*.py): the conversions and all three kernels are
+checked against the independent plain-C restatement in ``dsv3_oracle.c`` and
+against closed-form known answers; nothing here is "parity unpinned" except the
+choice among equal scores in ``gate`` (torch.topk leaves ties unspecified; the
+workloads are generated without ties).
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+FP8 = torch.float8_e4m3fn
+FP8_MAX = 448.0
+BLOCK = 128
+
+
+def ue8m0_round_up(s: torch.Tensor) -> torch.Tensor:
+    """s -> 2^ceil(log2 s) for positive normal binary32 (kernel.py:29-31).
+
+    Defined on the bits so that it does not depend on a libm: a power of two is
+    kept, any other value moves up to the next power of two.
+    """
+    bits = s.contiguous().view(torch.int32)
+    exp = bits >> 23
+    mant = bits & 0x7FFFFF
+    exp = exp + (mant != 0).to(torch.int32)
+    return (exp << 23).view(torch.float32)
+
+
+def act_quant(x: torch.Tensor, block_size: int = BLOCK,
+              scale_fmt: Optional[str] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """kernel.py:23-35: per run of ``block_size`` contiguous elements
+    amax = max|x|, clamped below at 1e-4; s = amax / 448; y = e4m3(x / s)."""
+    assert x.is_contiguous()
+    assert x.size(-1) % block_size == 0
+    xf = x.float().view(-1, block_size)
+    amax = xf.abs().amax(dim=-1, keepdim=True)
+    amax = torch.maximum(amax, torch.tensor(1e-4, dtype=torch.float32))
+    s = amax / 448.0
+    if scale_fmt == "ue8m0":
+        s = ue8m0_round_up(s)
+    y = (xf / s).to(FP8).view(x.shape)
+    s = s.view(*x.shape[:-1], x.size(-1) // block_size)
+    return y, s
+
+
+def expand_block_scale(s: torch.Tensor, m: int, n: int, block_size: int = BLOCK) -> torch.Tensor:
+    """[ceil(m/b), ceil(n/b)] block scales -> [m, n] per-element scales."""
+    return s.repeat_interleave(block_size, 0)[:m].repeat_interleave(block_size, 1)[:, :n]
+
+
+def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = BLOCK,
+                   out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """kernel.py:83-86: y[i,j] = out_dtype( f32(x[i,j]) * s[i//b, j//b] )."""
+    assert x.is_contiguous() and s.is_contiguous()
+    assert x.dim() == 2 and s.dim() == 2
+    m, n = x.shape
+    return (x.float() * expand_block_scale(s, m, n, block_size)).to(out_dtype)
+
+
+def fp8_gemm_f32(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Tensor) -> torch.Tensor:
+    """kernel.py:157-166 in binary32, result left in binary32:
+    c = sum_kb (a_kb @ b_kb^T) * a_s[:, kb, None] * b_s[n//128, kb][None, :]."""
+    k = a.size(-1)
+    m = a.numel() // k
+    n = b.size(0)
+    assert k % BLOCK == 0
+    af = a.reshape(m, k).float()
+    bf = b.float()
+    asf = a_s.reshape(m, -1).float()
+    nb = torch.arange(n) // BLOCK
+    acc = torch.zeros(m, n, dtype=torch.float32)
+    for kb in range(k // BLOCK):
+        sl = slice(kb * BLOCK, (kb + 1) * BLOCK)
+        dot = af[:, sl] @ bf[:, sl].t()
+        acc += dot * asf[:, kb, None] * b_s[nb, kb][None, :]
+    return acc.view(*a.shape[:-1], n)
+
+
+def fp8_gemm(a, a_s, b, b_s, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """kernel.py:167 + 193: the binary32 accumulator cast to the output dtype."""
+    return fp8_gemm_f32(a, a_s, b, b_s).to(out_dtype)
+
+
+def block_quant_weight(w: torch.Tensor, block_size: int = BLOCK) -> Tuple[torch.Tensor, torch.Tensor]:
+    """README_WEIGHTS.md:83-92: per 128x128 block (ragged edge blocks are
+    zero-padded, which leaves their amax unchanged) scale = amax / 448 and
+    w8 = e4m3(w / scale); the stored scale is the dequantisation multiplier
+    (``weight_scale_inv``)."""
+    m, n = w.shape
+    mb, nb = -(-m // block_size), -(-n // block_size)
+    wp = torch.zeros(mb * block_size, nb * block_size, dtype=torch.float32)
+    wp[:m, :n] = w.float()
+    blocks = wp.view(mb, block_size, nb, block_size)
+    amax = blocks.abs().amax(dim=(1, 3))
+    amax = torch.maximum(amax, torch.tensor(1e-4, dtype=torch.float32))
+    s = amax / 448.0
+    w8 = (blocks / s[:, None, :, None]).view(mb * block_size, nb * block_size)[:m, :n].contiguous().to(FP8)
+    return w8, s
+
+
+def linear(x, weight, bias=None, scale=None, gemm_impl: str = "fp8",
+           scale_fmt: Optional[str] = None) -> torch.Tensor:
+    """model.py:153-163.  ``scale`` plays the role of ``weight.scale``."""
+    if weight.element_size() > 1:
+        return F.linear(x, weight, bias)
+    if gemm_impl == "bf16":
+        return F.linear(x, weight_dequant(weight, scale, out_dtype=x.dtype), bias)
+    xq, xs = act_quant(x, BLOCK, scale_fmt)
+    y = fp8_gemm(xq, xs, weight, scale, out_dtype=x.dtype)
+    if bias is not None:
+        y += bias
+    return y
+
+
+def mlp(x, w1, s1, w2, s2, w3, s3, scale_fmt=None) -> torch.Tensor:
+    """model.py:532 / 633: w2( silu(w1 x) * w3 x ) with fp8 linears."""
+    h = F.silu(linear(x, w1, scale=s1, scale_fmt=scale_fmt)) * linear(x, w3, scale=s3, scale_fmt=scale_fmt)
+    return linear(h, w2, scale=s2, scale_fmt=scale_fmt)
+
+
+def gate(x, gate_weight, gate_bias, topk: int, n_groups: int, topk_groups: int,
+         route_scale: float, score_func: str = "sigmoid"):
+    """model.py:576-598."""
+    scores = F.linear(x, gate_weight)
+    if score_func == "softmax":
+        scores = scores.softmax(dim=-1, dtype=torch.float32)
+    else:
+        scores = scores.sigmoid()
+    original = scores
+    if gate_bias is not None:
+        scores = scores + gate_bias
+    if n_groups > 1:
+        scores = scores.view(x.size(0), n_groups, -1)
+        if gate_bias is None:
+            group_scores = scores.amax(dim=-1)
+        else:
+            group_scores = scores.topk(2, dim=-1)[0].sum(dim=-1)
+        idx = group_scores.topk(topk_groups, dim=-1)[1]
+        mask = torch.ones(x.size(0), n_groups, dtype=torch.bool).scatter_(1, idx, False)
+        scores = scores.masked_fill(mask.unsqueeze(-1), float("-inf")).flatten(1)
+    indices = torch.topk(scores, topk, dim=-1)[1]
+    weights = original.gather(1, indices)
+    if score_func == "sigmoid":
+        weights = weights / weights.sum(dim=-1, keepdim=True)
+    weights = weights * route_scale
+    return weights.type_as(x), indices
+
+
+def moe(x, weights, indices, experts, shared, scale_fmt=None) -> torch.Tensor:
+    """model.py:679-693 at world_size 1.  ``experts`` is a list of
+    (w1, s1, w2, s2, w3, s3); ``shared`` is one such tuple."""
+    shape = x.shape
+    x = x.view(-1, shape[-1])
+    y = torch.zeros_like(x)
+    counts = torch.bincount(indices.flatten(), minlength=len(experts)).tolist()
+    for i, ex in enumerate(experts):
+        if counts[i] == 0:
+            continue
+        idx, top = torch.where(indices == i)
+        y[idx] += mlp(x[idx], *ex, scale_fmt=scale_fmt) * weights[idx, top, None]
+    z = mlp(x, *shared)   # the shared expert is an MLP of Column/RowParallelLinear: no scale_fmt (model.py:233,262)
+    return (y + z).view(shape)

@@ -1,0 +1,168 @@
+"""GPU parity: fp8_gemm through the C ABI vs the fp32 CPU oracle
+(reference arithmetic: inference/kernel.py:145-172).
+
+Tolerance: max|err| <= 1e-2 * rms(ref) on the binary32 accumulator output; the
+bf16 output must equal the round-to-nearest-even bf16 of the kernel's own
+binary32 output bit for bit (half a bf16 ulp at the output tail is larger than
+the tolerance, so the bf16 tensor is not compared with the fp32 reference)."""
+import pytest
+import torch
+
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def K():
+    import dsv3fp8
+    return dsv3fp8
+
+
+def _gemm_both(K, a, a_s, b, b_s):
+    c32 = K.fp8_gemm_f32(a, a_s, b, b_s)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        c16 = K.fp8_gemm(a, a_s, b, b_s)
+    finally:
+        torch.set_default_dtype(old)
+    return c32, c16
+
+
+def _check(K, x, w8, ws, fmt=None):
+    a_ref, as_ref = oracle.act_quant(x, 128, fmt)
+    ref = oracle.fp8_gemm_f32(a_ref, as_ref, w8, ws)
+    a, a_s = a_ref.cuda(), as_ref.cuda()
+    c32, c16 = _gemm_both(K, a, a_s, w8.cuda(), ws.cuda())
+    assert c32.dtype == torch.float32 and c16.dtype == torch.bfloat16
+    assert c32.shape == ref.shape == c16.shape
+    rms = ref.pow(2).mean().sqrt().item()
+    err = (c32.cpu() - ref).abs().max().item()
+    assert err <= TOL * rms, f"max|err| {err:.3e} > {TOL} * rms {rms:.3e}"
+    assert torch.equal(c16.cpu().view(torch.int16), c32.cpu().to(torch.bfloat16).view(torch.int16))
+    return err / rms
+
+
+DECODE = [(7168, 1536), (1536, 24576), (7168, 576), (512, 32768), (16384, 7168)]
+
+
+@pytest.mark.parametrize("kn", DECODE)
+@pytest.mark.parametrize("m", [1, 8, 32, 64])
+def test_decode_shapes(K, kn, m):
+    from dsv3fp8 import workloads
+    k, n = kn
+    x = workloads.activations(m, k, seed=m)
+    w8, ws = workloads.weight(n, k, seed=n % 97)
+    _check(K, x, w8, ws)
+
+
+@pytest.mark.parametrize("m", [65, 100, 128, 257, 300])
+def test_mid_m(K, m):
+    from dsv3fp8 import workloads
+    x = workloads.activations(m, 1024, seed=m)
+    w8, ws = workloads.weight(640, 1024, seed=3)
+    _check(K, x, w8, ws)
+
+
+@pytest.mark.parametrize("n", [1, 15, 16, 100, 129, 576, 577, 1000])
+def test_ragged_n(K, n):
+    from dsv3fp8 import workloads
+    for m in (5, 130):
+        x = workloads.activations(m, 512, seed=n)
+        w8, ws = workloads.weight(n, 512, seed=n + 1)
+        _check(K, x, w8, ws)
+
+
+def test_ragged_n_equals_prefix_of_padded(K):
+    """N=576 must equal the first 576 columns of the N=640 problem built from the same rows."""
+    from dsv3fp8 import workloads
+    x = workloads.activations(64, 7168, seed=1)
+    w8, ws = workloads.weight(640, 7168, seed=2)
+    a, a_s = oracle.act_quant(x)
+    a, a_s = a.cuda(), a_s.cuda()
+    full = K.fp8_gemm_f32(a, a_s, w8.cuda(), ws.cuda())
+    part = K.fp8_gemm_f32(a, a_s, w8[:576].contiguous().cuda(), ws.cuda())
+    assert torch.equal(full[:, :576], part)
+
+
+def test_leading_dims(K):
+    from dsv3fp8 import workloads
+    x = workloads.activations(6, 256, seed=1).view(2, 3, 256)
+    w8, ws = workloads.weight(192, 256, seed=2)
+    _check(K, x, w8, ws)
+
+
+def test_ue8m0_activation_scales(K):
+    from dsv3fp8 import workloads
+    x = workloads.activations(48, 2048, seed=8, outliers=True)
+    w8, ws = workloads.weight(2048, 2048, seed=9)
+    _check(K, x, w8, ws, fmt="ue8m0")
+
+
+def test_exact_small_integers(K):
+    """Small-integer fp8 values and power-of-two scales: every partial sum is exact in
+    binary32, so the result is independent of summation order -> bit-exact."""
+    g = torch.Generator().manual_seed(0)
+    for (m, n, k) in [(3, 130, 256), (64, 256, 1024), (200, 384, 512)]:
+        a = torch.randint(-4, 5, (m, k), generator=g).float().to(torch.float8_e4m3fn)
+        b = torch.randint(-4, 5, (n, k), generator=g).float().to(torch.float8_e4m3fn)
+        a_s = torch.pow(2.0, torch.randint(-3, 4, (m, k // 128), generator=g).float())
+        b_s = torch.pow(2.0, torch.randint(-3, 4, (-(-n // 128), k // 128), generator=g).float())
+        ref = oracle.fp8_gemm_f32(a, a_s, b, b_s)
+        c32 = K.fp8_gemm_f32(a.cuda(), a_s.cuda(), b.cuda(), b_s.cuda())
+        assert torch.equal(c32.cpu(), ref)
+
+
+def test_one_hot_picks_single_products(K):
+    """One-hot activation rows select single weight values times both scales."""
+    k, n = 384, 160
+    g = torch.Generator().manual_seed(1)
+    b = torch.randint(0, 0x7F, (n, k), generator=g, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    b_s = torch.rand(2, 3, generator=g) + 0.5
+    a = torch.zeros(16, k)
+    cols = torch.randint(0, k, (16,), generator=g)
+    a[torch.arange(16), cols] = 2.0
+    a = a.to(torch.float8_e4m3fn)
+    a_s = torch.rand(16, 3, generator=g) + 0.5
+    c = K.fp8_gemm_f32(a.cuda(), a_s.cuda(), b.cuda(), b_s.cuda()).cpu()
+    nb = torch.arange(n) // 128
+    for i in range(16):
+        kb = int(cols[i]) // 128
+        want = (2.0 * b.float()[:, cols[i]]) * a_s[i, kb] * b_s[nb, kb]
+        assert torch.allclose(c[i], want, rtol=3e-7, atol=0)
+
+
+def test_prefill_sampled(K):
+    """M=4096, 7168 -> 18432 at full size; the oracle evaluates a sample of rows/columns."""
+    from dsv3fp8 import workloads
+    x = workloads.activations(4096, 7168, seed=0, device="cuda")
+    w8, ws = workloads.weight(18432, 7168, seed=1, device="cuda")
+    a, a_s = K.act_quant(x)
+    c32, c16 = _gemm_both(K, a, a_s, w8, ws)
+    rows = torch.arange(5, 4096, 97, device="cuda")
+    cols = torch.cat([torch.arange(0, 256), torch.arange(9000, 9300), torch.arange(18432 - 200, 18432)]).cuda()
+    # the oracle needs whole 128-row scale blocks of b: evaluate per 128-aligned column block
+    ref_cols = []
+    for blk in torch.unique(cols // 128).tolist():
+        ref_cols.append(oracle.fp8_gemm_f32(a[rows].cpu(), a_s[rows].cpu(),
+                                            w8[blk * 128:(blk + 1) * 128].cpu(), ws[blk:blk + 1].cpu()))
+    ref = torch.cat(ref_cols, 1)
+    colidx = torch.cat([torch.arange(b * 128, (b + 1) * 128) for b in torch.unique(cols // 128).tolist()]).cuda()
+    got = c32[rows][:, colidx].cpu()
+    rms = ref.pow(2).mean().sqrt().item()
+    assert (got - ref).abs().max().item() <= TOL * rms
+    assert torch.equal(c16.view(torch.int16), c32.to(torch.bfloat16).view(torch.int16))
+
+
+def test_asserts_match_reference(K):
+    a = torch.zeros(4, 256, dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn)
+    a_s = torch.ones(4, 2, device="cuda")
+    b = torch.zeros(128, 256, dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn)
+    b_s = torch.ones(1, 2, device="cuda")
+    with pytest.raises(AssertionError):
+        K.fp8_gemm(a.t(), a_s, b, b_s)
+    with pytest.raises(AssertionError):
+        K.fp8_gemm(a, a_s.t(), b, b_s)
