@@ -1,0 +1,104 @@
+"""Host-side contract of libdsv3fp8.so: it loads without a GPU, exports every symbol
+include/dsv3_fp8.h declares, and validates arguments before touching HIP."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "dsv3_fp8.h"
+
+
+@pytest.fixture(scope="module")
+def L():
+    from dsv3fp8 import _lib
+    return _lib
+
+
+def test_exports_every_declared_symbol(L):
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    declared = set(re.findall(r"\b(dsv3_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(L.EXPORTS), (declared, set(L.EXPORTS))
+    for name in declared:
+        assert hasattr(L.lib, name)
+    assert L.lib.dsv3_version() >= 100
+
+
+def test_status_strings(L):
+    seen = {L.status_string(c) for c in range(8)}
+    assert len(seen) == 8 and "ok" in seen
+    assert L.status_string(12345) == "unknown status"
+
+
+A16 = 0x1000  # a fake, 16-byte aligned, non-null address: validation must reject before dereferencing
+
+
+def test_act_quant_validation(L):
+    f = L.lib.dsv3_act_quant
+    assert f(None, L.BF16, A16, A16, 128, 128, 128, 0, None) == 1
+    assert f(A16, L.BF16, None, A16, 128, 128, 128, 0, None) == 1
+    assert f(A16, L.BF16, A16, None, 128, 128, 128, 0, None) == 1
+    assert f(A16, L.BF16, A16, A16, 100, 100, 128, 0, None) == 2        # last dim % block (kernel.py:52)
+    assert f(A16, L.BF16, A16, A16, -128, 128, 128, 0, None) == 2
+    assert f(A16, L.BF16, A16, A16, 384, 256, 128, 0, None) == 2        # numel not a multiple of last dim
+    assert f(A16, L.BF16, A16, A16, 128, 128, 100, 0, None) == 3
+    assert f(A16 + 2, L.BF16, A16, A16, 128, 128, 128, 0, None) == 4
+    assert f(A16, 9, A16, A16, 128, 128, 128, 0, None) == 5
+    assert f(A16, L.BF16, A16, A16, 128, 128, 128, 7, None) == 5
+    assert f(None, L.BF16, None, None, 0, 128, 128, 0, None) == 0       # empty input: nothing to do
+
+
+def test_weight_dequant_validation(L):
+    f = L.lib.dsv3_weight_dequant
+    assert f(None, A16, A16, L.BF16, 128, 128, 128, None) == 1
+    assert f(A16, None, A16, L.BF16, 128, 128, 128, None) == 1
+    assert f(A16, A16, None, L.BF16, 128, 128, 128, None) == 1
+    assert f(A16, A16, A16, L.BF16, -1, 128, 128, None) == 2
+    assert f(A16, A16, A16, L.BF16, 128, 128, 0, None) == 3
+    assert f(A16, A16, A16, 5, 128, 128, 128, None) == 5
+    assert f(A16, A16, A16 + 1, L.BF16, 128, 128, 128, None) == 4
+    assert f(None, None, None, L.BF16, 0, 128, 128, None) == 0
+
+
+def test_fp8_gemm_validation(L):
+    f = L.lib.dsv3_fp8_gemm
+    ws = L.lib.dsv3_fp8_gemm_workspace_bytes
+    assert f(None, A16, A16, A16, A16, L.BF16, 4, 128, 128, None, 0, None) == 1
+    assert f(A16, A16, A16, A16, None, L.BF16, 4, 128, 128, None, 0, None) == 1
+    assert f(A16, A16, A16, A16, A16, L.BF16, 4, 128, 100, None, 0, None) == 2    # K % 128
+    assert f(A16, A16, A16, A16, A16, L.BF16, -4, 128, 128, None, 0, None) == 2
+    assert f(A16 + 8, A16, A16, A16, A16, L.BF16, 4, 128, 128, None, 0, None) == 4
+    assert f(A16, A16, A16, A16, A16, 3, 4, 128, 128, None, 0, None) == 5
+    assert f(None, None, None, None, None, L.BF16, 0, 128, 128, None, 0, None) == 0
+    need = ws(8, 1536, 7168)
+    assert need > 0 and ws(4096, 18432, 7168) == 0 and ws(0, 1, 128) == 0 and ws(8, 8, 100) == 0
+    assert f(A16, A16, A16, A16, A16, L.BF16, 8, 1536, 7168, None, 0, None) == 6
+    assert f(A16, A16, A16, A16, A16, L.BF16, 8, 1536, 7168, A16, need - 1, None) == 6
+    assert f(A16, A16, A16, A16, A16, L.BF16, 8, 1536, 7168, A16 + 16, need, None) == 6
+
+
+def test_ops_shape_inference_and_no_cpu_fallback():
+    import dsv3fp8  # noqa: F401  (registers the ops)
+    x = torch.empty(2, 3, 256, device="meta", dtype=torch.bfloat16)
+    y, s = torch.ops.dsv3fp8.act_quant(x, 128, 0)
+    assert y.shape == (2, 3, 256) and y.dtype == torch.float8_e4m3fn and s.shape == (2, 3, 2) and s.dtype == torch.float32
+    w = torch.empty(576, 256, device="meta", dtype=torch.float8_e4m3fn)
+    ws = torch.empty(5, 2, device="meta")
+    assert torch.ops.dsv3fp8.weight_dequant(w, ws, 128, 0).dtype == torch.bfloat16
+    c = torch.ops.dsv3fp8.fp8_gemm(y, s, w, ws, 0)
+    assert c.shape == (2, 3, 576) and c.dtype == torch.bfloat16
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.dsv3fp8.act_quant(torch.zeros(1, 128, dtype=torch.bfloat16), 128, 0)   # CPU tensors: no kernel
+
+
+def test_python_wrappers_keep_the_reference_asserts():
+    import dsv3fp8
+    x = torch.empty(4, 100, device="meta", dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="divisible by block_size"):
+        dsv3fp8.act_quant(x)
+    with pytest.raises(AssertionError, match="contiguous"):
+        dsv3fp8.act_quant(torch.empty(256, 4, device="meta", dtype=torch.bfloat16).t())
+    with pytest.raises(AssertionError, match="2 dimensions"):
+        dsv3fp8.weight_dequant(torch.empty(2, 4, 4, device="meta", dtype=torch.float8_e4m3fn), torch.empty(1, 1, device="meta"))
