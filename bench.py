@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-scaled FP8 path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A step is one pass of the hot path -- the FP8 branch of ``linear()``
+(reference: inference/model.py:159-160): ``act_quant`` then ``fp8_gemm`` -- over
+one batch of M = 4096 synthetic tokens through the dense-MLP w1 projection
+(7168 -> 18432), inputs resident in HBM.  ``value`` is 2*M*N*K / step time.
+
+The JSON line also carries
+  roofline      the dominant kernel (fp8_gemm) timed alone with HIP events on the
+                launch stream: achieved TFLOP/s vs the dense fp8 MFMA peak;
+  cpu_baseline  the torch-CPU oracle timed on this host on a bounded row sample;
+  extras        the other configurations: act_quant / weight_dequant bandwidth,
+                the w2 prefill shape and the decode sweep (GB/s over algorithmic bytes,
+                weights rotated through > 512 MB so the Infinity Cache cannot hold them).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT / "deepseek-v3_amd"))
+sys.path.insert(0, str(ROOT))
+
+import torch  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 (no sparsity)
+METRIC = "fp8_gemm TFLOP/s & %fp8 MFMA peak @M=4096; decode-GEMM HBM GB/s @M=1-64"
+
+
+def _events(n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def time_loop(fn, steps: int, warmup: int) -> float:
+    """Average milliseconds per call over exactly `steps` calls (events on the launch stream)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = _events(2)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def time_graph(launches, replays: int = 5) -> float:
+    """Average microseconds per launch with the launches captured in one HIP graph, so that
+    back-to-back kernels are not separated by host launch latency.  `launches` is a list of
+    zero-argument callables (typically the same op over rotating buffers)."""
+    for fn in launches[: min(3, len(launches))]:
+        fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for fn in launches:
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(replays):
+        e0, e1 = _events(2)
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1))
+    return best * 1e3 / len(launches)
+
+
+def decode_bytes(m, n, k):
+    return n * k + 4 * (-(-n // 128)) * (k // 128) + m * k + 4 * m * (k // 128) + 2 * m * n
+
+
+def run_extras(K, W):
+    out = {}
+    x = W.activations(4096, 7168, 0, "cuda", outliers=True)
+    xs = [x.clone() for _ in range(12)]                       # 12 x 58.7 MB > Infinity Cache
+    us = time_graph([(lambda t=t: K.act_quant(t)) for t in xs] * 2)
+    out["act_quant_4096x7168"] = {"us": round(us, 2), "GBps": round(88.998e6 / us / 1e3, 1),
+                                  "hbm_frac": round(88.998e6 / us / 1e3 / HBM_PEAK_GBS, 3)}
+    del xs
+    w8, s = W.random_fp8_weight(18432, 7168, 2, "cuda")
+    ws_ = [w8.clone() for _ in range(5)]
+    us = time_graph([(lambda t=t: K.weight_dequant(t, s)) for t in ws_] * 2)
+    out["weight_dequant_18432x7168"] = {"us": round(us, 2), "GBps": round(396.394e6 / us / 1e3, 1),
+                                        "hbm_frac": round(396.394e6 / us / 1e3 / HBM_PEAK_GBS, 3)}
+    del ws_, w8
+    k, n = W.PREFILL_SHAPES["w2"]
+    a, a_s = K.act_quant(W.activations(4096, k, 0, "cuda"))
+    wq, wsc = W.weight(n, k, 1, "cuda")
+    ms = time_loop(lambda: K.fp8_gemm(a, a_s, wq, wsc), 10, 3)
+    tf = 2 * 4096 * n * k / ms / 1e9
+    out["fp8_gemm_M4096_w2_18432to7168"] = {"us": round(ms * 1e3, 1), "TFLOPs": round(tf, 1),
+                                           "mfma_frac": round(tf / FP8_MFMA_PEAK_TFLOPS, 3)}
+    del a, a_s, wq, wsc
+    dec = {}
+    for name, (k, n) in W.DECODE_SHAPES.items():
+        wq, wsc = W.weight(n, k, 1, "cuda")
+        copies = max(2, min(160, -(-640_000_000 // (n * k))))
+        wqs = [wq.clone() for _ in range(copies)]
+        for m in W.DECODE_M:
+            a, a_s = K.act_quant(W.activations(m, k, m, "cuda"))
+            launches = [(lambda t=t: K.fp8_gemm(a, a_s, t, wsc)) for t in wqs]
+            if len(launches) < 40:
+                launches = launches * (-(-40 // len(launches)))
+            us = time_graph(launches)
+            gbs = decode_bytes(m, n, k) / us / 1e3
+            dec[f"{name}_{k}to{n}_M{m}"] = {"us": round(us, 2), "GBps": round(gbs, 1),
+                                            "hbm_frac": round(gbs / HBM_PEAK_GBS, 3)}
+        del wqs
+    out["decode"] = dec
+    return out
+
+
+def cpu_baseline(W, rows: int = 1024):
+    """The torch-CPU oracle (a port of the reference arithmetic) on the first `rows` tokens of
+    the same workload, all host threads."""
+    from oracle import oracle
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, 16)))
+    x = W.activations(rows, 7168, 0, "cpu")
+    w8, ws = W.weight(18432, 7168, 1, "cpu")
+    oracle.linear(x[:64], w8, scale=ws)                      # warm-up
+    t0 = time.perf_counter()
+    oracle.linear(x, w8, scale=ws)
+    dt = time.perf_counter() - t0
+    return {"value": round(2 * rows * 18432 * 7168 / dt / 1e12, 4), "unit": "TFLOP/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle.linear() (act_quant + fp8_gemm, fp32 torch-CPU) on {rows} of 4096 rows, "
+                      f"K=7168 -> N=18432, {dt:.2f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path is built and measured on ONE GPU (one GPU's share of the work at its real "
+                 "shape); --gpus must be 1. Sharding is described in DESIGN.md.")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback.")
+
+    import dsv3fp8 as K                      # fails loudly if libdsv3fp8.so has not been built
+    from dsv3fp8 import workloads as W
+    torch.set_default_dtype(torch.bfloat16)  # as the reference's caller does (generate.py:109)
+    torch.cuda.set_device(0)
+
+    M = W.PREFILL_M
+    k, n = W.PREFILL_SHAPES["w1"]
+    x = W.activations(M, k, 0, "cuda")
+    w8, ws = W.weight(n, k, 1, "cuda")
+    flops = 2.0 * M * n * k
+
+    def step():
+        a, a_s = K.act_quant(x, 128, None)
+        return K.fp8_gemm(a, a_s, w8, ws)
+
+    ms = time_loop(step, args.steps, args.warmup)
+    value = flops / ms / 1e9                                 # TFLOP/s
+
+    a, a_s = K.act_quant(x)
+    gemm_ms = time_loop(lambda: K.fp8_gemm(a, a_s, w8, ws), args.steps, args.warmup)
+    achieved = flops / gemm_ms / 1e9
+
+    line = {
+        "metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 x fp8_e4m3 -> f32", "data": "synthetic",
+        "config": {"workload": "cfg4 prefill linear(): act_quant + fp8_gemm, M=4096 tokens, dense MLP w1 "
+                               "K=7168 -> N=18432, bf16 act ~N(0,1), fp8 weights block-quantised from ~N(0,0.02), "
+                               "bf16 out", "M": M, "N": n, "K": k, "block": 128},
+        "roofline": {"kernel": "fp8_gemm_tile_kernel", "bound": "mfma", "achieved": round(achieved, 2),
+                     "peak": FP8_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "launch_us": round(gemm_ms * 1e3, 2), "flops_per_launch": flops},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(W)
+    if not args.no_extras:
+        line["extras"] = run_extras(K, W)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
