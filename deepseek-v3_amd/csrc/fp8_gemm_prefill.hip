@@ -1,0 +1,325 @@
+// fp8_gemm, prefill kernel for gfx950 (reference: inference/kernel.py:118-172).
+//
+//   c[m,n] = sum_kb ( sum_{t<128} a[m,128kb+t] * b[n,128kb+t] ) * a_s[m,kb] * b_s[n/128,kb]
+//
+// 256 x 256 tile of C per workgroup, 8 wavefronts (4 along m x 2 along n), each
+// owning 64 (m) x 128 (n) as 4 x 8 MFMA tiles of 16x16 with
+// v_mfma_f32_16x16x128_f8f6f4: one instruction = one 128-wide scale block of K.
+// The raw block dot products are folded into binary32 accumulators held in
+// VGPRs with one FMA each by the block's scale.  The MFMA is issued with the
+// weight rows (n) as its A operand and the activation rows (m) as its B
+// operand, so a lane's four results share one m: the scale is a single value
+// per lane and 16-row sub-tile, and the four results are consecutive in n.
+//
+// K blocks of A and B (both K-contiguous, 128 bytes per row) are copied
+// global -> LDS with global_load_lds_dwordx4 (no VGPR staging), double
+// buffered.  Such a load writes a wavefront's 64 x 16 bytes to consecutive LDS
+// addresses, so the layout is chosen on the global side: 8 lanes fetch the 8
+// 16-byte chunks of one row in a permuted order p = c ^ f(row), which leaves the
+// later ds_read_b128 fragment reads (16 consecutive rows, same chunk) free of
+// bank conflicts.
+#include "common.hpp"
+#include <cstdlib>
+
+namespace dsv3 {
+namespace prefill {
+
+constexpr int BM = 256, BN = 256;
+constexpr int WAVES_M = 4, WAVES_N = 2;
+constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;      // 64 x 128 per wavefront
+constexpr int SM = WM / 16, SN = WN / 16;                // 4 x 8 MFMA tiles
+constexpr int THREADS = WAVES_M * WAVES_N * kWave;       // 512
+constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128;    // bytes per K block
+constexpr int LDS_A = 0, LDS_B = 2 * A_STAGE;            // [A s0 | A s1 | B s0 | B s1]
+constexpr int LDS_BYTES = 2 * (A_STAGE + B_STAGE);       // 128 KiB
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// chunk permutation inside a 128-byte LDS row (see file comment)
+// measured on gfx950 (SQ_LDS_BANK_CONFLICT == 0): 16 consecutive lanes reading the same logical chunk of
+// 16 consecutive 128-byte rows do not collide when the chunk index is xor-ed with (row & 7) ^ (row >> 3 & 1)
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+__device__ __forceinline__ v8i join(v4i lo, v4i hi) {
+    v8i r = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+    return r;
+}
+
+template <int CD, int ABL = 0>
+__global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c,
+        int M, int N, int K, int tiles_m, int tiles_n) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    // ---- workgroup -> tile: contiguous run of tiles per XCD, bands of GROUP_M tile rows
+    const int T = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int q = T / 8, r = T % 8, x = pid % 8;
+        pid = x * q + (x < r ? x : r) + pid / 8;
+    }
+    constexpr int GROUP_M = 4;
+    const int band = pid / (GROUP_M * tiles_n);
+    const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+    const int in_band = pid - band * GROUP_M * tiles_n;
+    const int tm = band * GROUP_M + in_band % band_rows;
+    const int tn = in_band / band_rows;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const long long dbg_t0 = (ABL & 16) ? clock64() : 0, dbg_w0 = (ABL & 16) ? wall_clock64() : 0;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & (WAVES_M - 1), wn = wave / WAVES_M;
+    const int KB = K / 128;
+
+    // ---- global -> LDS copy plan: a stage is 512 rows (256 of A, then 256 of B) = 64 KiB =
+    // 64 wavefront-loads of 1 KiB; wavefront w issues loads i*8 + w, i = 0..7 (i < 4: A, else B).
+    // Load q covers rows q*8 .. q*8+7; lane l -> row q*8 + l/8, LDS chunk l%8, global chunk (l%8)^f(row).
+    uint32_t src_off[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int q = i * 8 + wave;
+        const int row = (q & 31) * 8 + (lane >> 3);              // row inside A or B
+        const int ch = (lane & 7) ^ swz(row);
+        if (i < 4) src_off[i] = (uint32_t)min(m0 + row, M - 1) * (uint32_t)K + ch * 16;
+        else       src_off[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + ch * 16;
+    }
+    auto issue_load = [&](int i, int kb, int stage) {
+        const int q = i * 8 + wave;
+        const uint8_t* base = (i < 4) ? a : b;
+        const int dst = (i < 4 ? LDS_A + stage * A_STAGE : LDS_B + stage * B_STAGE) + (q & 31) * 1024;
+        __builtin_amdgcn_global_load_lds((gptr_t)(base + src_off[i] + (uint32_t)kb * 128u),
+                                         (lptr_t)(lds + dst), 16, 0, 0);
+    };
+    auto issue_loads = [&](int kb, int stage) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int q = i * 8 + wave;
+            const uint8_t* base = (i < 4) ? a : b;
+            const int dst = (i < 4 ? LDS_A + stage * A_STAGE : LDS_B + stage * B_STAGE) + (q & 31) * 1024;
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + src_off[i] + (uint32_t)kb * 128u),
+                                             (lptr_t)(lds + dst), 16, 0, 0);
+        }
+    };
+
+    // ---- fragment read addresses.  A lane reads row (lane&15) of a 16-row sub-tile and the 32 bytes
+    // at K offset 32*(lane>>4), i.e. chunks 2*(lane>>4) and 2*(lane>>4)+1, permuted by f(row).
+    const int fr = lane & 15, fq = lane >> 4;
+    const int fx = swz(fr);                                   // sub-tile bases are multiples of 16 rows
+    const int c0 = ((2 * fq) ^ fx) * 16, c1 = ((2 * fq + 1) ^ fx) * 16;
+    const int a_rd = LDS_A + (wm * WM + fr) * 128;            // + j*16*128 + stage*A_STAGE
+    const int b_rd = LDS_B + (wn * WN + fr) * 128;            // + i*16*128 + stage*B_STAGE
+
+    // ---- scales: a_s[m, kb] for the lane's row of each m sub-tile; b_s row of this wavefront's n range
+    uint32_t as_off[SM];
+#pragma unroll
+    for (int j = 0; j < SM; ++j)
+        as_off[j] = (uint32_t)min(m0 + wm * WM + j * 16 + fr, M - 1) * (uint32_t)KB;
+    const int nb_last = (N - 1) / 128;
+    const float* bs_src = b_s + (size_t)min((n0 + wn * WN) / 128, nb_last) * KB;
+
+    v4f acc[SN][SM];
+#pragma unroll
+    for (int i = 0; i < SN; ++i)
+#pragma unroll
+        for (int j = 0; j < SM; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // A zero the compiler cannot see through: indexing the (wavefront-uniform) b_s row with it keeps that load
+    // on the vector memory path.  A scalar load would share the LGKM counter with the LDS reads and, returning
+    // out of order, force every LDS wait in the loop down to lgkmcnt(0).
+    int vzero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(vzero));
+
+    // Software pipeline.  Per 16-column step i of a K block the wavefront issues
+    //     ds_read x2 (weights of step i+1) | MFMA j=0 | FMA of the pending tile | MFMA 1 | FMA tile 0 | MFMA 2 |
+    //     FMA tile 1 | MFMA 3 | FMA tile 2            (tile 3 stays pending into the next step)
+    // so every FMA reads a result that was issued two MFMAs earlier and the matrix pipe never waits on the
+    // vector pipe.  The tile left pending at the end of a K block is folded after the barrier, under the LDS
+    // latency of the next block's first fragment reads.
+    issue_loads(0, 0);
+    float sc[SM], sc_nxt[SM];
+    {
+        const float bs = bs_src[0];
+#pragma unroll
+        for (int j = 0; j < SM; ++j) sc_nxt[j] = a_s[as_off[j]] * bs;
+#pragma unroll
+        for (int j = 0; j < SM; ++j) sc[j] = 0.f;
+    }
+    v4f pend = {0.f, 0.f, 0.f, 0.f};      // raw dot products of (i = SN-1, j = SM-1) of the previous K block
+    __builtin_amdgcn_s_waitcnt(0x0f70 & 0x3f70);   // vmcnt(0)
+    __syncthreads();
+
+#define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+    long long tA = 0, tB = 0, tC = 0, tD = 0, tE = 0, t_prev = (ABL & 32) ? clock64() : 0;
+    for (int kb = 0; kb < KB; ++kb) {
+        const int stage = kb & 1;
+        const uint8_t* as_base = lds + a_rd + stage * A_STAGE;
+        const uint8_t* bs_base = lds + b_rd + stage * B_STAGE;
+
+        // weight rows (MFMA A operand) are streamed two steps ahead through three fragment buffers
+        v8i nf0 = join(*(const v4i*)(bs_base + c0), *(const v4i*)(bs_base + c1));
+        v8i mf[SM];                                                                 // activation rows: MFMA B operand
+#pragma unroll
+        for (int j = 0; j < SM; ++j)
+            mf[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
+        v8i nf1 = join(*(const v4i*)(bs_base + 2048 + c0), *(const v4i*)(bs_base + 2048 + c1));
+
+        // branch-free: the last iteration re-fetches its own block into the idle stage
+        const int kn = min(kb + 1, KB - 1);
+        float as_nxt[SM], bs_nxt = 0.f;
+
+        // fold the tile left over from the previous K block with that block's scale, then switch scales
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[SN - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[SN - 1][SM - 1][e]);
+#pragma unroll
+        for (int j = 0; j < SM; ++j) sc[j] = sc_nxt[j];
+        __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+        for (int i = 0; i < SN; ++i) {
+            // LDS reads complete in order: all but the newest two (the fragment of step i+1) have landed
+            if (i + 1 < SN) __builtin_amdgcn_s_waitcnt(0xc27f);          // lgkmcnt(2)
+            else            __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0)
+            __builtin_amdgcn_sched_barrier(0);
+            if ((ABL & 32) && i == 0) { const long long t = clock64(); tA += t - t_prev; t_prev = t; __builtin_amdgcn_sched_barrier(0); }
+            v8i nf2 = nf0;
+            if (i + 2 < SN && !(ABL & 8))
+                nf2 = join(*(const v4i*)(bs_base + (i + 2) * 2048 + c0), *(const v4i*)(bs_base + (i + 2) * 2048 + c1));
+            const v4f z = {0.f, 0.f, 0.f, 0.f};
+            v4f p[SM];
+            p[0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[0], z, 0, 0, 0, 0, 0, 0);
+            if (i > 0) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[i - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[i - 1][SM - 1][e]);
+            }
+#pragma unroll
+            for (int j = 1; j < SM; ++j) {
+                p[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[j], z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(p[j - 1][e], sc[j - 1], acc[i][j - 1][e]);
+            }
+            // one eighth of the next K block's global -> LDS copy and one scale load per step: the memory
+            // pipeline sees a steady trickle instead of a burst that would stall instruction issue
+            if (!(ABL & 1)) {
+                if (ABL & 64) {            // 2 loads per step in steps 0..3
+                    if (i < 4) { issue_load(2 * i, kn, stage ^ 1); issue_load(2 * i + 1, kn, stage ^ 1); }
+                } else if (ABL & 128) {    // 2,2,1,1,1,1
+                    if (i < 2) { issue_load(2 * i, kn, stage ^ 1); issue_load(2 * i + 1, kn, stage ^ 1); }
+                    else if (i < 6) issue_load(i + 2, kn, stage ^ 1);
+                } else {
+                    issue_load(i, (ABL & 4) ? 0 : kn, stage ^ 1);
+                }
+            }
+            if (i < SM) as_nxt[i] = a_s[as_off[i] + (uint32_t)kn];
+            if (i == SM) bs_nxt = bs_src[kn + vzero];     // through the vector path on purpose, see vzero
+            pend = p[SM - 1];
+            nf0 = nf1;
+            nf1 = nf2;
+            if (i + 2 < SN && !(ABL & 8)) DSV3_SGB(0x100, 2);
+            DSV3_SGB(0x008, 1);
+            if (i > 0) DSV3_SGB(0x002, 4);
+#pragma unroll
+            for (int j = 1; j < SM; ++j) { DSV3_SGB(0x008, 1); DSV3_SGB(0x002, 4); }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        if (ABL & 32) { __builtin_amdgcn_sched_barrier(0); const long long t = clock64(); tB += t - t_prev; t_prev = t; __builtin_amdgcn_sched_barrier(0); }
+#pragma unroll
+        for (int j = 0; j < SM; ++j) sc_nxt[j] = as_nxt[j] * bs_nxt;
+        if (!(ABL & 2)) {
+        __builtin_amdgcn_s_waitcnt(0x0f70 & 0x3f70);
+        if (ABL & 32) { __builtin_amdgcn_sched_barrier(0); const long long t = clock64(); tC += t - t_prev; t_prev = t; __builtin_amdgcn_sched_barrier(0); }
+        __syncthreads();
+        if (ABL & 32) { __builtin_amdgcn_sched_barrier(0); const long long t = clock64(); tD += t - t_prev; t_prev = t; __builtin_amdgcn_sched_barrier(0); }
+        }
+    }
+#undef DSV3_SGB
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[SN - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[SN - 1][SM - 1][e]);
+
+    if ((ABL & 32) && (tid == 0 || tid == 320) && (blockIdx.x % 193) == 0)
+        printf("blk %d wave %d: per K block: top+first LDS wait %lld, steps %lld, vmcnt wait %lld, barrier %lld\n", (int)blockIdx.x, tid >> 6, tA / KB, tB / KB, tC / KB, tD / KB);
+    if ((ABL & 16) && tid == 0 && (blockIdx.x % 97) == 0) {
+        const long long t1 = clock64(), w1 = wall_clock64();
+        printf("blk %d: %lld clk, %lld wall(100MHz) -> %.0f MHz\n", (int)blockIdx.x, t1 - dbg_t0, w1 - dbg_w0, (double)(t1 - dbg_t0) / ((double)(w1 - dbg_w0) / 100.0));
+    }
+    // ---- epilogue: lane holds c[m][n .. n+3] for every (i, j)
+    const bool vec_ok = (N % 4) == 0;
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        const int m = m0 + wm * WM + j * 16 + fr;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < SN; ++i) {
+            const int n = n0 + wn * WN + i * 16 + fq * 4;
+            typename OutT<CD>::type* dst = c + (size_t)m * N + n;
+            if (vec_ok && n + 3 < N) {
+                if (CD == DSV3_F32) {
+                    *(v4f*)dst = acc[i][j];
+                } else if (CD == DSV3_BF16) {
+                    v2u o = { pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3]) };
+                    *(v2u*)dst = o;
+                } else {
+                    v2u o = { pack_f16(acc[i][j][0], acc[i][j][1]), pack_f16(acc[i][j][2], acc[i][j][3]) };
+                    *(v2u*)dst = o;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) dst[e] = cvt_out<CD>(acc[i][j][e]);
+            }
+        }
+    }
+}
+
+}  // namespace prefill
+
+// Usable when the row offsets fit 32 bits; the caller falls back to the generic tile kernel otherwise.
+bool prefill_supported(int64_t m, int64_t n, int64_t k) {
+    return k >= 128 && m * k < (1ll << 32) && n * k < (1ll << 32);
+}
+
+template <int CD>
+int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+                   int64_t m, int64_t n, int64_t k, hipStream_t stream) {
+    using namespace prefill;
+    const int64_t tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
+    if (tm * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    auto kern = fp8_gemm_prefill_kernel<CD>;
+    static const int abl = std::getenv("DSV3_ABL") ? atoi(std::getenv("DSV3_ABL")) : 0;
+    if (abl == 1) kern = fp8_gemm_prefill_kernel<CD, 1>;
+    if (abl == 2) kern = fp8_gemm_prefill_kernel<CD, 2>;
+    if (abl == 3) kern = fp8_gemm_prefill_kernel<CD, 3>;
+    if (abl == 4) kern = fp8_gemm_prefill_kernel<CD, 4>;
+    if (abl == 6) kern = fp8_gemm_prefill_kernel<CD, 6>;
+    if (abl == 11) kern = fp8_gemm_prefill_kernel<CD, 11>;
+    if (abl == 16) kern = fp8_gemm_prefill_kernel<CD, 16>;
+    if (abl == 27) kern = fp8_gemm_prefill_kernel<CD, 27>;
+    if (abl == 32) kern = fp8_gemm_prefill_kernel<CD, 32>;
+    if (abl == 33) kern = fp8_gemm_prefill_kernel<CD, 33>;
+    if (abl == 64) kern = fp8_gemm_prefill_kernel<CD, 64>;
+    if (abl == 128) kern = fp8_gemm_prefill_kernel<CD, 128>;
+    if (abl == 96) kern = fp8_gemm_prefill_kernel<CD, 96>;
+    if (abl == 160) kern = fp8_gemm_prefill_kernel<CD, 160>;
+    bool granted[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
+    if (!granted[dev]) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
+            return DSV3_ERR_LAUNCH;
+        granted[dev] = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(THREADS), LDS_BYTES, stream,
+                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c,
+                       (int)m, (int)n, (int)k, (int)tm, (int)tn);
+    return launch_status();
+}
+
+template int launch_prefill<DSV3_BF16>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t);
+template int launch_prefill<DSV3_F16>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t);
+template int launch_prefill<DSV3_F32>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t);
+
+}  // namespace dsv3

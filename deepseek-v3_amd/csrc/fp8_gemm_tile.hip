@@ -19,6 +19,8 @@
 // Both operands take their 32 bytes per lane from the same K offsets, so the
 // result does not depend on how the instruction numbers K internally.
 #include "common.hpp"
+#include <cstdlib>
+#include <cstring>
 
 namespace dsv3 {
 namespace {
@@ -260,6 +262,18 @@ Plan make_plan(int64_t m, int64_t n, int64_t k) {
     return p;
 }
 
+// DSV3_GEMM_FORCE=tile|prefill pins the large-M kernel choice (tuning / debugging aid).
+int forced_kernel() {
+    static const int v = [] {
+        const char* e = std::getenv("DSV3_GEMM_FORCE");
+        if (!e) return 0;
+        if (!std::strcmp(e, "tile")) return 1;
+        if (!std::strcmp(e, "prefill")) return 2;
+        return 0;
+    }();
+    return v;
+}
+
 template <int CD>
 int launch_typed(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                  int64_t m, int64_t n, int64_t k, void* ws, hipStream_t st) {
@@ -271,6 +285,9 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
     }
     const Plan p = make_plan(m, n, k);
     if (p.splits == 1) {
+        const int force = forced_kernel();
+        if (prefill_supported(m, n, k) && m > 64 && (force == 2 || (force == 0 && m >= 192)))
+            return launch_prefill<CD>(a, a_s, b, b_s, c, m, n, k, st);
         if (p.bm == 32) return launch_cfg<32, 128, 32, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
         if (p.bm == 64) return launch_cfg<64, 128, 64, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
         return launch_cfg<128, 128, 64, 64, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
