@@ -19,7 +19,6 @@
 // later ds_read_b128 fragment reads (16 consecutive rows, same chunk) free of
 // bank conflicts.
 #include "common.hpp"
-#include <cstdlib>
 
 namespace dsv3 {
 namespace prefill {
@@ -46,7 +45,7 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
     return r;
 }
 
-template <int CD, int ABL = 0>
+template <int CD>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -70,7 +69,6 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const long long dbg_t0 = (ABL & 16) ? clock64() : 0, dbg_w0 = (ABL & 16) ? wall_clock64() : 0;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & (WAVES_M - 1), wn = wave / WAVES_M;
     const int KB = K / 128;
@@ -149,11 +147,10 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         for (int j = 0; j < SM; ++j) sc[j] = 0.f;
     }
     v4f pend = {0.f, 0.f, 0.f, 0.f};      // raw dot products of (i = SN-1, j = SM-1) of the previous K block
-    __builtin_amdgcn_s_waitcnt(0x0f70 & 0x3f70);   // vmcnt(0)
+    __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
     __syncthreads();
 
 #define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-    long long tA = 0, tB = 0, tC = 0, tD = 0, tE = 0, t_prev = (ABL & 32) ? clock64() : 0;
     for (int kb = 0; kb < KB; ++kb) {
         const int stage = kb & 1;
         const uint8_t* as_base = lds + a_rd + stage * A_STAGE;
@@ -184,9 +181,8 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
             if (i + 1 < SN) __builtin_amdgcn_s_waitcnt(0xc27f);          // lgkmcnt(2)
             else            __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0)
             __builtin_amdgcn_sched_barrier(0);
-            if ((ABL & 32) && i == 0) { const long long t = clock64(); tA += t - t_prev; t_prev = t; __builtin_amdgcn_sched_barrier(0); }
             v8i nf2 = nf0;
-            if (i + 2 < SN && !(ABL & 8))
+            if (i + 2 < SN)
                 nf2 = join(*(const v4i*)(bs_base + (i + 2) * 2048 + c0), *(const v4i*)(bs_base + (i + 2) * 2048 + c1));
             const v4f z = {0.f, 0.f, 0.f, 0.f};
             v4f p[SM];
@@ -203,22 +199,13 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
             }
             // one eighth of the next K block's global -> LDS copy and one scale load per step: the memory
             // pipeline sees a steady trickle instead of a burst that would stall instruction issue
-            if (!(ABL & 1)) {
-                if (ABL & 64) {            // 2 loads per step in steps 0..3
-                    if (i < 4) { issue_load(2 * i, kn, stage ^ 1); issue_load(2 * i + 1, kn, stage ^ 1); }
-                } else if (ABL & 128) {    // 2,2,1,1,1,1
-                    if (i < 2) { issue_load(2 * i, kn, stage ^ 1); issue_load(2 * i + 1, kn, stage ^ 1); }
-                    else if (i < 6) issue_load(i + 2, kn, stage ^ 1);
-                } else {
-                    issue_load(i, (ABL & 4) ? 0 : kn, stage ^ 1);
-                }
-            }
+            issue_load(i, kn, stage ^ 1);
             if (i < SM) as_nxt[i] = a_s[as_off[i] + (uint32_t)kn];
             if (i == SM) bs_nxt = bs_src[kn + vzero];     // through the vector path on purpose, see vzero
             pend = p[SM - 1];
             nf0 = nf1;
             nf1 = nf2;
-            if (i + 2 < SN && !(ABL & 8)) DSV3_SGB(0x100, 2);
+            if (i + 2 < SN) DSV3_SGB(0x100, 2);
             DSV3_SGB(0x008, 1);
             if (i > 0) DSV3_SGB(0x002, 4);
 #pragma unroll
@@ -226,26 +213,15 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        if (ABL & 32) { __builtin_amdgcn_sched_barrier(0); const long long t = clock64(); tB += t - t_prev; t_prev = t; __builtin_amdgcn_sched_barrier(0); }
 #pragma unroll
         for (int j = 0; j < SM; ++j) sc_nxt[j] = as_nxt[j] * bs_nxt;
-        if (!(ABL & 2)) {
-        __builtin_amdgcn_s_waitcnt(0x0f70 & 0x3f70);
-        if (ABL & 32) { __builtin_amdgcn_sched_barrier(0); const long long t = clock64(); tC += t - t_prev; t_prev = t; __builtin_amdgcn_sched_barrier(0); }
+        __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0): this wavefront's share of the next stage has landed
         __syncthreads();
-        if (ABL & 32) { __builtin_amdgcn_sched_barrier(0); const long long t = clock64(); tD += t - t_prev; t_prev = t; __builtin_amdgcn_sched_barrier(0); }
-        }
     }
 #undef DSV3_SGB
 #pragma unroll
     for (int e = 0; e < 4; ++e) acc[SN - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[SN - 1][SM - 1][e]);
 
-    if ((ABL & 32) && (tid == 0 || tid == 320) && (blockIdx.x % 193) == 0)
-        printf("blk %d wave %d: per K block: top+first LDS wait %lld, steps %lld, vmcnt wait %lld, barrier %lld\n", (int)blockIdx.x, tid >> 6, tA / KB, tB / KB, tC / KB, tD / KB);
-    if ((ABL & 16) && tid == 0 && (blockIdx.x % 97) == 0) {
-        const long long t1 = clock64(), w1 = wall_clock64();
-        printf("blk %d: %lld clk, %lld wall(100MHz) -> %.0f MHz\n", (int)blockIdx.x, t1 - dbg_t0, w1 - dbg_w0, (double)(t1 - dbg_t0) / ((double)(w1 - dbg_w0) / 100.0));
-    }
     // ---- epilogue: lane holds c[m][n .. n+3] for every (i, j)
     const bool vec_ok = (N % 4) == 0;
 #pragma unroll
@@ -289,22 +265,7 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
     const int64_t tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     auto kern = fp8_gemm_prefill_kernel<CD>;
-    static const int abl = std::getenv("DSV3_ABL") ? atoi(std::getenv("DSV3_ABL")) : 0;
-    if (abl == 1) kern = fp8_gemm_prefill_kernel<CD, 1>;
-    if (abl == 2) kern = fp8_gemm_prefill_kernel<CD, 2>;
-    if (abl == 3) kern = fp8_gemm_prefill_kernel<CD, 3>;
-    if (abl == 4) kern = fp8_gemm_prefill_kernel<CD, 4>;
-    if (abl == 6) kern = fp8_gemm_prefill_kernel<CD, 6>;
-    if (abl == 11) kern = fp8_gemm_prefill_kernel<CD, 11>;
-    if (abl == 16) kern = fp8_gemm_prefill_kernel<CD, 16>;
-    if (abl == 27) kern = fp8_gemm_prefill_kernel<CD, 27>;
-    if (abl == 32) kern = fp8_gemm_prefill_kernel<CD, 32>;
-    if (abl == 33) kern = fp8_gemm_prefill_kernel<CD, 33>;
-    if (abl == 64) kern = fp8_gemm_prefill_kernel<CD, 64>;
-    if (abl == 128) kern = fp8_gemm_prefill_kernel<CD, 128>;
-    if (abl == 96) kern = fp8_gemm_prefill_kernel<CD, 96>;
-    if (abl == 160) kern = fp8_gemm_prefill_kernel<CD, 160>;
-    bool granted[64] = {};
+    static bool granted[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
     if (!granted[dev]) {

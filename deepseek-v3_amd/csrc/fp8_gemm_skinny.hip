@@ -1,0 +1,307 @@
+// fp8_gemm for decode shapes (M <= 64) on gfx950: a weight-streaming kernel
+// (reference arithmetic: inference/kernel.py:145-172).
+//
+//   c[m,n] = sum_kb ( sum_{t<128} a[m,128kb+t] * b[n,128kb+t] ) * a_s[m,kb] * b_s[n/128,kb]
+//
+// With M <= 64 every weight byte is used once, so the kernel is bound by how
+// fast b can be pulled out of HBM.  There is no reuse to stage: each wavefront
+// loads its weight rows straight from global memory into the register layout of
+// v_mfma_f32_16x16x128_f8f6f4 (lane l holds row l%16, 32 bytes of the K block)
+// and keeps several K blocks of loads in flight.  The activations (at most
+// 64 x K bytes, shared by every wavefront) come through the vector L1/L2.
+//
+// Work split: a workgroup owns 16*S weight rows and a contiguous range of K
+// blocks (grid.y = split over K across workgroups); inside the workgroup the
+// wavefronts split that range again and their partial sums are added in LDS in
+// a fixed order, so the result does not depend on timing.  With more than one
+// workgroup along K the partial [M,N] slabs go to the caller's workspace and a
+// second kernel adds them, again in a fixed order.
+//
+// Both MFMA operands take their 32 bytes per lane from the same K offsets
+// ({16q..16q+15} and {64+16q..64+16q+15}, q = lane/16), chosen so that the four
+// lanes that share a row read 64 contiguous bytes per load instruction.
+#include "common.hpp"
+
+namespace dsv3 {
+namespace skinny {
+
+constexpr int kMaxWaves = 8;
+
+__device__ __forceinline__ v8i join(v4i lo, v4i hi) {
+    v8i r = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+    return r;
+}
+
+// a = what the lane loaded from rows 0..7, b = from rows 8..15 (see the weight loads in the kernel).  Lanes with
+// (lane & 15) < 8 own a row of the first group: their fragment is [a, b-of-lane^8 ... no: a-of-lane^8's second half];
+// written out: first 16 bytes  = lane<8 ? a : ror8(b);  last 16 bytes = lane<8 ? ror8(a) : b.
+__device__ __forceinline__ v8i untangle(v4i a, v4i b) {
+    v8i r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        // row_ror:8 inside each 16-lane row; bank_mask picks the lanes that take the rotated value
+        r[i]     = __builtin_amdgcn_update_dpp(a[i], b[i], 0x128, 0xf, 0xc, false);
+        r[4 + i] = __builtin_amdgcn_update_dpp(b[i], a[i], 0x128, 0xf, 0x3, false);
+    }
+    return r;
+}
+
+// measured on gfx950: 16 consecutive lanes reading one logical 16-byte chunk of 16 consecutive 128-byte LDS rows
+// do not collide when the chunk index is xor-ed with this function of the row
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// MT: 16-row activation sub-tiles (M <= 16*MT); S: 16-row weight strips per wavefront;
+// NPF: K blocks of weight loads kept in flight per wavefront.
+//
+// The workgroup first copies the activations of its whole K range (and their scales) into LDS; the wavefronts
+// then read them with ds_read while the weight loads stream through a register ring.  LDS reads and vector
+// memory loads retire on different counters, so fetching an activation never drains the weight ring.
+constexpr int kSlabChunks = 4;             // 16-byte activation chunks a thread stages on the way to LDS
+
+template <int MT, int S, int NPF>
+__global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 4))) void fp8_gemm_skinny_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        void* __restrict__ out, int out_dtype,      // out_dtype: dsv3_dtype of `out` (F32 slabs when gridDim.y > 1)
+        int M, int N, int K, int kb_per_wg) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n_waves = blockDim.x >> 6;
+    const int KB = K >> 7;
+    const int fr = lane & 15, fq = lane >> 4;
+
+    // K blocks of this workgroup, then of this wavefront
+    const int wg_kb0 = blockIdx.y * kb_per_wg;
+    const int wg_nkb = min(kb_per_wg, KB - wg_kb0);
+    const int per_wave = (wg_nkb + n_waves - 1) / n_waves;
+    const int kb0 = wg_kb0 + wave * per_wave;                 // first K block of the wavefront (global index)
+    const int nkb = max(0, min(per_wave, wg_kb0 + wg_nkb - kb0));
+
+    const int n0 = blockIdx.x * (16 * S);
+    // Weight loads: an instruction fetches 8 rows x 128 contiguous bytes (lanes with fr < 8 take the first 64
+    // bytes of row fr&7, lanes with fr >= 8 the last 64 bytes of the same row); a second one does rows 8..15.
+    // The halves that landed in the wrong lane are exchanged between lanes fr and fr^8 with DPP row rotates
+    // when the fragment is assembled.  (One instruction per 16 rows x 64 bytes would put the data straight into
+    // MFMA layout but reaches markedly less HBM bandwidth.)
+    const uint8_t* wsrc[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+        wsrc[s] = b + (size_t)min(n0 + s * 16 + (fr & 7), N - 1) * K + (size_t)kb0 * 128 + (fr >> 3) * 64 + fq * 16;
+    // rows 8..15 of the strip: +8 rows, clamped to the last row of b
+    size_t wrow8[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+        wrow8[s] = (size_t)(min(n0 + s * 16 + (fr & 7) + 8, N - 1) - min(n0 + s * 16 + (fr & 7), N - 1)) * K;
+
+    // ---- activations of the workgroup's K range -> LDS, packed: slab row kb*M + m holds the 128 bytes of
+    // activation row m in K block kb (16-byte chunks permuted by swz(slab row)); the scales follow as
+    // [kb*M + m] floats.  A fragment read always spans 16 consecutive slab rows; when M is not a multiple of
+    // 16 the surplus rows belong to the next K block (or to the 16 rows of padding at the end) and only feed
+    // output columns that are never stored.
+    // Their loads are issued first: vector loads retire in issue order, so the slab can be written to LDS while
+    // the (younger) weight loads below are still in flight.
+    const int slab_rows = kb_per_wg * M + 16;
+    uint8_t* act = lds;
+    float* act_s = (float*)(lds + (size_t)slab_rows * 128);
+    const int chunks = wg_nkb * M * 8;                         // 16-byte chunks to copy (<= kSlabChunks * threads)
+    v4i stage[kSlabChunks];
+    float stage_s = 0.f;
+#pragma unroll
+    for (int i = 0; i < kSlabChunks; ++i) {
+        const int c = tid + i * (int)blockDim.x;
+        if (c < chunks) {
+            const int ch = c & 7, R = c >> 3, row = R % M, kb = R / M;
+            stage[i] = *(const v4i*)(a + (size_t)row * K + (size_t)(wg_kb0 + kb) * 128 + ch * 16);
+        }
+    }
+    if (tid < wg_nkb * M)      // scale of (row, K block) with the weight block's scale already folded in
+        stage_s = a_s[(size_t)(tid % M) * KB + wg_kb0 + tid / M] * b_s[(size_t)min(n0 >> 7, (N - 1) >> 7) * KB + wg_kb0 + tid / M];
+
+    // ---- start the weight stream: the first NPF K blocks of every strip
+    v4i wlo[NPF][S], whi[NPF][S];
+    auto fetch = [&](int p, int k) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            wlo[p][s] = __builtin_nontemporal_load((const v4i*)(wsrc[s] + k * 128));               // rows 0..7
+            whi[p][s] = __builtin_nontemporal_load((const v4i*)(wsrc[s] + wrow8[s] + k * 128));    // rows 8..15
+        }
+    };
+#pragma unroll
+    for (int p = 0; p < NPF; ++p)
+        if (p < nkb) fetch(p, p);
+
+#pragma unroll
+    for (int i = 0; i < kSlabChunks; ++i) {
+        const int c = tid + i * (int)blockDim.x;
+        if (c < chunks) {
+            const int ch = c & 7, R = c >> 3;
+            *(v4i*)(act + R * 128 + ((ch ^ swz(R)) * 16)) = stage[i];
+        }
+    }
+    if (tid < wg_nkb * M) act_s[tid] = stage_s;
+    __syncthreads();
+
+    v4f acc[S][MT];
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) acc[s][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // a lane's fragment: slab row (K block)*M + 16j + fr, logical chunks fq and 4 + fq of the K block
+    const int row0 = (kb0 - wg_kb0) * M + fr;
+
+    // The wavefront works through its K blocks in batches of NPF: all weight loads of a batch are issued back to
+    // back, then consumed in order.  Memory-level parallelism across batches comes from the other wavefronts of
+    // the CU (up to 16), which are at different points of their own batches.
+    for (int kb = 0; kb < nkb; kb += NPF) {
+        if (kb > 0) {
+#pragma unroll
+            for (int p = 0; p < NPF; ++p)
+                if (kb + p < nkb) fetch(p, kb + p);
+        }
+#pragma unroll
+        for (int p = 0; p < NPF; ++p) {
+            const int k = kb + p;
+            if (k < nkb) {                                    // wavefront-uniform
+                v8i af[MT], wf[S];
+                float sc[MT];
+#pragma unroll
+                for (int j = 0; j < MT; ++j) {
+                    const int R = row0 + k * M + j * 16, fx = swz(R);
+                    const uint8_t* r = act + R * 128;
+                    af[j] = join(*(const v4i*)(r + ((fq ^ fx) * 16)), *(const v4i*)(r + (((4 + fq) ^ fx) * 16)));
+                    sc[j] = act_s[R];
+                }
+#pragma unroll
+                for (int s = 0; s < S; ++s) wf[s] = untangle(wlo[p][s], whi[p][s]);
+#pragma unroll
+                for (int s = 0; s < S; ++s)
+#pragma unroll
+                    for (int j = 0; j < MT; ++j) {
+                        const v4f z = {0.f, 0.f, 0.f, 0.f};
+                        const v4f p4 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[s], af[j], z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[s][j][e] = __builtin_fmaf(p4[e], sc[j], acc[s][j][e]);
+                    }
+            }
+        }
+    }
+    __syncthreads();                                        // everyone is done with the activation slab
+
+    // ---- add the wavefronts' partial sums in LDS (fixed order), then store
+    v4f* red = (v4f*)lds;                                   // [wave][s*MT + j][lane]
+    constexpr int TILES = S * MT;
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) red[(wave * TILES + s * MT + j) * 64 + lane] = acc[s][j];
+    __syncthreads();
+
+    const size_t slab = (size_t)blockIdx.y * M * N;          // split-K slab of the fp32 workspace (0 when gridDim.y == 1)
+    for (int slot = tid; slot < TILES * 64; slot += blockDim.x) {
+        v4f v = red[slot];
+        for (int w = 1; w < n_waves; ++w) {
+            const v4f u = red[w * TILES * 64 + slot];
+            v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
+        }
+        const int t = slot >> 6, l = slot & 63;
+        const int s = t / MT, j = t % MT;
+        const int m = j * 16 + (l & 15);
+        const int n = n0 + s * 16 + (l >> 4) * 4;
+        if (m >= M) continue;
+        const size_t idx = slab + (size_t)m * N + n;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (n + e >= N) break;
+            if (out_dtype == DSV3_F32)       ((float*)out)[idx + e] = v[e];
+            else if (out_dtype == DSV3_BF16) ((uint16_t*)out)[idx + e] = cvt_out<DSV3_BF16>(v[e]);
+            else                             ((uint16_t*)out)[idx + e] = cvt_out<DSV3_F16>(v[e]);
+        }
+    }
+}
+
+struct Plan { int mt, s, waves, splits, kb_per_wg; };
+
+// The kernels here run for 5-30 us, so the grid is sized to be resident in ONE round: the workgroups of a
+// second, partly filled round would leave most of the chip idle for half the run.  Within that limit: as many
+// wavefronts as possible (memory-level parallelism), at least two K blocks per wavefront, and few K splits
+// across workgroups (each costs an [M,N] fp32 slab of traffic plus the reduction pass).
+inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
+    const int64_t kb = k / 128;
+    const int64_t capacity = 256 * 16;                         // resident wavefronts: 256 CUs x 16 (<= 128 VGPRs)
+    Plan best{};
+    bool have = false;
+    // wider strips per wavefront (S) cut the number of workgroups when the activation slab forces many K splits
+    for (int s_ : {1, 2, 4}) {
+        Plan p;
+        p.mt = 1;
+        p.s = s_;
+        const int64_t groups = (n + 16 * s_ - 1) / (16 * s_);
+        int waves = 4;
+        while (waves > 1 && (kb / waves < 2 || groups * waves > capacity)) waves >>= 1;
+        int64_t splits = capacity / (groups * waves);
+        const int64_t max_splits = kb / (2 * waves) > 0 ? kb / (2 * waves) : 1;
+        if (splits > max_splits) splits = max_splits;
+        // the activation slab (m rows x 128 B per K block) is staged through kSlabChunks registers per thread,
+        // and one scale per thread
+        int64_t slab_kb = (int64_t)kSlabChunks * waves * 64 / (m * 8);
+        if (slab_kb > waves * 64 / m) slab_kb = waves * 64 / m;
+        if (slab_kb < 1) continue;
+        const int64_t min_splits = (kb + slab_kb - 1) / slab_kb;
+        if (splits < min_splits) splits = min_splits;
+        if (splits < 1) splits = 1;
+        p.waves = waves;
+        p.kb_per_wg = (int)((kb + splits - 1) / splits);
+        p.splits = (int)((kb + p.kb_per_wg - 1) / p.kb_per_wg);
+        const bool fits = groups * p.splits * waves <= capacity;
+        if (!have || fits) { best = p; have = true; }
+        if (fits) break;
+    }
+    return best;
+}
+
+template <int MT, int S>
+void launch_cfg(const Plan& p, const void* a, const float* a_s, const void* b, const float* b_s,
+                void* out, int out_dtype, int m, int n, int k, hipStream_t st) {
+    constexpr int NPF = 8 / S;
+    const unsigned groups = (unsigned)((n + 16 * S - 1) / (16 * S));
+    const size_t red_bytes = (size_t)p.waves * S * MT * 64 * sizeof(v4f);
+    const size_t slab_bytes = ((size_t)p.kb_per_wg * m + 16) * 128 + (size_t)p.kb_per_wg * m * 4;
+    const size_t lds = red_bytes > slab_bytes ? red_bytes : slab_bytes;
+    hipLaunchKernelGGL((fp8_gemm_skinny_kernel<MT, S, NPF>), dim3(groups, (unsigned)p.splits), dim3(p.waves * kWave), lds, st,
+                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, out_dtype, m, n, k, p.kb_per_wg);
+}
+
+}  // namespace skinny
+
+bool skinny_supported(int64_t m, int64_t n, int64_t k) {
+    return m >= 1 && m <= 16 && k >= 128 && n >= 1 && (n + 15) / 16 <= 0x7fffffff;
+}
+
+size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+    const skinny::Plan p = skinny::make_plan(m, n, k);
+    return p.splits > 1 ? (size_t)p.splits * (size_t)m * (size_t)n * sizeof(float) : 0;
+}
+
+// Runs the streaming kernel; *splits_out tells the caller how many fp32 slabs were written to `ws`
+// (1 = the result went straight to c).
+int launch_skinny(const void* a, const float* a_s, const void* b, const float* b_s, void* c, int c_dtype,
+                  int64_t m, int64_t n, int64_t k, void* ws, int* splits_out, hipStream_t st) {
+    using namespace skinny;
+    const Plan p = make_plan(m, n, k);
+    void* out = p.splits > 1 ? ws : c;
+    const int od = p.splits > 1 ? (int)DSV3_F32 : c_dtype;
+    *splits_out = p.splits;
+#define DSV3_CASE(MT_, S_) launch_cfg<MT_, S_>(p, a, a_s, b, b_s, out, od, (int)m, (int)n, (int)k, st); break
+    switch (p.mt * 10 + p.s) {
+        case 11: DSV3_CASE(1, 1);
+        case 12: DSV3_CASE(1, 2);
+        case 14: DSV3_CASE(1, 4);
+        default: return DSV3_ERR_BAD_SHAPE;
+    }
+#undef DSV3_CASE
+    return launch_status();
+}
+
+}  // namespace dsv3

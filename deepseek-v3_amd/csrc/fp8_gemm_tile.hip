@@ -283,9 +283,18 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
                            (const float*)nullptr, (typename OutT<CD>::type*)c, mn0, 0);
         return launch_status();
     }
+    const int force = forced_kernel();
+    if (force != 1 && skinny_supported(m, n, k)) {          // decode shapes: weight-streaming kernel
+        int splits = 1;
+        const int rc = launch_skinny(a, a_s, b, b_s, c, CD, m, n, k, ws, &splits, st);
+        if (rc != DSV3_OK || splits == 1) return rc;
+        const int64_t mn = m * n;
+        hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
+                           (const float*)ws, (typename OutT<CD>::type*)c, mn, splits);
+        return launch_status();
+    }
     const Plan p = make_plan(m, n, k);
     if (p.splits == 1) {
-        const int force = forced_kernel();
         if (prefill_supported(m, n, k) && m > 64 && (force == 2 || (force == 0 && m >= 192)))
             return launch_prefill<CD>(a, a_s, b, b_s, c, m, n, k, st);
         if (p.bm == 32) return launch_cfg<32, 128, 32, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
@@ -307,7 +316,9 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
 size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
     if (m <= 0 || n <= 0 || k <= 0) return 0;
     const Plan p = make_plan(m, n, k);
-    return p.splits > 1 ? (size_t)p.splits * (size_t)m * (size_t)n * sizeof(float) : 0;
+    const size_t tile_ws = p.splits > 1 ? (size_t)p.splits * (size_t)m * (size_t)n * sizeof(float) : 0;
+    const size_t skinny_ws = skinny_supported(m, n, k) ? skinny_workspace_bytes(m, n, k) : 0;
+    return tile_ws > skinny_ws ? tile_ws : skinny_ws;
 }
 
 int launch_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
