@@ -19,7 +19,7 @@ namespace dsv3 {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 4;   // independent 16-byte loads in flight per lane
+constexpr int kUnroll = 2;   // independent 16-byte loads in flight per lane (2 measured best: more costs occupancy)
 
 template <int XD> struct In;
 template <> struct In<DSV3_BF16> {

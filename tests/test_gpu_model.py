@@ -1,0 +1,128 @@
+"""GPU parity of the host-side callers (dsv3fp8.model, the mirror of the reference's inference/model.py
+linear()/Linear/MLP/Gate/Expert/MoE) against the torch-CPU oracle on small configurations."""
+import pytest
+import torch
+
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+FP8 = torch.float8_e4m3fn
+
+
+@pytest.fixture()
+def M():
+    from dsv3fp8 import model
+    old_impl, old_dtype = model.gemm_impl, torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)          # as the reference's entry point does (generate.py:109)
+    model.Linear.dtype = FP8
+    yield model
+    model.gemm_impl = old_impl
+    model.Linear.dtype = torch.bfloat16
+    model.Linear.scale_fmt = None
+    torch.set_default_dtype(old_dtype)
+
+
+def _fill(lin, seed):
+    """Random block-quantised weight into an fp8 Linear (keeps the weight.scale attribute, like load_model)."""
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(lin.out_features, lin.in_features, generator=g) * 0.05).bfloat16()
+    w8, s = oracle.block_quant_weight(w)
+    with torch.no_grad():
+        lin.weight.copy_(w8.cuda())
+        lin.scale.copy_(s.cuda())
+    return w8, s
+
+
+def _close(got, ref, tol=2e-2):
+    got, ref = got.float().cpu(), ref.float()
+    rms = ref.pow(2).mean().sqrt().item()
+    assert (got - ref).abs().max().item() <= tol * max(rms, 1e-6) + 2 ** -8 * ref.abs().max().item()
+
+
+@pytest.mark.parametrize("impl", ["fp8", "bf16"])
+def test_linear_dispatch(M, impl):
+    M.gemm_impl = impl
+    with torch.device("cuda"):
+        lin = M.Linear(512, 384, bias=True)
+    assert lin.weight.dtype == FP8 and lin.scale.shape == (3, 4) and lin.weight.scale is lin.scale
+    w8, s = _fill(lin, 1)
+    with torch.no_grad():
+        lin.bias.copy_(torch.linspace(-1, 1, 384))
+    x = torch.randn(2, 5, 512, generator=torch.Generator().manual_seed(2)).bfloat16()
+    with torch.inference_mode():
+        y = lin(x.cuda())
+    ref = oracle.linear(x, w8, bias=lin.bias.detach().cpu(), scale=s, gemm_impl=impl)
+    assert y.shape == (2, 5, 384) and y.dtype == torch.bfloat16
+    _close(y, ref)
+
+
+def test_wide_weights_take_f_linear(M):
+    with torch.device("cuda"):
+        lin = M.Linear(256, 128, dtype=torch.bfloat16)
+    assert lin.scale is None
+    torch.nn.init.normal_(lin.weight, std=0.05)
+    x = torch.randn(4, 256, device="cuda").bfloat16()
+    assert torch.equal(lin(x), torch.nn.functional.linear(x, lin.weight))
+
+
+def test_scale_fmt_only_reaches_plain_linear(M):
+    M.gemm_impl = "fp8"
+    M.Linear.scale_fmt = "ue8m0"
+    with torch.device("cuda"):
+        plain, col = M.Linear(256, 128), M.ColumnParallelLinear(256, 128)
+    w8, s = _fill(plain, 3)
+    _fill(col, 3)
+    x = torch.randn(8, 256, generator=torch.Generator().manual_seed(4)).bfloat16()
+    with torch.inference_mode():
+        yp, yc = plain(x.cuda()), col(x.cuda())
+    _close(yp, oracle.linear(x, w8, scale=s, scale_fmt="ue8m0"), tol=1e-2)
+    _close(yc, oracle.linear(x, w8, scale=s, scale_fmt=None), tol=1e-2)
+
+
+def test_moe_layer_small(M):
+    M.gemm_impl = "fp8"
+    args = M.ModelArgs(dim=256, inter_dim=512, moe_inter_dim=128, n_routed_experts=8, n_shared_experts=1,
+                       n_activated_experts=2, n_expert_groups=2, n_limited_groups=1, route_scale=2.5)
+    with torch.device("cuda"):
+        moe = M.MoE(args)
+    assert moe.gate.bias is None and moe.gate.weight.dtype == torch.bfloat16
+    g = torch.Generator().manual_seed(5)
+    gw = (torch.randn(8, 256, generator=g) * 0.05).bfloat16()     # scores ~ N(0, 0.8): away from sigmoid saturation
+    with torch.no_grad():
+        moe.gate.weight.copy_(gw.cuda())
+    experts = []
+    for i, ex in enumerate(moe.experts):
+        w1, s1 = _fill(ex.w1, 10 + 3 * i); w2, s2 = _fill(ex.w2, 11 + 3 * i); w3, s3 = _fill(ex.w3, 12 + 3 * i)
+        experts.append((w1, s1, w2, s2, w3, s3))
+    sh = moe.shared_experts
+    shared = (*_fill(sh.w1, 90), *_fill(sh.w2, 91), *_fill(sh.w3, 92))
+    x = torch.randn(3, 7, 256, generator=g).bfloat16()
+    with torch.inference_mode():
+        y = moe(x.cuda())
+        wts, idx = moe.gate(x.view(-1, 256).cuda())
+    ref_w, ref_i = oracle.gate(x.view(-1, 256), gw, None, topk=2, n_groups=2, topk_groups=1, route_scale=2.5)
+    # the router's bf16 GEMM runs in a different summation order on the GPU: near-ties may flip, the bulk may not
+    same = (idx.cpu().sort(-1)[0] == ref_i.sort(-1)[0]).all(-1).float().mean().item()
+    assert same >= 0.8, same
+    ref = oracle.moe(x, wts.cpu(), idx.cpu(), experts, shared)
+    assert y.shape == x.shape
+    _close(y, ref, tol=5e-2)
+
+
+def test_gate_with_bias_671b_width(M):
+    args = M.ModelArgs(n_routed_experts=64, n_expert_groups=8, n_limited_groups=4, n_activated_experts=8)
+    with torch.device("cuda"):
+        gate = M.Gate(args)
+    assert gate.bias is not None and gate.bias.dtype == torch.float32
+    g = torch.Generator().manual_seed(6)
+    gw = (torch.randn(64, 7168, generator=g) * 0.02).bfloat16()
+    gb = torch.randn(64, generator=g) * 0.1
+    with torch.no_grad():
+        gate.weight.copy_(gw.cuda()); gate.bias.copy_(gb.cuda())
+    x = torch.randn(32, 7168, generator=g).bfloat16()
+    w, idx = gate(x.cuda())
+    assert w.dtype == torch.bfloat16 and idx.shape == (32, 8)
+    assert all(len(set(r.tolist())) == 8 for r in idx.cpu())
+    assert all(len(set((r // 8).tolist())) <= 4 for r in idx.cpu())
+    assert torch.allclose(w.float().sum(-1).cpu(), torch.full((32,), 2.5, dtype=torch.float32), atol=0.05)
