@@ -78,6 +78,18 @@ def time_graph(launches, replays: int = 5) -> float:
     return best * 1e3 / len(launches)
 
 
+def measured_traffic():
+    """HBM bytes per launch of the dominant kernel on this workload, from the committed rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE summary (profiles/fp8_gemm_prefill_traffic.json); None when it has not been taken."""
+    f = ROOT / "profiles" / "fp8_gemm_prefill_traffic.json"
+    if not f.exists():
+        return None
+    try:
+        return json.loads(f.read_text())["hbm_bytes_per_launch"]
+    except (ValueError, KeyError):
+        return None
+
+
 def decode_bytes(m, n, k):
     return n * k + 4 * (-(-n // 128)) * (k // 128) + m * k + 4 * m * (k // 128) + 2 * m * n
 
@@ -120,7 +132,43 @@ def run_extras(K, W):
                                             "hbm_frac": round(gbs / HBM_PEAK_GBS, 3)}
         del wqs
     out["decode"] = dec
+    out["moe_layer_T4096"] = run_moe(K, W)
     return out
+
+
+def run_moe(K, W, tokens: int = 4096):
+    """BASELINE config 5: one MoE layer (256 routed + 1 shared SwiGLU experts, 7168 -> 2048 -> 7168, fp8
+    block-scaled weights generated on the device), T tokens, sigmoid gate with bias over random logits'
+    weights, 8 groups / top-4 groups / top-8 experts, route_scale 2.5, executed as the reference does:
+    one pass over the experts' token lists (model.py:679-693)."""
+    from dsv3fp8 import model as Mdl
+    old = Mdl.gemm_impl, Mdl.Linear.dtype
+    Mdl.gemm_impl, Mdl.Linear.dtype = "fp8", torch.float8_e4m3fn
+    try:
+        args = Mdl.ModelArgs()
+        with torch.device("cuda"):
+            moe = Mdl.MoE(args)
+        g = torch.Generator(device="cuda").manual_seed(5)
+        with torch.no_grad():
+            moe.gate.weight.copy_(torch.randn(args.n_routed_experts, args.dim, generator=g, device="cuda") * 0.02)
+            moe.gate.bias.copy_(torch.randn(args.n_routed_experts, generator=g, device="cuda") * 0.1)
+            protos = [W.weight(args.moe_inter_dim, args.dim, 40, "cuda"), W.weight(args.dim, args.moe_inter_dim, 41, "cuda")]
+            for ex in list(moe.experts) + [moe.shared_experts]:
+                for lin, (w8, sc) in ((ex.w1, protos[0]), (ex.w3, protos[0]), (ex.w2, protos[1])):
+                    lin.weight.copy_(w8)          # distinct storage per expert: 11.3 GB of weights are streamed
+                    lin.scale.copy_(sc)
+        x = W.activations(tokens, args.dim, 6, "cuda")
+        with torch.inference_mode():
+            ms = time_loop(lambda: moe(x), 3, 1)
+        flops = 2.0 * 3 * args.dim * args.moe_inter_dim * (tokens * args.n_activated_experts + tokens)
+        wbytes = 257 * 3 * args.dim * args.moe_inter_dim
+        return {"ms": round(ms, 3), "TFLOPs": round(flops / ms / 1e9, 1),
+                "weight_stream_GBps": round(wbytes / ms / 1e6, 1),
+                "mfma_frac": round(flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 4),
+                "hbm_frac": round(wbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                "note": "expert loop as in the reference (host-driven, 3 act_quant + 3 fp8_gemm per expert)"}
+    finally:
+        Mdl.gemm_impl, Mdl.Linear.dtype = old
 
 
 def cpu_baseline(W, rows: int = 1024):
@@ -147,6 +195,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 1 GiB device copy (a kernel of known HBM traffic) so that rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is built and measured on ONE GPU (one GPU's share of the work at its real "
@@ -176,17 +227,24 @@ def main():
     gemm_ms = time_loop(lambda: K.fp8_gemm(a, a_s, w8, ws), args.steps, args.warmup)
     achieved = flops / gemm_ms / 1e9
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     line = {
         "metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp8_e4m3 x fp8_e4m3 -> f32", "data": "synthetic",
+        "dtype": "fp8_e4m3 (f32 accumulate)", "data": "synthetic",
         "config": {"workload": "cfg4 prefill linear(): act_quant + fp8_gemm, M=4096 tokens, dense MLP w1 "
                                "K=7168 -> N=18432, bf16 act ~N(0,1), fp8 weights block-quantised from ~N(0,0.02), "
                                "bf16 out", "M": M, "N": n, "K": k, "block": 128},
-        "roofline": {"kernel": "fp8_gemm_tile_kernel", "bound": "mfma", "achieved": round(achieved, 2),
+        "roofline": {"kernel": "fp8_gemm_prefill_kernel", "bound": "mfma", "achieved": round(achieved, 2),
                      "peak": FP8_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4), "traffic": measured_traffic(),
                      "launch_us": round(gemm_ms * 1e3, 2), "flops_per_launch": flops},
     }
     if not args.no_cpu:
