@@ -72,6 +72,10 @@ int launch_fp8_gemm(const void* a, const float* a_s, const void* b, const float*
                     void* workspace, size_t workspace_bytes, hipStream_t stream);
 size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 bool prefill_supported(int64_t m, int64_t n, int64_t k);
+bool stream_supported(int64_t m, int64_t n, int64_t k);
+size_t stream_workspace_bytes(int64_t m, int64_t n, int64_t k);
+int launch_stream(const void* a, const float* a_s, const void* b, const float* b_s, void* c, int c_dtype,
+                  int64_t m, int64_t n, int64_t k, void* ws, int* splits_out, hipStream_t st);
 bool skinny_supported(int64_t m, int64_t n, int64_t k);
 size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t k);
 int launch_skinny(const void* a, const float* a_s, const void* b, const float* b_s, void* c, int c_dtype,

@@ -284,9 +284,11 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
         return launch_status();
     }
     const int force = forced_kernel();
-    if (force != 1 && skinny_supported(m, n, k)) {          // decode shapes: weight-streaming kernel
+    const bool use_stream = force != 1 && stream_supported(m, n, k);
+    if (use_stream || (force != 1 && skinny_supported(m, n, k))) {          // decode shapes: weight-streaming kernels
         int splits = 1;
-        const int rc = launch_skinny(a, a_s, b, b_s, c, CD, m, n, k, ws, &splits, st);
+        const int rc = use_stream ? launch_stream(a, a_s, b, b_s, c, CD, m, n, k, ws, &splits, st)
+                                  : launch_skinny(a, a_s, b, b_s, c, CD, m, n, k, ws, &splits, st);
         if (rc != DSV3_OK || splits == 1) return rc;
         const int64_t mn = m * n;
         hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
@@ -317,8 +319,10 @@ size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
     if (m <= 0 || n <= 0 || k <= 0) return 0;
     const Plan p = make_plan(m, n, k);
     const size_t tile_ws = p.splits > 1 ? (size_t)p.splits * (size_t)m * (size_t)n * sizeof(float) : 0;
-    const size_t skinny_ws = skinny_supported(m, n, k) ? skinny_workspace_bytes(m, n, k) : 0;
-    return tile_ws > skinny_ws ? tile_ws : skinny_ws;
+    size_t need = tile_ws;
+    if (skinny_supported(m, n, k) && skinny_workspace_bytes(m, n, k) > need) need = skinny_workspace_bytes(m, n, k);
+    if (stream_supported(m, n, k) && stream_workspace_bytes(m, n, k) > need) need = stream_workspace_bytes(m, n, k);
+    return need;
 }
 
 int launch_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,

@@ -83,7 +83,7 @@ int dsv3_act_quant(const void* x, int x_dtype, void* y, float* s,
  *     y[i,j] = y_dtype( f32(x[i,j]) * s[i / block_size, j / block_size] )
  * x: [m,n] fp8 bytes, s: [ceil(m/block_size), ceil(n/block_size)] binary32,
  * y: [m,n] of y_dtype.  Any m, n >= 0 and any block_size >= 1; block_size 128
- * with n % 16 == 0 and 16-byte aligned x, y takes the vectorised kernel.
+ * with n % 8 == 0, 8-byte aligned x and 16-byte aligned y takes the vectorised kernel.
  */
 int dsv3_weight_dequant(const void* x, const float* s, void* y, int y_dtype,
                         int64_t m, int64_t n, int block_size, void* stream);
