@@ -132,12 +132,16 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     asm volatile("v_mov_b32 %0, 0" : "=v"(vzero));
 
     // Software pipeline.  Per 16-column step i of a K block the wavefront issues
-    //     ds_read x2 (weights of step i+1) | MFMA j=0 | FMA of the pending tile | MFMA 1 | FMA tile 0 | MFMA 2 |
+    //     ds_read x2 (weights of step i+2) | MFMA j=0 | FMA of the pending tile | MFMA 1 | FMA tile 0 | MFMA 2 |
     //     FMA tile 1 | MFMA 3 | FMA tile 2            (tile 3 stays pending into the next step)
     // so every FMA reads a result that was issued two MFMAs earlier and the matrix pipe never waits on the
-    // vector pipe.  The tile left pending at the end of a K block is folded after the barrier, under the LDS
-    // latency of the next block's first fragment reads.
-    issue_loads(0, 0);
+    // vector pipe.
+    //
+    // The workgroup barrier of a K block sits before step kSync = SN-2, not at the block's end: by then every
+    // fragment the block still needs is in registers, so after the barrier the idle LDS stage can be refilled
+    // (block kb+2) and the first fragments of block kb+1 are read from the other stage while the last
+    // 2 x SM MFMAs of block kb run.  The next block then starts with its operands already in registers.
+    constexpr int kSync = SN - 2;
     float sc[SM], sc_nxt[SM];
     {
         const float bs = bs_src[0];
@@ -146,26 +150,31 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 #pragma unroll
         for (int j = 0; j < SM; ++j) sc[j] = 0.f;
     }
-    v4f pend = {0.f, 0.f, 0.f, 0.f};      // raw dot products of (i = SN-1, j = SM-1) of the previous K block
+    issue_loads(0, 0);
     __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
     __syncthreads();
+    issue_loads(min(1, KB - 1), 1);
+    v4f pend = {0.f, 0.f, 0.f, 0.f};      // raw dot products of (i = SN-1, j = SM-1) of the previous K block
+    v8i nf0, nf1, mf[SM];                 // weight fragments of steps i, i+1 (MFMA A operand); activation fragments (B operand)
+    {
+        const uint8_t* as_base = lds + a_rd;
+        const uint8_t* bs_base = lds + b_rd;
+        nf0 = join(*(const v4i*)(bs_base + c0), *(const v4i*)(bs_base + c1));
+#pragma unroll
+        for (int j = 0; j < SM; ++j)
+            mf[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
+        nf1 = join(*(const v4i*)(bs_base + 2048 + c0), *(const v4i*)(bs_base + 2048 + c1));
+    }
 
 #define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
     for (int kb = 0; kb < KB; ++kb) {
         const int stage = kb & 1;
-        const uint8_t* as_base = lds + a_rd + stage * A_STAGE;
         const uint8_t* bs_base = lds + b_rd + stage * B_STAGE;
+        const uint8_t* as_next = lds + a_rd + (stage ^ 1) * A_STAGE;
+        const uint8_t* bs_next = lds + b_rd + (stage ^ 1) * B_STAGE;
 
-        // weight rows (MFMA A operand) are streamed two steps ahead through three fragment buffers
-        v8i nf0 = join(*(const v4i*)(bs_base + c0), *(const v4i*)(bs_base + c1));
-        v8i mf[SM];                                                                 // activation rows: MFMA B operand
-#pragma unroll
-        for (int j = 0; j < SM; ++j)
-            mf[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
-        v8i nf1 = join(*(const v4i*)(bs_base + 2048 + c0), *(const v4i*)(bs_base + 2048 + c1));
-
-        // branch-free: the last iteration re-fetches its own block into the idle stage
-        const int kn = min(kb + 1, KB - 1);
+        // branch-free: past the end the loop re-fetches the last block into a stage nobody reads again
+        const int kn = min(kb + 1, KB - 1), kn2 = min(kb + 2, KB - 1);
         float as_nxt[SM], bs_nxt = 0.f;
 
         // fold the tile left over from the previous K block with that block's scale, then switch scales
@@ -177,16 +186,25 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 
 #pragma unroll
         for (int i = 0; i < SN; ++i) {
-            // LDS reads complete in order: all but the newest two (the fragment of step i+1) have landed
-            if (i + 1 < SN) __builtin_amdgcn_s_waitcnt(0xc27f);          // lgkmcnt(2)
-            else            __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0)
-            __builtin_amdgcn_sched_barrier(0);
-            v8i nf2 = nf0;
-            if (i + 2 < SN)
+            if (i == kSync) {
+                // every LDS read of this stage has returned and this wavefront's share of the other stage
+                // (and the next block's scales) has landed
+#pragma unroll
+                for (int j = 0; j < SM; ++j) sc_nxt[j] = as_nxt[j] * bs_nxt;
+                __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // weight rows are streamed two steps ahead; the last two steps fetch steps 0 and 1 of the next block
+            v8i nf2;
+            if (i < kSync)
                 nf2 = join(*(const v4i*)(bs_base + (i + 2) * 2048 + c0), *(const v4i*)(bs_base + (i + 2) * 2048 + c1));
+            else
+                nf2 = join(*(const v4i*)(bs_next + (i - kSync) * 2048 + c0), *(const v4i*)(bs_next + (i - kSync) * 2048 + c1));
             const v4f z = {0.f, 0.f, 0.f, 0.f};
             v4f p[SM];
             p[0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[0], z, 0, 0, 0, 0, 0, 0);
+            if (i == SN - 1) mf[0] = join(*(const v4i*)(as_next + c0), *(const v4i*)(as_next + c1));
             if (i > 0) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[i - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[i - 1][SM - 1][e]);
@@ -194,33 +212,37 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 #pragma unroll
             for (int j = 1; j < SM; ++j) {
                 p[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[j], z, 0, 0, 0, 0, 0, 0);
+                if (i == SN - 1) mf[j] = join(*(const v4i*)(as_next + j * 2048 + c0), *(const v4i*)(as_next + j * 2048 + c1));
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(p[j - 1][e], sc[j - 1], acc[i][j - 1][e]);
             }
-            // one eighth of the next K block's global -> LDS copy and one scale load per step: the memory
-            // pipeline sees a steady trickle instead of a burst that would stall instruction issue
-            issue_load(i, kn, stage ^ 1);
+            if (i >= kSync) {
+                // refill the stage this block has finished reading with block kb+2
+#pragma unroll
+                for (int t = 0; t < 4; ++t) issue_load((i - kSync) * 4 + t, kn2, stage);
+            }
             if (i < SM) as_nxt[i] = a_s[as_off[i] + (uint32_t)kn];
             if (i == SM) bs_nxt = bs_src[kn + vzero];     // through the vector path on purpose, see vzero
             pend = p[SM - 1];
             nf0 = nf1;
             nf1 = nf2;
-            if (i + 2 < SN) DSV3_SGB(0x100, 2);
+            DSV3_SGB(0x100, 2);
             DSV3_SGB(0x008, 1);
+            if (i == SN - 1) DSV3_SGB(0x100, 2);
             if (i > 0) DSV3_SGB(0x002, 4);
 #pragma unroll
-            for (int j = 1; j < SM; ++j) { DSV3_SGB(0x008, 1); DSV3_SGB(0x002, 4); }
+            for (int j = 1; j < SM; ++j) {
+                DSV3_SGB(0x008, 1);
+                if (i == SN - 1) DSV3_SGB(0x100, 2);
+                DSV3_SGB(0x002, 4);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
-
-#pragma unroll
-        for (int j = 0; j < SM; ++j) sc_nxt[j] = as_nxt[j] * bs_nxt;
-        __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0): this wavefront's share of the next stage has landed
-        __syncthreads();
     }
 #undef DSV3_SGB
 #pragma unroll
     for (int e = 0; e < 4; ++e) acc[SN - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[SN - 1][SM - 1][e]);
+    __builtin_amdgcn_s_waitcnt(0x0f70);             // the clamped refills of the last two blocks are still in flight
 
     // ---- epilogue: lane holds c[m][n .. n+3] for every (i, j)
     const bool vec_ok = (N % 4) == 0;
@@ -284,3 +306,4 @@ template int launch_prefill<DSV3_F16>(const void*, const float*, const void*, co
 template int launch_prefill<DSV3_F32>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t);
 
 }  // namespace dsv3
+
