@@ -78,4 +78,61 @@ int dsv3_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b
     return launch_fp8_gemm(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+int dsv3_fp8_gemm_grouped_tile_rows(void) { return grouped_tile_rows(); }
+
+int dsv3_group_tiles(const int32_t* counts, int groups, int max_tiles,
+                     int32_t* tile_group, int32_t* tile_row0, int32_t* tile_rows, void* stream) {
+    if (groups < 0 || max_tiles < 0) return DSV3_ERR_BAD_SHAPE;
+    if (max_tiles == 0) return DSV3_OK;
+    if ((groups > 0 && !counts) || !tile_group || !tile_row0 || !tile_rows) return DSV3_ERR_NULL_POINTER;
+    return launch_group_tiles(counts, groups, grouped_tile_rows(), max_tiles, tile_group, tile_row0, tile_rows,
+                              (hipStream_t)stream);
+}
+
+int dsv3_fp8_gemm_grouped(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
+                          const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
+                          void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                          const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
+                          int64_t num_tiles, void* stream) {
+    if (!valid_dtype(c_dtype)) return DSV3_ERR_BAD_DTYPE;
+    if (m < 0 || n < 0 || k < 0 || a_num_rows < 0 || num_tiles < 0 || b_group_stride < 0 || bs_group_stride < 0)
+        return DSV3_ERR_BAD_SHAPE;
+    if (k % 128 != 0 || k == 0) return DSV3_ERR_BAD_SHAPE;
+    if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (m == 0 || n == 0 || num_tiles == 0) return DSV3_OK;
+    if (!a || !a_s || !b || !b_s || !c || !tile_group || !tile_row0 || !tile_rows) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(a, 16) || !aligned(b, 16) || b_group_stride % 16 != 0 || !aligned(a_s, 4) || !aligned(b_s, 4) ||
+        !aligned(c, c_dtype == DSV3_F32 ? 16 : 8))
+        return DSV3_ERR_MISALIGNED;
+    if (!grouped_supported(a_num_rows, n, k)) return DSV3_ERR_BAD_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    switch (c_dtype) {
+        case DSV3_BF16: return launch_grouped<DSV3_BF16>(a, a_s, a_rows, b, b_s, c, m, n, k, num_tiles, tile_group, tile_row0, tile_rows, b_group_stride, bs_group_stride, st);
+        case DSV3_F16:  return launch_grouped<DSV3_F16>(a, a_s, a_rows, b, b_s, c, m, n, k, num_tiles, tile_group, tile_row0, tile_rows, b_group_stride, bs_group_stride, st);
+        default:        return launch_grouped<DSV3_F32>(a, a_s, a_rows, b, b_s, c, m, n, k, num_tiles, tile_group, tile_row0, tile_rows, b_group_stride, bs_group_stride, st);
+    }
+}
+
+int dsv3_swiglu_quant(const void* h, int h_dtype, void* y, float* s, int64_t rows, int64_t inter,
+                      int block_size, int scale_fmt, void* stream) {
+    if (h_dtype != DSV3_BF16) return DSV3_ERR_BAD_DTYPE;
+    if (scale_fmt != DSV3_SCALE_FMT_NONE && scale_fmt != DSV3_SCALE_FMT_UE8M0) return DSV3_ERR_BAD_DTYPE;
+    if (block_size != 128) return DSV3_ERR_BAD_BLOCK;
+    if (rows < 0 || inter < 0 || inter % 128 != 0) return DSV3_ERR_BAD_SHAPE;
+    if (rows == 0 || inter == 0) return DSV3_OK;
+    if (!h || !y || !s) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(h, 16) || !aligned(y, 8) || !aligned(s, 4)) return DSV3_ERR_MISALIGNED;
+    return launch_swiglu_quant(h, y, s, rows, inter, scale_fmt, (hipStream_t)stream);
+}
+
+int dsv3_moe_combine(const void* expert_out, int dtype, const int32_t* rows, const void* weights,
+                     const void* shared, void* y, int64_t tokens, int topk, int64_t dim, void* stream) {
+    if (dtype != DSV3_BF16) return DSV3_ERR_BAD_DTYPE;
+    if (tokens < 0 || topk < 0 || dim < 0 || dim % 8 != 0 || tokens > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (tokens == 0 || dim == 0) return DSV3_OK;
+    if (!y || (topk > 0 && (!expert_out || !rows || !weights))) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(expert_out, 16) || !aligned(shared, 16) || !aligned(y, 16)) return DSV3_ERR_MISALIGNED;
+    return launch_moe_combine(expert_out, rows, weights, shared, y, tokens, topk, dim, (hipStream_t)stream);
+}
+
 }  // extern "C"

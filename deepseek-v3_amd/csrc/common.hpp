@@ -83,5 +83,16 @@ int launch_skinny(const void* a, const float* a_s, const void* b, const float* b
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, hipStream_t stream);
+int grouped_tile_rows();
+bool grouped_supported(int64_t a_num_rows, int64_t n, int64_t k);
+template <int CD>
+int launch_grouped(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s, void* c,
+                   int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
+                   const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream);
+int launch_swiglu_quant(const void* h, void* y, float* s, int64_t rows, int64_t inter, int scale_fmt, hipStream_t st);
+int launch_moe_combine(const void* out, const int* rows, const void* w, const void* shared, void* y,
+                       int64_t tokens, int topk, int64_t dim, hipStream_t st);
+int launch_group_tiles(const int* counts, int groups, int tile_rows, int max_tiles,
+                       int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st);
 
 }  // namespace dsv3

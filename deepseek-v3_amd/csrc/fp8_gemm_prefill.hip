@@ -45,28 +45,61 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
     return r;
 }
 
-template <int CD>
+// Grouped mode (G): the rows of a (and of c) are cut into groups, each multiplied by its own weight matrix --
+// the per-expert token lists of the reference's MoE layer (inference/model.py:684-689).  A row tile belongs to one
+// group; a table built on the device (no host round trip for the group sizes) gives each tile slot its group,
+// its first row in c and its row count, or group -1 for an unused slot.  a_rows, when given, maps a row of c to
+// the row of a it reads (token gather); otherwise a and c share row numbers.
+struct GroupTable {
+    const int* tile_group;   // [tiles_m]
+    const int* tile_row0;    // [tiles_m] first row of the tile in c (and in a_rows)
+    const int* tile_rows;    // [tiles_m] 1 .. BM
+    const int* a_rows;       // [rows of c] or nullptr
+    int64_t b_stride;        // bytes between consecutive groups' weights
+    int64_t bs_stride;       // floats between consecutive groups' weight scales
+};
+
+template <int CD, bool G>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
-        int M, int N, int K, int tiles_m, int tiles_n) {
+        int M, int N, int K, int tiles_m, int tiles_n, GroupTable g) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
-    // ---- workgroup -> tile: contiguous run of tiles per XCD, bands of GROUP_M tile rows
+    // ---- workgroup -> tile: contiguous run of tiles per XCD; dense mode walks bands of GROUP_M tile rows,
+    // grouped mode keeps the column tiles of one row tile together (they share the gathered rows of a)
     const int T = tiles_m * tiles_n;
     int pid = blockIdx.x;
     {
         const int q = T / 8, r = T % 8, x = pid % 8;
         pid = x * q + (x < r ? x : r) + pid / 8;
     }
-    constexpr int GROUP_M = 4;
-    const int band = pid / (GROUP_M * tiles_n);
-    const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
-    const int in_band = pid - band * GROUP_M * tiles_n;
-    const int tm = band * GROUP_M + in_band % band_rows;
-    const int tn = in_band / band_rows;
-    const int m0 = tm * BM, n0 = tn * BN;
+    int m0, n0, rows_here;              // first row of the tile in c, first column, valid rows
+    if (G) {
+        const int tm = pid / tiles_n, tn = pid - tm * tiles_n;
+        const int grp = g.tile_group[tm];
+        if (grp < 0) return;            // uniform over the workgroup, before any barrier
+        m0 = g.tile_row0[tm];
+        rows_here = g.tile_rows[tm];
+        n0 = tn * BN;
+        b += (size_t)grp * g.b_stride;
+        b_s += (size_t)grp * g.bs_stride;
+    } else {
+        constexpr int GROUP_M = 4;
+        const int band = pid / (GROUP_M * tiles_n);
+        const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+        const int in_band = pid - band * GROUP_M * tiles_n;
+        const int tm = band * GROUP_M + in_band % band_rows;
+        const int tn = in_band / band_rows;
+        m0 = tm * BM; n0 = tn * BN;
+        rows_here = min(BM, M - m0);
+    }
+    // row of a behind row r of the tile; rows past the tile's end repeat its last row (their results are dropped)
+    auto a_row = [&](int r) -> uint32_t {
+        const int rr = m0 + min(r, rows_here - 1);
+        return (uint32_t)((G && g.a_rows) ? g.a_rows[rr] : rr);
+    };
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -82,7 +115,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const int q = i * 8 + wave;
         const int row = (q & 31) * 8 + (lane >> 3);              // row inside A or B
         const int ch = (lane & 7) ^ swz(row);
-        if (i < 4) src_off[i] = (uint32_t)min(m0 + row, M - 1) * (uint32_t)K + ch * 16;
+        if (i < 4) src_off[i] = a_row(row) * (uint32_t)K + ch * 16;
         else       src_off[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + ch * 16;
     }
     auto issue_load = [&](int i, int kb, int stage) {
@@ -115,7 +148,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     uint32_t as_off[SM];
 #pragma unroll
     for (int j = 0; j < SM; ++j)
-        as_off[j] = (uint32_t)min(m0 + wm * WM + j * 16 + fr, M - 1) * (uint32_t)KB;
+        as_off[j] = a_row(wm * WM + j * 16 + fr) * (uint32_t)KB;
     const int nb_last = (N - 1) / 128;
     const float* bs_src = b_s + (size_t)min((n0 + wn * WN) / 128, nb_last) * KB;
 
@@ -248,8 +281,9 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const bool vec_ok = (N % 4) == 0;
 #pragma unroll
     for (int j = 0; j < SM; ++j) {
-        const int m = m0 + wm * WM + j * 16 + fr;
-        if (m >= M) continue;
+        const int r = wm * WM + j * 16 + fr;
+        if (r >= rows_here) continue;
+        const int m = m0 + r;
 #pragma unroll
         for (int i = 0; i < SN; ++i) {
             const int n = n0 + wn * WN + i * 16 + fq * 4;
@@ -280,13 +314,14 @@ bool prefill_supported(int64_t m, int64_t n, int64_t k) {
     return k >= 128 && m * k < (1ll << 32) && n * k < (1ll << 32);
 }
 
-template <int CD>
-int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
-                   int64_t m, int64_t n, int64_t k, hipStream_t stream) {
+namespace {
+template <int CD, bool G>
+int launch_kernel(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+                  int64_t m, int64_t n, int64_t k, int64_t tm, prefill::GroupTable g, hipStream_t stream) {
     using namespace prefill;
-    const int64_t tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
+    const int64_t tn = (n + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
-    auto kern = fp8_gemm_prefill_kernel<CD>;
+    auto kern = fp8_gemm_prefill_kernel<CD, G>;
     static bool granted[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
@@ -297,13 +332,42 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(THREADS), LDS_BYTES, stream,
                        (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c,
-                       (int)m, (int)n, (int)k, (int)tm, (int)tn);
+                       (int)m, (int)n, (int)k, (int)tm, (int)tn, g);
     return launch_status();
 }
+}  // namespace
 
-template int launch_prefill<DSV3_BF16>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t);
-template int launch_prefill<DSV3_F16>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t);
-template int launch_prefill<DSV3_F32>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t);
+template <int CD>
+int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+                   int64_t m, int64_t n, int64_t k, hipStream_t stream) {
+    return launch_kernel<CD, false>(a, a_s, b, b_s, c, m, n, k, (m + prefill::BM - 1) / prefill::BM,
+                                    prefill::GroupTable{}, stream);
+}
+
+// Rows per tile slot of the grouped kernel: the caller's tile table is built for this height.
+int grouped_tile_rows() { return prefill::BM; }
+
+// a: [a_num_rows, k] fp8 with scales a_s; c: [m, n]; group tables as described at GroupTable.  Byte offsets of a
+// and of one group's weights must fit 32 bits.
+bool grouped_supported(int64_t a_num_rows, int64_t n, int64_t k) {
+    return k >= 128 && k % 128 == 0 && n >= 1 && a_num_rows * k < (1ll << 32) && n * k < (1ll << 32);
+}
+
+template <int CD>
+int launch_grouped(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s, void* c,
+                   int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
+                   const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream) {
+    prefill::GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
+    return launch_kernel<CD, true>(a, a_s, b, b_s, c, m, n, k, num_tiles, g, stream);
+}
+
+#define DSV3_INST(CD) \
+    template int launch_prefill<CD>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t); \
+    template int launch_grouped<CD>(const void*, const float*, const int*, const void*, const float*, void*, int64_t, int64_t, int64_t, \
+                                    int64_t, const int*, const int*, const int*, int64_t, int64_t, hipStream_t);
+DSV3_INST(DSV3_BF16)
+DSV3_INST(DSV3_F16)
+DSV3_INST(DSV3_F32)
+#undef DSV3_INST
 
 }  // namespace dsv3
-

@@ -1,0 +1,178 @@
+// Stream kernels around the grouped fp8_gemm of a mixture-of-experts layer
+// (reference: inference/model.py:601-633 Expert, :669-693 MoE.forward).
+//
+//   swiglu_quant   g = silu(h1) * h3 rounded as the reference's bf16 tensor ops round it, then act_quant(g)
+//                  (inference/model.py:633 feeding Linear -> inference/kernel.py:23-35) in one pass
+//   moe_combine    y[t] = (sum over the token's experts, ascending expert index, of out * weight) + shared,
+//                  every step rounded to bf16 exactly where model.py:689-693 rounds
+//   group_tiles    per-group row counts -> the tile table the grouped GEMM reads (no host round trip)
+#include "common.hpp"
+
+namespace dsv3 {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float round_bf16(float v) { return bf16lo_to_f32(pack_bf16(v, 0.f) & 0xffffu); }
+
+template <int CTRL> __device__ __forceinline__ float dpp_max(float v) {
+    int o = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
+    return fmaxf(v, __builtin_bit_cast(float, o));
+}
+
+// h: [rows, 2*inter] bf16 (h1 | h3 side by side), y: [rows, inter] e4m3, s: [rows, inter/128].
+// A lane owns 8 consecutive output columns; the 16 lanes of a DPP row own one 128-wide scale block.
+template <bool UE8M0>
+__global__ __launch_bounds__(kThreads) void swiglu_quant_kernel(
+        const v4u* __restrict__ h, v2u* __restrict__ y, float* __restrict__ s,
+        int64_t n_chunks, int chunks_per_row) {
+    const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const bool live = c < n_chunks;
+    const int64_t cc = live ? c : 0;
+    const int64_t row = cc / chunks_per_row;
+    const int col = (int)(cc - row * chunks_per_row);
+    const v4u a = __builtin_nontemporal_load(h + row * 2 * chunks_per_row + col);
+    const v4u b = __builtin_nontemporal_load(h + row * 2 * chunks_per_row + chunks_per_row + col);
+    float g[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float x1 = (i & 1) ? bf16hi_to_f32(a[i >> 1]) : bf16lo_to_f32(a[i >> 1]);
+        const float x3 = (i & 1) ? bf16hi_to_f32(b[i >> 1]) : bf16lo_to_f32(b[i >> 1]);
+        const float sl = round_bf16(x1 / (1.0f + expf(-x1)));     // F.silu on a bf16 tensor: binary32 inside, bf16 out
+        g[i] = live ? round_bf16(sl * x3) : 0.f;                  // bf16 * bf16 -> bf16
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(g[i]));
+    amax = dpp_max<0xB1>(amax);    // quad_perm [1,0,3,2]
+    amax = dpp_max<0x4E>(amax);    // quad_perm [2,3,0,1]
+    amax = dpp_max<0x141>(amax);   // row_half_mirror
+    amax = dpp_max<0x140>(amax);   // row_mirror
+    amax = fmaxf(amax, 1e-4f);
+    float sc = amax / 448.f;
+    if (UE8M0) {
+        uint32_t bits = f32_as_u32(sc);
+        bits = ((bits >> 23) + ((bits & 0x7fffffu) ? 1u : 0u)) << 23;
+        sc = u32_as_f32(bits);
+    }
+    // correctly rounded g / sc for bf16 g with |g| <= amax (same evaluation as act_quant)
+    const float r = 1.0f / sc;
+    float q[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float q0 = g[i] * r;
+        const float e = __builtin_fmaf(-q0, sc, g[i]);
+        q[i] = __builtin_copysignf(__builtin_fmaf(e, r, q0), g[i]);
+    }
+    if (live) {
+        v2u o;
+        o.x = pack_fp8x4(q[0], q[1], q[2], q[3]);
+        o.y = pack_fp8x4(q[4], q[5], q[6], q[7]);
+        __builtin_nontemporal_store(o, &y[c]);
+        if ((c & 15) == 0) s[c >> 4] = sc;
+    }
+}
+
+// One workgroup per token.  rows[t, k] is the row of `out` holding the token's k-th expert output in ascending
+// expert order, w[t, k] the matching routing weight (bf16).
+__global__ __launch_bounds__(kThreads) void moe_combine_kernel(
+        const v4u* __restrict__ out, const int* __restrict__ rows, const uint16_t* __restrict__ w,
+        const v4u* __restrict__ shared, v4u* __restrict__ y, int topk, int chunks_per_row) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < chunks_per_row; c += kThreads) {
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+        for (int k = 0; k < topk; ++k) {
+            const int r = rows[t * topk + k];
+            const float wk = bf16lo_to_f32(w[t * topk + k]);
+            const v4u v = out[(int64_t)r * chunks_per_row + c];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x = (i & 1) ? bf16hi_to_f32(v[i >> 1]) : bf16lo_to_f32(v[i >> 1]);
+                acc[i] = round_bf16(acc[i] + round_bf16(x * wk));       // y[idx] += expert_out * weight
+            }
+        }
+        if (shared) {
+            const v4u z = shared[(int64_t)t * chunks_per_row + c];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x = (i & 1) ? bf16hi_to_f32(z[i >> 1]) : bf16lo_to_f32(z[i >> 1]);
+                acc[i] = round_bf16(acc[i] + x);                         // y + z
+            }
+        }
+        v4u o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = pack_bf16(acc[2 * i], acc[2 * i + 1]);
+        y[(int64_t)t * chunks_per_row + c] = o;
+    }
+}
+
+// counts[g] rows per group, groups laid out back to back in c.  Tile slots are handed out group by group,
+// ceil(count / tile_rows) each; slots past the last one are marked unused.  One workgroup, any group count.
+__global__ __launch_bounds__(kThreads) void group_tiles_kernel(
+        const int* __restrict__ counts, int groups, int tile_rows, int max_tiles,
+        int* __restrict__ tile_group, int* __restrict__ tile_row0, int* __restrict__ tile_nrows) {
+    __shared__ int tile_base[kThreads + 1], row_base[kThreads + 1];
+    int done_tiles = 0, done_rows = 0;
+    for (int g0 = 0; g0 < groups; g0 += kThreads) {
+        const int g = g0 + threadIdx.x;
+        const int cnt = g < groups ? counts[g] : 0;
+        const int nt = (cnt + tile_rows - 1) / tile_rows;
+        // exclusive scans over this batch of groups (Hillis-Steele in LDS)
+        tile_base[threadIdx.x + 1] = nt; row_base[threadIdx.x + 1] = cnt;
+        if (threadIdx.x == 0) { tile_base[0] = 0; row_base[0] = 0; }
+        __syncthreads();
+        for (int d = 1; d < kThreads; d <<= 1) {
+            const int a = threadIdx.x + 1 >= d + 1 ? tile_base[threadIdx.x + 1 - d] : 0;
+            const int b = threadIdx.x + 1 >= d + 1 ? row_base[threadIdx.x + 1 - d] : 0;
+            __syncthreads();
+            tile_base[threadIdx.x + 1] += a; row_base[threadIdx.x + 1] += b;
+            __syncthreads();
+        }
+        const int t0 = done_tiles + tile_base[threadIdx.x], r0 = done_rows + row_base[threadIdx.x];
+        for (int i = 0; i < nt; ++i) {
+            if (t0 + i < max_tiles) {
+                tile_group[t0 + i] = g;
+                tile_row0[t0 + i] = r0 + i * tile_rows;
+                tile_nrows[t0 + i] = min(tile_rows, cnt - i * tile_rows);
+            }
+        }
+        done_tiles += tile_base[kThreads]; done_rows += row_base[kThreads];
+        __syncthreads();
+    }
+    for (int t = done_tiles + threadIdx.x; t < max_tiles; t += kThreads) {
+        tile_group[t] = -1; tile_row0[t] = 0; tile_nrows[t] = 0;
+    }
+}
+
+}  // namespace
+
+int launch_swiglu_quant(const void* h, void* y, float* s, int64_t rows, int64_t inter, int scale_fmt, hipStream_t st) {
+    const int64_t n_chunks = rows * inter / 8;
+    const int64_t grid = (n_chunks + kThreads - 1) / kThreads;
+    if (grid > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (scale_fmt == DSV3_SCALE_FMT_UE8M0)
+        hipLaunchKernelGGL(swiglu_quant_kernel<true>, dim3((unsigned)grid), dim3(kThreads), 0, st,
+                           (const v4u*)h, (v2u*)y, s, n_chunks, (int)(inter / 8));
+    else
+        hipLaunchKernelGGL(swiglu_quant_kernel<false>, dim3((unsigned)grid), dim3(kThreads), 0, st,
+                           (const v4u*)h, (v2u*)y, s, n_chunks, (int)(inter / 8));
+    return launch_status();
+}
+
+int launch_moe_combine(const void* out, const int* rows, const void* w, const void* shared, void* y,
+                       int64_t tokens, int topk, int64_t dim, hipStream_t st) {
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)tokens), dim3(kThreads), 0, st,
+                       (const v4u*)out, rows, (const uint16_t*)w, (const v4u*)shared, (v4u*)y, topk, (int)(dim / 8));
+    return launch_status();
+}
+
+int launch_group_tiles(const int* counts, int groups, int tile_rows, int max_tiles,
+                       int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st) {
+    hipLaunchKernelGGL(group_tiles_kernel, dim3(1), dim3(kThreads), 0, st,
+                       counts, groups, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows);
+    return launch_status();
+}
+
+}  // namespace dsv3

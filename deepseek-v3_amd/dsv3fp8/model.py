@@ -19,6 +19,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
+from . import ops
 from .kernel import act_quant, fp8_gemm, weight_dequant
 
 world_size = 1
@@ -179,7 +180,15 @@ class Expert(nn.Module):
 
 class MoE(nn.Module):
     """Mixture-of-experts layer (model.py:636-693): route, run every expert that received tokens on its token
-    list, scatter-add the weighted outputs in expert order, add the shared expert."""
+    list, scatter-add the weighted outputs in expert order, add the shared expert.
+
+    With FP8 experts and ``gemm_impl == "fp8"`` the token lists stay on the device: the routed experts run as
+    two grouped GEMMs over expert-sorted rows (w1|w3 stacked, then w2) with SwiGLU and the re-quantisation fused
+    between them, and one kernel adds the weighted outputs per token in the order the reference's loop does.
+    ``MoE.grouped = False`` selects the reference's expert-by-expert loop (same kernels, one expert at a time).
+    """
+
+    grouped: bool = True
 
     def __init__(self, args: ModelArgs):
         super().__init__()
@@ -195,11 +204,72 @@ class MoE(nn.Module):
                                       if self.experts_start_idx <= i < self.experts_end_idx else None
                                       for i in range(self.n_routed_experts)])
         self.shared_experts = MLP(args.dim, args.n_shared_experts * args.moe_inter_dim)
+        self._stacked = None
+
+    def stack_experts(self) -> None:
+        """Move the routed experts' weights into two contiguous buffers, [E, 2*inter, dim] (w1 over w3) and
+        [E, dim, inter] (w2), with their scales alongside; each expert's parameters become views of them, so
+        ``load_model``-style in-place copies and the expert-by-expert path keep working on the same memory."""
+        if self._stacked is not None:
+            return
+        exs = list(self.experts)
+        inter, dim = exs[0].w1.out_features, self.dim
+        assert inter % block_size == 0 and dim % block_size == 0
+        dev, fp8 = exs[0].w1.weight.device, exs[0].w1.weight.dtype
+        n = len(exs)
+        ib, db = inter // block_size, dim // block_size
+        with torch.no_grad():
+            w13 = torch.empty(n, 2 * inter, dim, dtype=fp8, device=dev)
+            s13 = torch.empty(n, 2 * ib, db, dtype=torch.float32, device=dev)
+            w2 = torch.empty(n, dim, inter, dtype=fp8, device=dev)
+            s2 = torch.empty(n, db, ib, dtype=torch.float32, device=dev)
+            for i, ex in enumerate(exs):
+                for lin, wv, sv in ((ex.w1, w13[i, :inter], s13[i, :ib]), (ex.w3, w13[i, inter:], s13[i, ib:]),
+                                    (ex.w2, w2[i], s2[i])):
+                    wv.view(torch.uint8).copy_(lin.weight.data.view(torch.uint8))
+                    sv.copy_(lin.scale.data)
+                    lin.weight.data = wv
+                    lin.scale.data = sv
+        self._stacked = (w13, s13, w2, s2)
+
+    def _grouped_ok(self, x: torch.Tensor) -> bool:
+        ex = self.experts[self.experts_start_idx]
+        return (self.grouped and gemm_impl == "fp8" and world_size == 1 and x.is_cuda
+                and ex.w1.weight.element_size() == 1 and x.dtype == torch.bfloat16
+                and torch.get_default_dtype() == torch.bfloat16
+                and ex.w1.out_features % block_size == 0 and self.dim % block_size == 0)
+
+    def _forward_grouped(self, x: torch.Tensor, weights: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+        self.stack_experts()
+        w13, s13, w2, s2 = self._stacked
+        tokens, topk = indices.shape
+        pairs = tokens * topk
+        flat = indices.reshape(-1)
+        order = torch.argsort(flat, stable=True)                       # expert-sorted row -> (token, slot) pair
+        counts = torch.bincount(flat, minlength=self.n_routed_experts).to(torch.int32)
+        a_rows = (order // topk).to(torch.int32)                       # token behind each expert-sorted row
+        max_tiles = pairs // ops.grouped_tile_rows() + self.n_routed_experts
+        tile_group, tile_row0, tile_rows = torch.ops.dsv3fp8.group_tiles(counts, max_tiles)
+        fmt = ops._lib.SCALE_FMT_UE8M0 if Linear.scale_fmt == "ue8m0" else ops._lib.SCALE_FMT_NONE
+        code = ops.dtype_code(torch.get_default_dtype())
+        xq, xs = act_quant(x, block_size, Linear.scale_fmt)           # quantised once: 1x128 blocks are per token
+        h = torch.ops.dsv3fp8.fp8_gemm_grouped(xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, code)
+        gq, gs = torch.ops.dsv3fp8.swiglu_quant(h, block_size, fmt)
+        out = torch.ops.dsv3fp8.fp8_gemm_grouped(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code)
+        # the reference adds a token's expert outputs in ascending expert index (its loop order, model.py:684-689)
+        slot = indices.argsort(dim=1)
+        pos = torch.empty_like(order)
+        pos[order] = torch.arange(pairs, device=order.device)
+        rows = pos.view(tokens, topk).gather(1, slot).to(torch.int32)
+        z = self.shared_experts(x)
+        return torch.ops.dsv3fp8.moe_combine(out, rows, weights.gather(1, slot).contiguous(), z.contiguous())
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         shape = x.size()
         x = x.view(-1, self.dim)
         weights, indices = self.gate(x)
+        if self._grouped_ok(x):
+            return self._forward_grouped(x, weights, indices).view(shape)
         y = torch.zeros_like(x)
         counts = torch.bincount(indices.flatten(), minlength=self.n_routed_experts).tolist()
         for i in range(self.experts_start_idx, self.experts_end_idx):

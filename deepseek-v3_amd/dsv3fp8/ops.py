@@ -1,7 +1,8 @@
 """PyTorch-ROCm custom ops over the C ABI.
 
-``torch.ops.dsv3fp8.{act_quant, weight_dequant, fp8_gemm}`` take and return
-torch tensors; the device implementations hand raw device pointers and the
+``torch.ops.dsv3fp8.{act_quant, weight_dequant, fp8_gemm}`` and the grouped
+mixture-of-experts ops ``{group_tiles, fp8_gemm_grouped, swiglu_quant, moe_combine}``
+take and return torch tensors; the device implementations hand raw device pointers and the
 current HIP stream of the tensors' device to libdsv3fp8.so.  Only a device
 ("CUDA" dispatch key, which is HIP on ROCm) implementation and a shape-only Meta
 implementation are registered: calling an op on CPU tensors raises.
@@ -22,6 +23,11 @@ _libdef = torch.library.Library("dsv3fp8", "DEF")
 _libdef.define("act_quant(Tensor x, int block_size, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("weight_dequant(Tensor x, Tensor s, int block_size, int out_dtype) -> Tensor")
 _libdef.define("fp8_gemm(Tensor a, Tensor a_s, Tensor b, Tensor b_s, int out_dtype) -> Tensor")
+_libdef.define("group_tiles(Tensor counts, int max_tiles) -> (Tensor, Tensor, Tensor)")
+_libdef.define("fp8_gemm_grouped(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b, Tensor b_s, int rows, "
+               "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int out_dtype) -> Tensor")
+_libdef.define("swiglu_quant(Tensor h, int block_size, int scale_fmt) -> (Tensor, Tensor)")
+_libdef.define("moe_combine(Tensor expert_out, Tensor rows, Tensor weights, Tensor? shared) -> Tensor")
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -98,7 +104,91 @@ def _fp8_gemm_meta(a, a_s, b, b_s, out_dtype):
     return a.new_empty(*a.size()[:-1], b.size(0), dtype=_CODE_DTYPE[out_dtype])
 
 
+def grouped_tile_rows() -> int:
+    return int(_lib.lib.dsv3_fp8_gemm_grouped_tile_rows())
+
+
+def _group_tiles_dev(counts: torch.Tensor, max_tiles: int):
+    assert counts.dtype == torch.int32 and counts.is_contiguous() and counts.dim() == 1
+    out = torch.empty(3, max(max_tiles, 1), dtype=torch.int32, device=counts.device)
+    with torch.cuda.device(counts.device):
+        rc = _lib.lib.dsv3_group_tiles(counts.data_ptr(), counts.numel(), max_tiles,
+                                       out[0].data_ptr(), out[1].data_ptr(), out[2].data_ptr(), _stream(counts))
+    _lib.check(rc, "dsv3_group_tiles")
+    return out[0, :max_tiles], out[1, :max_tiles], out[2, :max_tiles]
+
+
+def _group_tiles_meta(counts, max_tiles):
+    return tuple(counts.new_empty(max_tiles, dtype=torch.int32) for _ in range(3))
+
+
+def _fp8_gemm_grouped_dev(a, a_s, a_rows, b, b_s, rows: int, tile_group, tile_row0, tile_rows, out_dtype: int):
+    # a: [A, k] fp8; b: [groups, n, k] fp8; b_s: [groups, ceil(n/128), k/128]; result [rows, n]
+    assert a.dim() == 2 and b.dim() == 3 and b_s.dim() == 3 and a.is_contiguous() and b.is_contiguous()
+    assert a_s.is_contiguous() and b_s.is_contiguous() and b.size(0) == b_s.size(0)
+    for t in (tile_group, tile_row0, tile_rows):
+        assert t.dtype == torch.int32 and t.is_contiguous() and t.numel() == tile_group.numel()
+    if a_rows is not None:
+        assert a_rows.dtype == torch.int32 and a_rows.is_contiguous() and a_rows.numel() == rows
+    k, n = a.size(1), b.size(1)
+    assert b.size(2) == k
+    c = a.new_empty(rows, n, dtype=_CODE_DTYPE[out_dtype])
+    with torch.cuda.device(a.device):
+        rc = _lib.lib.dsv3_fp8_gemm_grouped(
+            a.data_ptr(), a_s.data_ptr(), a_rows.data_ptr() if a_rows is not None else None, a.size(0),
+            b.data_ptr(), b_s.data_ptr(), b.stride(0), b_s.stride(0),
+            c.data_ptr(), out_dtype, rows, n, k,
+            tile_group.data_ptr(), tile_row0.data_ptr(), tile_rows.data_ptr(), tile_group.numel(), _stream(a))
+    _lib.check(rc, "dsv3_fp8_gemm_grouped")
+    return c
+
+
+def _fp8_gemm_grouped_meta(a, a_s, a_rows, b, b_s, rows, tile_group, tile_row0, tile_rows, out_dtype):
+    return a.new_empty(rows, b.size(1), dtype=_CODE_DTYPE[out_dtype])
+
+
+def _swiglu_quant_dev(h: torch.Tensor, block_size: int, scale_fmt: int):
+    assert h.dim() == 2 and h.is_contiguous() and h.size(1) % 2 == 0
+    rows, inter = h.size(0), h.size(1) // 2
+    y = h.new_empty(rows, inter, dtype=FP8)
+    s = h.new_empty(rows, inter // block_size, dtype=torch.float32)
+    with torch.cuda.device(h.device):
+        rc = _lib.lib.dsv3_swiglu_quant(h.data_ptr(), dtype_code(h.dtype), y.data_ptr(), s.data_ptr(),
+                                        rows, inter, block_size, scale_fmt, _stream(h))
+    _lib.check(rc, "dsv3_swiglu_quant")
+    return y, s
+
+
+def _swiglu_quant_meta(h, block_size, scale_fmt):
+    rows, inter = h.size(0), h.size(1) // 2
+    return h.new_empty(rows, inter, dtype=FP8), h.new_empty(rows, inter // block_size, dtype=torch.float32)
+
+
+def _moe_combine_dev(expert_out, rows, weights, shared):
+    assert expert_out.dim() == 2 and expert_out.is_contiguous() and rows.dtype == torch.int32
+    assert rows.is_contiguous() and weights.is_contiguous() and rows.shape == weights.shape
+    assert weights.dtype == expert_out.dtype and (shared is None or (shared.is_contiguous() and shared.dtype == expert_out.dtype))
+    tokens, topk = rows.shape
+    y = expert_out.new_empty(tokens, expert_out.size(1))
+    with torch.cuda.device(expert_out.device):
+        rc = _lib.lib.dsv3_moe_combine(expert_out.data_ptr(), dtype_code(expert_out.dtype), rows.data_ptr(),
+                                       weights.data_ptr(), shared.data_ptr() if shared is not None else None,
+                                       y.data_ptr(), tokens, topk, expert_out.size(1), _stream(expert_out))
+    _lib.check(rc, "dsv3_moe_combine")
+    return y
+
+
+def _moe_combine_meta(expert_out, rows, weights, shared):
+    return expert_out.new_empty(rows.size(0), expert_out.size(1))
+
+
 _libimpl = torch.library.Library("dsv3fp8", "IMPL")
+for _name, _dev, _meta in (("group_tiles", _group_tiles_dev, _group_tiles_meta),
+                           ("fp8_gemm_grouped", _fp8_gemm_grouped_dev, _fp8_gemm_grouped_meta),
+                           ("swiglu_quant", _swiglu_quant_dev, _swiglu_quant_meta),
+                           ("moe_combine", _moe_combine_dev, _moe_combine_meta)):
+    _libimpl.impl(_name, _dev, "CUDA")
+    _libimpl.impl(_name, _meta, "Meta")
 _libimpl.impl("act_quant", _act_quant_dev, "CUDA")
 _libimpl.impl("weight_dequant", _weight_dequant_dev, "CUDA")
 _libimpl.impl("fp8_gemm", _fp8_gemm_dev, "CUDA")

@@ -109,6 +109,66 @@ int dsv3_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b
 /* Bytes of scratch dsv3_fp8_gemm needs for this problem (0 when none). */
 size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 
+/*
+ * ---- Mixture-of-experts layer on the same GEMM (inference/model.py:601-633 Expert, :669-693 MoE.forward) ----
+ *
+ * The reference walks its experts one by one: bincount(...).tolist() (a host sync, :683), then per expert
+ * where / gather / 3 x (act_quant + fp8_gemm) / scatter-add (:684-689).  The functions below compute the same
+ * values with the token lists kept on the device: rows of the activation matrix are grouped by expert
+ * ("groups"), every group is multiplied by its own weight matrix in one launch, and the weighted outputs are
+ * summed per token in ascending expert order, rounding to bf16 where the reference's tensor ops round.
+ */
+
+/* Height of a row tile of dsv3_fp8_gemm_grouped; dsv3_group_tiles cuts groups into tiles of this many rows. */
+int dsv3_fp8_gemm_grouped_tile_rows(void);
+
+/*
+ * Tile table for dsv3_fp8_gemm_grouped from per-group row counts (device int32 [groups]; the counts the
+ * reference takes from bincount at inference/model.py:683).  Groups are laid out back to back in row order;
+ * group g gets ceil(counts[g] / tile_rows) consecutive tile slots.  Writes three device int32 arrays of
+ * max_tiles entries: the group of each slot (-1 for unused slots), its first row and its row count.
+ * max_tiles >= total_rows / tile_rows + groups always suffices.
+ */
+int dsv3_group_tiles(const int32_t* counts, int groups, int max_tiles,
+                     int32_t* tile_group, int32_t* tile_row0, int32_t* tile_rows, void* stream);
+
+/*
+ * Grouped fp8_gemm (inference/kernel.py:145-172 applied per expert as in inference/model.py:684-689):
+ *     for every tile slot t with group g = tile_group[t] >= 0, rows r in [tile_row0[t], tile_row0[t]+tile_rows[t]):
+ *         c[r, :] = fp8_gemm( a[src(r), :], a_s[src(r), :], b + g*b_group_stride, b_s + g*bs_group_stride )
+ *     src(r) = a_rows ? a_rows[r] : r
+ * a: [a_num_rows, k] fp8, a_s: [a_num_rows, k/128]; a_rows (optional, device int32 [m]) gathers token rows;
+ * b: per-group weights [n, k] fp8, b_group_stride bytes apart; b_s: per-group scales [ceil(n/128), k/128],
+ * bs_group_stride floats apart; c: [m, n] of c_dtype.  Rows of c not covered by a tile are left untouched.
+ * k % 128 == 0, k >= 128; a_num_rows*k and n*k below 2^32.
+ */
+int dsv3_fp8_gemm_grouped(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
+                          const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
+                          void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                          const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
+                          int64_t num_tiles, void* stream);
+
+/*
+ * silu(h1) * h3 followed by act_quant, in one pass (inference/model.py:633 feeding the act_quant of w2's
+ * linear(), inference/model.py:159, inference/kernel.py:23-35):
+ *     g = bf16( bf16( silu(h1) ) * h3 );  (y, s) = act_quant(g, 128, scale_fmt)
+ * h: [rows, 2*inter] with h1 = h[:, :inter], h3 = h[:, inter:] (the two projections of one grouped GEMM);
+ * y: [rows, inter] e4m3; s: [rows, inter/128].  h_dtype must be DSV3_BF16 and block_size 128.
+ */
+int dsv3_swiglu_quant(const void* h, int h_dtype, void* y, float* s, int64_t rows, int64_t inter,
+                      int block_size, int scale_fmt, void* stream);
+
+/*
+ * Weighted scatter-add of the expert outputs plus the shared expert (inference/model.py:689-693):
+ *     y[t] = 0;  for j < topk:  y[t] = bf16( y[t] + bf16( expert_out[rows[t,j]] * weights[t,j] ) );
+ *     if shared:  y[t] = bf16( y[t] + shared[t] )
+ * rows: device int32 [tokens, topk], listing each token's rows of expert_out in ascending expert order (the
+ * order in which the reference's loop over experts adds them); weights: [tokens, topk]; all tensors of
+ * `dtype`, which must be DSV3_BF16; dim % 8 == 0.
+ */
+int dsv3_moe_combine(const void* expert_out, int dtype, const int32_t* rows, const void* weights,
+                     const void* shared, void* y, int64_t tokens, int topk, int64_t dim, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

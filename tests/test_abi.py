@@ -102,3 +102,50 @@ def test_python_wrappers_keep_the_reference_asserts():
         dsv3fp8.act_quant(torch.empty(256, 4, device="meta", dtype=torch.bfloat16).t())
     with pytest.raises(AssertionError, match="2 dimensions"):
         dsv3fp8.weight_dequant(torch.empty(2, 4, 4, device="meta", dtype=torch.float8_e4m3fn), torch.empty(1, 1, device="meta"))
+
+
+def test_grouped_validation(L):
+    f = L.lib.dsv3_fp8_gemm_grouped
+    assert L.lib.dsv3_fp8_gemm_grouped_tile_rows() > 0
+    ok = dict(a=A16, a_s=A16, a_rows=None, an=64, b=A16, b_s=A16, bst=128 * 128, sst=1, c=A16, cd=L.BF16,
+              m=64, n=128, k=128, tg=A16, t0=A16, tr=A16, nt=2, st=None)
+
+    def call(**kw):
+        v = {**ok, **kw}
+        return f(*[v[key] for key in ("a", "a_s", "a_rows", "an", "b", "b_s", "bst", "sst", "c", "cd", "m", "n", "k",
+                                      "tg", "t0", "tr", "nt", "st")])
+    assert call(a=None) == 1 and call(tg=None) == 1 and call(c=None) == 1
+    assert call(k=100) == 2 and call(k=0) == 2 and call(m=-1) == 2 and call(nt=-1) == 2
+    assert call(an=1 << 30, k=128 * 64) == 2                 # byte offsets of a beyond 32 bits
+    assert call(a=A16 + 4) == 4 and call(bst=100) == 4
+    assert call(cd=7) == 5
+    assert call(m=0, a=None, tg=None) == 0 and call(nt=0) == 0
+
+
+def test_group_tiles_validation(L):
+    f = L.lib.dsv3_group_tiles
+    assert f(None, 4, 8, A16, A16, A16, None) == 1
+    assert f(A16, 4, 8, None, A16, A16, None) == 1
+    assert f(A16, -1, 8, A16, A16, A16, None) == 2
+    assert f(A16, 4, 0, None, None, None, None) == 0
+
+
+def test_swiglu_quant_validation(L):
+    f = L.lib.dsv3_swiglu_quant
+    assert f(None, L.BF16, A16, A16, 4, 128, 128, 0, None) == 1
+    assert f(A16, L.F32, A16, A16, 4, 128, 128, 0, None) == 5          # bf16 only
+    assert f(A16, L.BF16, A16, A16, 4, 128, 64, 0, None) == 3
+    assert f(A16, L.BF16, A16, A16, 4, 100, 128, 0, None) == 2
+    assert f(A16, L.BF16, A16, A16, 4, 128, 128, 9, None) == 5
+    assert f(A16 + 2, L.BF16, A16, A16, 4, 128, 128, 0, None) == 4
+    assert f(None, L.BF16, None, None, 0, 128, 128, 0, None) == 0
+
+
+def test_moe_combine_validation(L):
+    f = L.lib.dsv3_moe_combine
+    assert f(None, L.BF16, A16, A16, None, A16, 4, 2, 128, None) == 1
+    assert f(A16, L.BF16, A16, A16, None, None, 4, 2, 128, None) == 1
+    assert f(A16, L.F16, A16, A16, None, A16, 4, 2, 128, None) == 5
+    assert f(A16, L.BF16, A16, A16, None, A16, 4, 2, 100, None) == 2
+    assert f(A16 + 2, L.BF16, A16, A16, None, A16, 4, 2, 128, None) == 4
+    assert f(None, L.BF16, None, None, None, None, 0, 2, 128, None) == 0

@@ -1,0 +1,182 @@
+"""GPU parity of the grouped mixture-of-experts path (group_tiles, fp8_gemm_grouped, swiglu_quant, moe_combine
+and MoE.forward on top of them) against the torch-CPU oracle of inference/model.py:601-633, 669-693."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+FP8 = torch.float8_e4m3fn
+
+
+@pytest.fixture(scope="module")
+def K():
+    import dsv3fp8
+    from dsv3fp8 import ops  # noqa: F401  (registers torch.ops.dsv3fp8)
+    return dsv3fp8
+
+
+def _tables(counts, max_tiles):
+    from dsv3fp8 import ops
+    R = ops.grouped_tile_rows()
+    tg, t0, tr = torch.ops.dsv3fp8.group_tiles(torch.tensor(counts, dtype=torch.int32, device="cuda"), max_tiles)
+    return R, tg, t0, tr
+
+
+@pytest.mark.parametrize("counts", [[5, 0, 300, 256, 1], [0, 0, 0], [700], list(range(0, 600, 7))])
+def test_group_tiles(K, counts):
+    total = sum(counts)
+    R, tg, t0, tr = _tables(counts, 1)
+    max_tiles = total // R + len(counts)
+    R, tg, t0, tr = _tables(counts, max_tiles)
+    exp, row = [], 0
+    for g, c in enumerate(counts):
+        for i in range(0, c, R):
+            exp.append((g, row + i, min(R, c - i)))
+        row += c
+    got = list(zip(tg.tolist(), t0.tolist(), tr.tolist()))
+    assert got[:len(exp)] == exp
+    assert all(g == -1 and n == 0 for g, _, n in got[len(exp):]) and len(got) == max_tiles
+
+
+def _grouped_case(counts, n, k, seed, gather):
+    g = torch.Generator().manual_seed(seed)
+    groups, rows = len(counts), sum(counts)
+    src_rows = rows + 3 if gather else rows
+    x = torch.randn(src_rows, k, generator=g).bfloat16()
+    xq, xs = oracle.act_quant(x)
+    w = [oracle.block_quant_weight((torch.randn(n, k, generator=g) * 0.05).bfloat16()) for _ in range(groups)]
+    a_rows = torch.randint(0, src_rows, (rows,), generator=g, dtype=torch.int32) if gather else None
+    return xq, xs, w, a_rows
+
+
+@pytest.mark.parametrize("counts,n,k,gather", [
+    ([5, 0, 300, 256, 1], 384, 512, True),
+    ([129, 64], 576, 256, False),            # ragged n: 576 = 2 tiles + 64, 5 scale rows
+    ([40] * 6, 256, 1152, True),             # odd number of K blocks
+])
+def test_fp8_gemm_grouped_vs_oracle(K, counts, n, k, gather):
+    from dsv3fp8 import ops
+    xq, xs, w, a_rows = _grouped_case(counts, n, k, 11, gather)
+    rows = sum(counts)
+    R, tg, t0, tr = _tables(counts, rows // ops.grouped_tile_rows() + len(counts))
+    b = torch.stack([wi[0].view(torch.uint8) for wi in w]).view(FP8).cuda()
+    b_s = torch.stack([wi[1] for wi in w]).cuda()
+    out32 = torch.ops.dsv3fp8.fp8_gemm_grouped(xq.cuda(), xs.cuda(), a_rows.cuda() if gather else None, b, b_s, rows,
+                                               tg, t0, tr, ops.dtype_code(torch.float32))
+    out16 = torch.ops.dsv3fp8.fp8_gemm_grouped(xq.cuda(), xs.cuda(), a_rows.cuda() if gather else None, b, b_s, rows,
+                                               tg, t0, tr, ops.dtype_code(torch.bfloat16))
+    assert out32.shape == (rows, n) and out16.dtype == torch.bfloat16
+    assert torch.equal(out16.float(), out32.bfloat16().float())          # bf16 output = RNE of the fp32 result
+    row = 0
+    for gi, c in enumerate(counts):
+        if c == 0:
+            continue
+        idx = a_rows[row:row + c].long() if gather else torch.arange(row, row + c)
+        ref = oracle.fp8_gemm_f32(xq[idx], xs[idx], w[gi][0], w[gi][1])
+        err = (out32[row:row + c].cpu() - ref).abs().max().item()
+        assert err <= 1e-2 * ref.pow(2).mean().sqrt().item(), (gi, err)     # tolerance of the fp32 output
+        row += c
+
+
+@pytest.mark.parametrize("fmt", [None, "ue8m0"])
+def test_swiglu_quant(K, fmt):
+    g = torch.Generator().manual_seed(3)
+    rows, inter = 37, 384
+    h = (torch.randn(rows, 2 * inter, generator=g) * 2).bfloat16()
+    h[0, :inter] = 0                                      # an all-zero block: s = 1e-4/448, y = 0
+    h[1, 5] = 60.0                                        # silu saturates to x
+    from dsv3fp8 import _lib
+    y, s = torch.ops.dsv3fp8.swiglu_quant(h.cuda(), 128, _lib.SCALE_FMT_UE8M0 if fmt else _lib.SCALE_FMT_NONE)
+    gref = F.silu(h[:, :inter]) * h[:, inter:]            # bf16 tensor ops, as model.py:633
+    yr, sr = oracle.act_quant(gref, 128, fmt)
+    assert y.shape == (rows, inter) and s.shape == (rows, inter // 128)
+    # exp() of the device and of the CPU may differ in the last place: allow a bf16 ulp of g on a few elements
+    same_scale = (s.cpu() == sr).float().mean().item()
+    same_code = (y.cpu().view(torch.uint8) == yr.view(torch.uint8)).float().mean().item()
+    assert same_scale >= 0.97 and same_code >= 0.995, (same_scale, same_code)
+    deq = y.cpu().float() * s.cpu().repeat_interleave(128, 1)
+    ref = yr.float() * sr.repeat_interleave(128, 1)
+    assert (deq - ref).abs().max().item() <= 0.07 * ref.abs().max().item()
+    # against the same chain on the device (same exp): bit-identical
+    gd = F.silu(h.cuda()[:, :inter]) * h.cuda()[:, inter:]
+    yd, sd = K.act_quant(gd.contiguous(), 128, fmt)
+    assert torch.equal(s, sd) and torch.equal(y.view(torch.uint8), yd.view(torch.uint8))
+
+
+@pytest.mark.parametrize("with_shared", [True, False])
+def test_moe_combine_bit_exact(K, with_shared):
+    g = torch.Generator().manual_seed(4)
+    tokens, topk, dim, experts = 33, 4, 264, 9
+    scores = torch.rand(tokens, experts, generator=g)
+    indices = scores.topk(topk, dim=-1)[1]
+    weights = torch.rand(tokens, topk, generator=g).bfloat16()
+    flat = indices.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    out = torch.randn(tokens * topk, dim, generator=g).bfloat16()       # expert-sorted rows
+    z = torch.randn(tokens, dim, generator=g).bfloat16()
+    # reference: the loop of model.py:684-693 on the CPU
+    y = torch.zeros(tokens, dim, dtype=torch.bfloat16)
+    row = 0
+    for e in range(experts):
+        idx, top = torch.where(indices == e)
+        if idx.numel() == 0:
+            continue
+        y[idx] += out[row:row + idx.numel()] * weights[idx, top, None]
+        row += idx.numel()
+    ref = y + z if with_shared else y
+    slot = indices.argsort(dim=1)
+    pos = torch.empty_like(order)
+    pos[order] = torch.arange(tokens * topk)
+    rows = pos.view(tokens, topk).gather(1, slot).to(torch.int32)
+    got = torch.ops.dsv3fp8.moe_combine(out.cuda(), rows.cuda(), weights.gather(1, slot).contiguous().cuda(),
+                                        z.cuda() if with_shared else None)
+    assert torch.equal(got.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+def test_moe_grouped_matches_expert_loop_and_oracle(K):
+    from dsv3fp8 import model as M
+    old = (M.gemm_impl, torch.get_default_dtype(), M.Linear.dtype)
+    torch.set_default_dtype(torch.bfloat16)
+    M.Linear.dtype = FP8
+    M.gemm_impl = "fp8"
+    try:
+        args = M.ModelArgs(dim=256, inter_dim=512, moe_inter_dim=128, n_routed_experts=8, n_shared_experts=1,
+                           n_activated_experts=2, n_expert_groups=2, n_limited_groups=1, route_scale=2.5)
+        with torch.device("cuda"):
+            moe = M.MoE(args)
+        g = torch.Generator().manual_seed(5)
+        with torch.no_grad():
+            moe.gate.weight.copy_((torch.randn(8, 256, generator=g) * 0.05).bfloat16().cuda())
+        experts = []
+
+        def fill(lin, seed):
+            gg = torch.Generator().manual_seed(seed)
+            w8, s = oracle.block_quant_weight((torch.randn(lin.out_features, lin.in_features, generator=gg) * 0.05).bfloat16())
+            with torch.no_grad():
+                lin.weight.copy_(w8.cuda()); lin.scale.copy_(s.cuda())
+            return w8, s
+        for i, ex in enumerate(moe.experts):
+            w1, s1 = fill(ex.w1, 10 + 3 * i); w2, s2 = fill(ex.w2, 11 + 3 * i); w3, s3 = fill(ex.w3, 12 + 3 * i)
+            experts.append((w1, s1, w2, s2, w3, s3))
+        sh = moe.shared_experts
+        shared = (*fill(sh.w1, 90), *fill(sh.w2, 91), *fill(sh.w3, 92))
+        x = torch.randn(300, 256, generator=g).bfloat16()
+        with torch.inference_mode():
+            M.MoE.grouped = True
+            y_grouped = moe(x.cuda())
+            assert moe._stacked is not None and moe.experts[3].w1.weight.data_ptr() == moe._stacked[0][3].data_ptr()
+            M.MoE.grouped = False
+            y_loop = moe(x.cuda())                      # the reference's loop on the (now stacked) expert weights
+            wts, idx = moe.gate(x.cuda())
+        ref = oracle.moe(x, wts.cpu(), idx.cpu(), experts, shared)
+        rms = ref.float().pow(2).mean().sqrt().item()
+        # same kernels' arithmetic up to the GEMM's summation order: a bf16 ulp here and there
+        assert (y_grouped.float() - y_loop.float()).abs().max().item() <= 3e-2 * rms
+        assert (y_grouped.float().cpu() - ref.float()).abs().max().item() <= 5e-2 * rms + 2 ** -8 * ref.abs().max().item()
+    finally:
+        M.MoE.grouped = True
+        M.gemm_impl, M.Linear.dtype = old[0], old[2]
+        torch.set_default_dtype(old[1])
