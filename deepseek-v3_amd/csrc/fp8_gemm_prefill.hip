@@ -18,6 +18,7 @@
 // 16-byte chunks of one row in a permuted order p = c ^ f(row), which leaves the
 // later ds_read_b128 fragment reads (16 consecutive rows, same chunk) free of
 // bank conflicts.
+#include <type_traits>
 #include "common.hpp"
 
 namespace dsv3 {
@@ -141,14 +142,19 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const int fr = lane & 15, fq = lane >> 4;
     const int fx = swz(fr);                                   // sub-tile bases are multiples of 16 rows
     const int c0 = ((2 * fq) ^ fx) * 16, c1 = ((2 * fq + 1) ^ fx) * 16;
-    const int a_rd = LDS_A + (wm * WM + fr) * 128;            // + j*16*128 + stage*A_STAGE
+    // 16-row sub-tile j of this wavefront: 64 consecutive rows in dense mode; in grouped mode the sub-tiles are
+    // dealt round-robin over the four m-wavefronts, so that a tile with few valid rows (a small expert) leaves
+    // every SIMD the same share of work instead of idling two of them
+    auto sub_row = [&](int j) { return G ? (j * WAVES_M + wm) * 16 : wm * WM + j * 16; };
+    constexpr int A_JSTRIDE = (G ? WAVES_M : 1) * 2048;       // LDS bytes between consecutive sub-tiles of a wavefront
+    const int a_rd = LDS_A + (sub_row(0) + fr) * 128;         // + j*A_JSTRIDE + stage*A_STAGE
     const int b_rd = LDS_B + (wn * WN + fr) * 128;            // + i*16*128 + stage*B_STAGE
 
     // ---- scales: a_s[m, kb] for the lane's row of each m sub-tile; b_s row of this wavefront's n range
     uint32_t as_off[SM];
 #pragma unroll
     for (int j = 0; j < SM; ++j)
-        as_off[j] = a_row(wm * WM + j * 16 + fr) * (uint32_t)KB;
+        as_off[j] = a_row(sub_row(j) + fr) * (uint32_t)KB;
     const int nb_last = (N - 1) / 128;
     const float* bs_src = b_s + (size_t)min((n0 + wn * WN) / 128, nb_last) * KB;
 
@@ -175,113 +181,138 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     // (block kb+2) and the first fragments of block kb+1 are read from the other stage while the last
     // 2 x SM MFMAs of block kb run.  The next block then starts with its operands already in registers.
     constexpr int kSync = SN - 2;
-    float sc[SM], sc_nxt[SM];
-    {
-        const float bs = bs_src[0];
-#pragma unroll
-        for (int j = 0; j < SM; ++j) sc_nxt[j] = a_s[as_off[j]] * bs;
-#pragma unroll
-        for (int j = 0; j < SM; ++j) sc[j] = 0.f;
-    }
-    issue_loads(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
-    __syncthreads();
-    issue_loads(min(1, KB - 1), 1);
-    v4f pend = {0.f, 0.f, 0.f, 0.f};      // raw dot products of (i = SN-1, j = SM-1) of the previous K block
-    v8i nf0, nf1, mf[SM];                 // weight fragments of steps i, i+1 (MFMA A operand); activation fragments (B operand)
-    {
-        const uint8_t* as_base = lds + a_rd;
-        const uint8_t* bs_base = lds + b_rd;
-        nf0 = join(*(const v4i*)(bs_base + c0), *(const v4i*)(bs_base + c1));
-#pragma unroll
-        for (int j = 0; j < SM; ++j)
-            mf[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
-        nf1 = join(*(const v4i*)(bs_base + 2048 + c0), *(const v4i*)(bs_base + 2048 + c1));
-    }
+    // sub-tiles of this wavefront that hold at least one valid row (all four in dense mode; the clamped rows of an
+    // edge tile are computed and dropped there).  The pipeline below is instantiated per count, so a wavefront
+    // issues MFMAs and FMAs only for live sub-tiles; one without any only feeds LDS and keeps the barriers.
+    const int ja_live = G ? max(0, min(SM, ((rows_here + 15) / 16 - wm + WAVES_M - 1) / WAVES_M)) : SM;
 
 #define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-    for (int kb = 0; kb < KB; ++kb) {
-        const int stage = kb & 1;
-        const uint8_t* bs_base = lds + b_rd + stage * B_STAGE;
-        const uint8_t* as_next = lds + a_rd + (stage ^ 1) * A_STAGE;
-        const uint8_t* bs_next = lds + b_rd + (stage ^ 1) * B_STAGE;
-
-        // branch-free: past the end the loop re-fetches the last block into a stage nobody reads again
-        const int kn = min(kb + 1, KB - 1), kn2 = min(kb + 2, KB - 1);
-        float as_nxt[SM], bs_nxt = 0.f;
-
-        // fold the tile left over from the previous K block with that block's scale, then switch scales
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[SN - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[SN - 1][SM - 1][e]);
-#pragma unroll
-        for (int j = 0; j < SM; ++j) sc[j] = sc_nxt[j];
-        __builtin_amdgcn_sched_barrier(0);
-
-#pragma unroll
-        for (int i = 0; i < SN; ++i) {
-            if (i == kSync) {
-                // every LDS read of this stage has returned and this wavefront's share of the other stage
-                // (and the next block's scales) has landed
-#pragma unroll
-                for (int j = 0; j < SM; ++j) sc_nxt[j] = as_nxt[j] * bs_nxt;
-                __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
+    auto pipeline = [&](auto ja_tag) {
+        constexpr int JA = decltype(ja_tag)::value;
+        issue_loads(0, 0);
+        if constexpr (JA == 0) {
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+            __syncthreads();
+            issue_loads(min(1, KB - 1), 1);
+            for (int kb = 0; kb < KB; ++kb) {
+                __builtin_amdgcn_s_waitcnt(0x0f70);
                 __syncthreads();
-                __builtin_amdgcn_sched_barrier(0);
+                issue_loads(min(kb + 2, KB - 1), kb & 1);
             }
-            // weight rows are streamed two steps ahead; the last two steps fetch steps 0 and 1 of the next block
-            v8i nf2;
-            if (i < kSync)
-                nf2 = join(*(const v4i*)(bs_base + (i + 2) * 2048 + c0), *(const v4i*)(bs_base + (i + 2) * 2048 + c1));
-            else
-                nf2 = join(*(const v4i*)(bs_next + (i - kSync) * 2048 + c0), *(const v4i*)(bs_next + (i - kSync) * 2048 + c1));
-            const v4f z = {0.f, 0.f, 0.f, 0.f};
-            v4f p[SM];
-            p[0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[0], z, 0, 0, 0, 0, 0, 0);
-            if (i == SN - 1) mf[0] = join(*(const v4i*)(as_next + c0), *(const v4i*)(as_next + c1));
-            if (i > 0) {
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+        } else {
+        float sc[JA], sc_nxt[JA];
+        {
+            const float bs = bs_src[0];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[i - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[i - 1][SM - 1][e]);
-            }
+            for (int j = 0; j < JA; ++j) sc_nxt[j] = a_s[as_off[j]] * bs;
 #pragma unroll
-            for (int j = 1; j < SM; ++j) {
-                p[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[j], z, 0, 0, 0, 0, 0, 0);
-                if (i == SN - 1) mf[j] = join(*(const v4i*)(as_next + j * 2048 + c0), *(const v4i*)(as_next + j * 2048 + c1));
+            for (int j = 0; j < JA; ++j) sc[j] = 0.f;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
+        __syncthreads();
+        issue_loads(min(1, KB - 1), 1);
+        v4f pend = {0.f, 0.f, 0.f, 0.f};      // raw dot products of (i = SN-1, j = JA-1) of the previous K block
+        v8i nf0, nf1, mf[JA];                 // weight fragments of steps i, i+1 (MFMA A operand); activation fragments (B operand)
+        {
+            const uint8_t* as_base = lds + a_rd;
+            const uint8_t* bs_base = lds + b_rd;
+            nf0 = join(*(const v4i*)(bs_base + c0), *(const v4i*)(bs_base + c1));
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(p[j - 1][e], sc[j - 1], acc[i][j - 1][e]);
-            }
-            if (i >= kSync) {
-                // refill the stage this block has finished reading with block kb+2
+            for (int j = 0; j < JA; ++j)
+                mf[j] = join(*(const v4i*)(as_base + j * A_JSTRIDE + c0), *(const v4i*)(as_base + j * A_JSTRIDE + c1));
+            nf1 = join(*(const v4i*)(bs_base + 2048 + c0), *(const v4i*)(bs_base + 2048 + c1));
+        }
+
+        for (int kb = 0; kb < KB; ++kb) {
+            const int stage = kb & 1;
+            const uint8_t* bs_base = lds + b_rd + stage * B_STAGE;
+            const uint8_t* as_next = lds + a_rd + (stage ^ 1) * A_STAGE;
+            const uint8_t* bs_next = lds + b_rd + (stage ^ 1) * B_STAGE;
+
+            // branch-free: past the end the loop re-fetches the last block into a stage nobody reads again
+            const int kn = min(kb + 1, KB - 1), kn2 = min(kb + 2, KB - 1);
+            float as_nxt[JA], bs_nxt = 0.f;
+
+            // fold the tile left over from the previous K block with that block's scale, then switch scales
 #pragma unroll
-                for (int t = 0; t < 4; ++t) issue_load((i - kSync) * 4 + t, kn2, stage);
-            }
-            if (i < SM) as_nxt[i] = a_s[as_off[i] + (uint32_t)kn];
-            if (i == SM) bs_nxt = bs_src[kn + vzero];     // through the vector path on purpose, see vzero
-            pend = p[SM - 1];
-            nf0 = nf1;
-            nf1 = nf2;
-            DSV3_SGB(0x100, 2);
-            DSV3_SGB(0x008, 1);
-            if (i == SN - 1) DSV3_SGB(0x100, 2);
-            if (i > 0) DSV3_SGB(0x002, 4);
+            for (int e = 0; e < 4; ++e) acc[SN - 1][JA - 1][e] = __builtin_fmaf(pend[e], sc[JA - 1], acc[SN - 1][JA - 1][e]);
 #pragma unroll
-            for (int j = 1; j < SM; ++j) {
+            for (int j = 0; j < JA; ++j) sc[j] = sc_nxt[j];
+            __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+            for (int i = 0; i < SN; ++i) {
+                if (i == kSync) {
+                    // every LDS read of this stage has returned and this wavefront's share of the other stage
+                    // (and the next block's scales) has landed
+#pragma unroll
+                    for (int j = 0; j < JA; ++j) sc_nxt[j] = as_nxt[j] * bs_nxt;
+                    __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
+                    __syncthreads();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // weight rows are streamed two steps ahead; the last two steps fetch steps 0 and 1 of the next block
+                v8i nf2;
+                if (i < kSync)
+                    nf2 = join(*(const v4i*)(bs_base + (i + 2) * 2048 + c0), *(const v4i*)(bs_base + (i + 2) * 2048 + c1));
+                else
+                    nf2 = join(*(const v4i*)(bs_next + (i - kSync) * 2048 + c0), *(const v4i*)(bs_next + (i - kSync) * 2048 + c1));
+                const v4f z = {0.f, 0.f, 0.f, 0.f};
+                v4f p[JA];
+                p[0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[0], z, 0, 0, 0, 0, 0, 0);
+                if (i == SN - 1) mf[0] = join(*(const v4i*)(as_next + c0), *(const v4i*)(as_next + c1));
+                if (i > 0) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i - 1][JA - 1][e] = __builtin_fmaf(pend[e], sc[JA - 1], acc[i - 1][JA - 1][e]);
+                }
+#pragma unroll
+                for (int j = 1; j < JA; ++j) {
+                    p[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[j], z, 0, 0, 0, 0, 0, 0);
+                    if (i == SN - 1) mf[j] = join(*(const v4i*)(as_next + j * A_JSTRIDE + c0), *(const v4i*)(as_next + j * A_JSTRIDE + c1));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(p[j - 1][e], sc[j - 1], acc[i][j - 1][e]);
+                }
+                if (i >= kSync) {
+                    // refill the stage this block has finished reading with block kb+2
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) issue_load((i - kSync) * 4 + t, kn2, stage);
+                }
+                if (i < JA) as_nxt[i] = a_s[as_off[i] + (uint32_t)kn];
+                if (i == SM) bs_nxt = bs_src[kn + vzero];     // through the vector path on purpose, see vzero
+                pend = p[JA - 1];
+                nf0 = nf1;
+                nf1 = nf2;
+                DSV3_SGB(0x100, 2);
                 DSV3_SGB(0x008, 1);
                 if (i == SN - 1) DSV3_SGB(0x100, 2);
-                DSV3_SGB(0x002, 4);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-#undef DSV3_SGB
+                if (i > 0) DSV3_SGB(0x002, 4);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[SN - 1][SM - 1][e] = __builtin_fmaf(pend[e], sc[SM - 1], acc[SN - 1][SM - 1][e]);
-    __builtin_amdgcn_s_waitcnt(0x0f70);             // the clamped refills of the last two blocks are still in flight
+                for (int j = 1; j < JA; ++j) {
+                    DSV3_SGB(0x008, 1);
+                    if (i == SN - 1) DSV3_SGB(0x100, 2);
+                    DSV3_SGB(0x002, 4);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[SN - 1][JA - 1][e] = __builtin_fmaf(pend[e], sc[JA - 1], acc[SN - 1][JA - 1][e]);
+        __builtin_amdgcn_s_waitcnt(0x0f70);             // the clamped refills of the last two blocks are still in flight
+        }
+    };
+    if (!G || ja_live == 4) pipeline(std::integral_constant<int, 4>{});
+    else if (ja_live == 3)  pipeline(std::integral_constant<int, 3>{});
+    else if (ja_live == 2)  pipeline(std::integral_constant<int, 2>{});
+    else if (ja_live == 1)  pipeline(std::integral_constant<int, 1>{});
+    else { pipeline(std::integral_constant<int, 0>{}); return; }
+#undef DSV3_SGB
 
     // ---- epilogue: lane holds c[m][n .. n+3] for every (i, j)
     const bool vec_ok = (N % 4) == 0;
 #pragma unroll
     for (int j = 0; j < SM; ++j) {
-        const int r = wm * WM + j * 16 + fr;
+        const int r = sub_row(j) + fr;
         if (r >= rows_here) continue;
         const int m = m0 + r;
 #pragma unroll
