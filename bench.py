@@ -139,10 +139,11 @@ def run_extras(K, W):
 def run_moe(K, W, tokens: int = 4096):
     """BASELINE config 5: one MoE layer (256 routed + 1 shared SwiGLU experts, 7168 -> 2048 -> 7168, fp8
     block-scaled weights generated on the device), T tokens, sigmoid gate with bias over random logits'
-    weights, 8 groups / top-4 groups / top-8 experts, route_scale 2.5, executed as the reference does:
-    one pass over the experts' token lists (model.py:679-693)."""
+    weights, 8 groups / top-4 groups / top-8 experts, route_scale 2.5.  Timed twice: the grouped path
+    (device-side token lists, two grouped GEMMs, fused SwiGLU + re-quantisation, ordered combine) and the
+    reference's host-driven pass over the experts' token lists (model.py:679-693) on the same kernels."""
     from dsv3fp8 import model as Mdl
-    old = Mdl.gemm_impl, Mdl.Linear.dtype
+    old = Mdl.gemm_impl, Mdl.Linear.dtype, Mdl.MoE.grouped
     Mdl.gemm_impl, Mdl.Linear.dtype = "fp8", torch.float8_e4m3fn
     try:
         args = Mdl.ModelArgs()
@@ -157,18 +158,24 @@ def run_moe(K, W, tokens: int = 4096):
                 for lin, (w8, sc) in ((ex.w1, protos[0]), (ex.w3, protos[0]), (ex.w2, protos[1])):
                     lin.weight.copy_(w8)          # distinct storage per expert: 11.3 GB of weights are streamed
                     lin.scale.copy_(sc)
+        moe.stack_experts()
         x = W.activations(tokens, args.dim, 6, "cuda")
-        with torch.inference_mode():
-            ms = time_loop(lambda: moe(x), 3, 1)
         flops = 2.0 * 3 * args.dim * args.moe_inter_dim * (tokens * args.n_activated_experts + tokens)
         wbytes = 257 * 3 * args.dim * args.moe_inter_dim
-        return {"ms": round(ms, 3), "TFLOPs": round(flops / ms / 1e9, 1),
-                "weight_stream_GBps": round(wbytes / ms / 1e6, 1),
-                "mfma_frac": round(flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 4),
-                "hbm_frac": round(wbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
-                "note": "expert loop as in the reference (host-driven, 3 act_quant + 3 fp8_gemm per expert)"}
+        res = {}
+        with torch.inference_mode():
+            for key, grouped, steps in (("grouped", True, 10), ("expert_loop", False, 2)):
+                Mdl.MoE.grouped = grouped
+                ms = time_loop(lambda: moe(x), steps, 2 if grouped else 1)
+                res[key] = {"ms": round(ms, 3), "TFLOPs": round(flops / ms / 1e9, 1),
+                            "weight_stream_GBps": round(wbytes / ms / 1e6, 1),
+                            "mfma_frac": round(flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 4),
+                            "hbm_frac": round(wbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        res["note"] = ("grouped: MoE.forward as shipped (no host sync); expert_loop: the reference's per-expert "
+                       "loop, 3 act_quant + 3 fp8_gemm per expert")
+        return res
     finally:
-        Mdl.gemm_impl, Mdl.Linear.dtype = old
+        Mdl.gemm_impl, Mdl.Linear.dtype, Mdl.MoE.grouped = old
 
 
 def cpu_baseline(W, rows: int = 1024):
