@@ -31,7 +31,9 @@ constexpr int SM = WM / 16, SN = WN / 16;                // 4 x 8 MFMA tiles
 constexpr int THREADS = WAVES_M * WAVES_N * kWave;       // 512
 constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128;    // bytes per K block
 constexpr int LDS_A = 0, LDS_B = 2 * A_STAGE;            // [A s0 | A s1 | B s0 | B s1]
-constexpr int LDS_BYTES = 2 * (A_STAGE + B_STAGE);       // 128 KiB
+constexpr int SC_STAGE = 8 * 256;                        // scales of one K block: one 64-float slot per wavefront
+constexpr int LDS_SC = 2 * (A_STAGE + B_STAGE);
+constexpr int LDS_BYTES = LDS_SC + 2 * SC_STAGE;         // 128 KiB of tiles + 2.5 KiB of scales
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -150,25 +152,28 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const int a_rd = LDS_A + (sub_row(0) + fr) * 128;         // + j*A_JSTRIDE + stage*A_STAGE
     const int b_rd = LDS_B + (wn * WN + fr) * 128;            // + i*16*128 + stage*B_STAGE
 
-    // ---- scales: a_s[m, kb] for the lane's row of each m sub-tile; b_s row of this wavefront's n range
-    uint32_t as_off[SM];
-#pragma unroll
-    for (int j = 0; j < SM; ++j)
-        as_off[j] = a_row(sub_row(j) + fr) * (uint32_t)KB;
+    // ---- scales.  They take the same route as the tiles: global -> LDS (4 bytes per lane), double buffered,
+    // requested one block ahead, read back after the block's barrier.  An ordinary global load inside the K
+    // loop is not an option: issued behind the wavefront's outstanding direct-to-LDS loads it holds the
+    // wavefront until those have returned -- a memory round trip per K block, measured at 30% of the kernel.
+    // Wavefronts 0-3 fetch a_s[row, kb] of 64 tile rows each, wavefront 4 the b_s rows of the two column halves
+    // (wavefronts 5-7 repeat that into slots nobody reads, which keeps the loop free of branches).
     const int nb_last = (N - 1) / 128;
-    const float* bs_src = b_s + (size_t)min((n0 + wn * WN) / 128, nb_last) * KB;
+    const float* sc_base = wave < 4 ? a_s : b_s;
+    const uint32_t sc_off = wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KB
+                                     : (uint32_t)min(n0 / 128 + lane, nb_last) * (uint32_t)KB;
+    auto issue_scales = [&](int kb, int stage) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(sc_base + sc_off + (uint32_t)kb),
+                                         (lptr_t)(lds + LDS_SC + stage * SC_STAGE + wave * 256), 4, 0, 0);
+    };
+    auto lds_as = [&](int j, int stage) { return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (sub_row(j) + fr) * 4); };
+    auto lds_bs = [&](int stage) { return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (BM + wn) * 4); };
 
     v4f acc[SN][SM];
 #pragma unroll
     for (int i = 0; i < SN; ++i)
 #pragma unroll
         for (int j = 0; j < SM; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
-
-    // A zero the compiler cannot see through: indexing the (wavefront-uniform) b_s row with it keeps that load
-    // on the vector memory path.  A scalar load would share the LGKM counter with the LDS reads and, returning
-    // out of order, force every LDS wait in the loop down to lgkmcnt(0).
-    int vzero;
-    asm volatile("v_mov_b32 %0, 0" : "=v"(vzero));
 
     // Software pipeline.  Per 16-column step i of a K block the wavefront issues
     //     ds_read x2 (weights of step i+2) | MFMA j=0 | FMA of the pending tile | MFMA 1 | FMA tile 0 | MFMA 2 |
@@ -190,28 +195,32 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     auto pipeline = [&](auto ja_tag) {
         constexpr int JA = decltype(ja_tag)::value;
         issue_loads(0, 0);
+        issue_scales(0, 0);
         if constexpr (JA == 0) {
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();
             issue_loads(min(1, KB - 1), 1);
+            issue_scales(min(1, KB - 1), 1);
             for (int kb = 0; kb < KB; ++kb) {
                 __builtin_amdgcn_s_waitcnt(0x0f70);
                 __syncthreads();
                 issue_loads(min(kb + 2, KB - 1), kb & 1);
+                issue_scales(min(kb + 2, KB - 1), kb & 1);
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);
         } else {
         float sc[JA], sc_nxt[JA];
-        {
-            const float bs = bs_src[0];
-#pragma unroll
-            for (int j = 0; j < JA; ++j) sc_nxt[j] = a_s[as_off[j]] * bs;
-#pragma unroll
-            for (int j = 0; j < JA; ++j) sc[j] = 0.f;
-        }
         __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
         __syncthreads();
         issue_loads(min(1, KB - 1), 1);
+        issue_scales(min(1, KB - 1), 1);
+        {
+            const float bs = lds_bs(0);
+#pragma unroll
+            for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, 0) * bs;
+#pragma unroll
+            for (int j = 0; j < JA; ++j) sc[j] = 0.f;
+        }
         v4f pend = {0.f, 0.f, 0.f, 0.f};      // raw dot products of (i = SN-1, j = JA-1) of the previous K block
         v8i nf0, nf1, mf[JA];                 // weight fragments of steps i, i+1 (MFMA A operand); activation fragments (B operand)
         {
@@ -231,8 +240,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
             const uint8_t* bs_next = lds + b_rd + (stage ^ 1) * B_STAGE;
 
             // branch-free: past the end the loop re-fetches the last block into a stage nobody reads again
-            const int kn = min(kb + 1, KB - 1), kn2 = min(kb + 2, KB - 1);
-            float as_nxt[JA], bs_nxt = 0.f;
+            const int kn2 = min(kb + 2, KB - 1);
 
             // fold the tile left over from the previous K block with that block's scale, then switch scales
 #pragma unroll
@@ -245,11 +253,15 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
             for (int i = 0; i < SN; ++i) {
                 if (i == kSync) {
                     // every LDS read of this stage has returned and this wavefront's share of the other stage
-                    // (and the next block's scales) has landed
-#pragma unroll
-                    for (int j = 0; j < JA; ++j) sc_nxt[j] = as_nxt[j] * bs_nxt;
+                    // (tiles and scales of block kb+1) has landed
                     __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
                     __syncthreads();
+                    {
+                        const float bs = lds_bs(stage ^ 1);
+#pragma unroll
+                        for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, stage ^ 1) * bs;
+                    }
+                    issue_scales(kn2, stage);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // weight rows are streamed two steps ahead; the last two steps fetch steps 0 and 1 of the next block
@@ -278,8 +290,6 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 #pragma unroll
                     for (int t = 0; t < 4; ++t) issue_load((i - kSync) * 4 + t, kn2, stage);
                 }
-                if (i < JA) as_nxt[i] = a_s[as_off[i] + (uint32_t)kn];
-                if (i == SM) bs_nxt = bs_src[kn + vzero];     // through the vector path on purpose, see vzero
                 pend = p[JA - 1];
                 nf0 = nf1;
                 nf1 = nf2;
