@@ -199,12 +199,16 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         if constexpr (JA == 0) {
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();
-            issue_loads(min(1, KB - 1), 1);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) issue_load(t, min(1, KB - 1), 1);
             issue_scales(min(1, KB - 1), 1);
             for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+                for (int t = 4; t < 8; ++t) issue_load(t, min(kb + 1, KB - 1), (kb & 1) ^ 1);
                 __builtin_amdgcn_s_waitcnt(0x0f70);
                 __syncthreads();
-                issue_loads(min(kb + 2, KB - 1), kb & 1);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) issue_load(t, min(kb + 2, KB - 1), kb & 1);
                 issue_scales(min(kb + 2, KB - 1), kb & 1);
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -212,7 +216,8 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         float sc[JA], sc_nxt[JA];
         __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
         __syncthreads();
-        issue_loads(min(1, KB - 1), 1);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) issue_load(t, min(1, KB - 1), 1);
         issue_scales(min(1, KB - 1), 1);
         {
             const float bs = lds_bs(0);
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
             const uint8_t* bs_next = lds + b_rd + (stage ^ 1) * B_STAGE;
 
             // branch-free: past the end the loop re-fetches the last block into a stage nobody reads again
-            const int kn2 = min(kb + 2, KB - 1);
+            const int kn1 = min(kb + 1, KB - 1), kn2 = min(kb + 2, KB - 1);
 
             // fold the tile left over from the previous K block with that block's scale, then switch scales
 #pragma unroll
@@ -285,10 +290,16 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 #pragma unroll
                     for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(p[j - 1][e], sc[j - 1], acc[i][j - 1][e]);
                 }
+                // Refill of the stage that the barrier freed, spread over four steps so that the address unit sees
+                // two loads per wavefront at a time and not a burst of eight from every wavefront at once: the
+                // activation half of block kb+2 now, the weight half of block kb+1 in the first two steps.
                 if (i >= kSync) {
-                    // refill the stage this block has finished reading with block kb+2
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) issue_load((i - kSync) * 4 + t, kn2, stage);
+                    issue_load((i - kSync) * 2, kn2, stage);
+                    issue_load((i - kSync) * 2 + 1, kn2, stage);
+                }
+                if (i < 2) {
+                    issue_load(4 + i * 2, kn1, stage ^ 1);
+                    issue_load(5 + i * 2, kn1, stage ^ 1);
                 }
                 pend = p[JA - 1];
                 nf0 = nf1;
