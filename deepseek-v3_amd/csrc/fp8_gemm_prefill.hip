@@ -24,16 +24,26 @@
 namespace dsv3 {
 namespace prefill {
 
-constexpr int BM = 256, BN = 256;
+constexpr int BN = 256;
 constexpr int WAVES_M = 4, WAVES_N = 2;
-constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;      // 64 x 128 per wavefront
-constexpr int SM = WM / 16, SN = WN / 16;                // 4 x 8 MFMA tiles
+constexpr int WN = BN / WAVES_N, SN = WN / 16;           // 128 columns = 8 MFMA tiles per wavefront
 constexpr int THREADS = WAVES_M * WAVES_N * kWave;       // 512
-constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128;    // bytes per K block
-constexpr int LDS_A = 0, LDS_B = 2 * A_STAGE;            // [A s0 | A s1 | B s0 | B s1]
 constexpr int SC_STAGE = 8 * 256;                        // scales of one K block: one 64-float slot per wavefront
-constexpr int LDS_SC = 2 * (A_STAGE + B_STAGE);
-constexpr int LDS_BYTES = LDS_SC + 2 * SC_STAGE;         // 128 KiB of tiles + 2.5 KiB of scales
+
+// Tile height TM and number of LDS stages S.  <256, 2>: the large-M shape, 64 x 128 per wavefront, 2 x 64 KiB of
+// tiles.  <128, 3>: 32 x 128 per wavefront, 3 x 48 KiB -- the loads of a K block then have two blocks of time to
+// land, which is what matters when a tile has little arithmetic per block (the ~128-row groups of an MoE layer:
+// a global -> LDS round trip under load, ~1.4 us, is longer than such a block's MFMA time).
+template <int TM, int S> struct Cfg {
+    static constexpr int WM = TM / WAVES_M, SM = WM / 16;
+    static constexpr int A_LOADS = TM / 64, B_LOADS = BN / 64;        // 1 KiB wavefront-loads per wavefront and stage
+    static constexpr int LOADS = A_LOADS + B_LOADS + 1;               // ... plus the scale load
+    static constexpr int A_STAGE = TM * 128, B_STAGE = BN * 128;      // bytes per K block
+    static constexpr int LDS_A = 0, LDS_B = S * A_STAGE;              // [A stages | B stages | scale stages]
+    static constexpr int LDS_SC = S * (A_STAGE + B_STAGE);
+    static constexpr int LDS_BYTES = LDS_SC + S * SC_STAGE;
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS of a gfx950 compute unit");
+};
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -42,6 +52,12 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // measured on gfx950 (SQ_LDS_BANK_CONFLICT == 0): 16 consecutive lanes reading the same logical chunk of
 // 16 consecutive 128-byte rows do not collide when the chunk index is xor-ed with (row & 7) ^ (row >> 3 & 1)
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// Workgroup barrier without the memory fence of __syncthreads(): that fence waits for every outstanding vector
+// memory operation of the wavefront, i.e. also for the direct-to-LDS loads of later K blocks that are meant to stay
+// in flight across the barrier.  What a barrier has to order here is spelled out at each use: the wavefront's own
+// LDS reads (lgkmcnt) and exactly those of its loads whose data the other wavefronts are about to read (vmcnt(n)).
+__device__ __forceinline__ void wg_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
     v8i r = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
@@ -56,18 +72,21 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
 struct GroupTable {
     const int* tile_group;   // [tiles_m]
     const int* tile_row0;    // [tiles_m] first row of the tile in c (and in a_rows)
-    const int* tile_rows;    // [tiles_m] 1 .. BM
+    const int* tile_rows;    // [tiles_m] 1 .. TM
     const int* a_rows;       // [rows of c] or nullptr
     int64_t b_stride;        // bytes between consecutive groups' weights
     int64_t bs_stride;       // floats between consecutive groups' weight scales
 };
 
-template <int CD, bool G>
+template <int CD, bool G, int TM, int S>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
         int M, int N, int K, int tiles_m, int tiles_n, GroupTable g) {
+    using C = Cfg<TM, S>;
+    constexpr int WM = C::WM, SM = C::SM, A_LOADS = C::A_LOADS, B_LOADS = C::B_LOADS;
+    constexpr int A_STAGE = C::A_STAGE, B_STAGE = C::B_STAGE, LDS_A = C::LDS_A, LDS_B = C::LDS_B, LDS_SC = C::LDS_SC;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     // ---- workgroup -> tile: contiguous run of tiles per XCD; dense mode walks bands of GROUP_M tile rows,
@@ -95,8 +114,8 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const int in_band = pid - band * GROUP_M * tiles_n;
         const int tm = band * GROUP_M + in_band % band_rows;
         const int tn = in_band / band_rows;
-        m0 = tm * BM; n0 = tn * BN;
-        rows_here = min(BM, M - m0);
+        m0 = tm * TM; n0 = tn * BN;
+        rows_here = min(TM, M - m0);
     }
     // row of a behind row r of the tile; rows past the tile's end repeat its last row (their results are dropped)
     auto a_row = [&](int r) -> uint32_t {
@@ -109,34 +128,26 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const int wm = wave & (WAVES_M - 1), wn = wave / WAVES_M;
     const int KB = K / 128;
 
-    // ---- global -> LDS copy plan: a stage is 512 rows (256 of A, then 256 of B) = 64 KiB =
-    // 64 wavefront-loads of 1 KiB; wavefront w issues loads i*8 + w, i = 0..7 (i < 4: A, else B).
-    // Load q covers rows q*8 .. q*8+7; lane l -> row q*8 + l/8, LDS chunk l%8, global chunk (l%8)^f(row).
-    uint32_t src_off[8];
+    // ---- global -> LDS copy plan: a stage is TM rows of A, then 256 of B, in 1 KiB wavefront-loads of 8 rows;
+    // wavefront w issues A loads t*8 + w (t < A_LOADS) and B loads t*8 + w (t < B_LOADS).
+    // Lane l of a load -> row 8q + l/8, LDS chunk l%8, global chunk (l%8)^f(row).
+    uint32_t src_off[A_LOADS + B_LOADS];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int q = i * 8 + wave;
-        const int row = (q & 31) * 8 + (lane >> 3);              // row inside A or B
+    for (int t = 0; t < A_LOADS + B_LOADS; ++t) {
+        const int q = (t < A_LOADS ? t : t - A_LOADS) * 8 + wave;
+        const int row = q * 8 + (lane >> 3);                     // row inside A or B
         const int ch = (lane & 7) ^ swz(row);
-        if (i < 4) src_off[i] = a_row(row) * (uint32_t)K + ch * 16;
-        else       src_off[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + ch * 16;
+        if (t < A_LOADS) src_off[t] = a_row(row) * (uint32_t)K + ch * 16;
+        else             src_off[t] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + ch * 16;
     }
-    auto issue_load = [&](int i, int kb, int stage) {
-        const int q = i * 8 + wave;
-        const uint8_t* base = (i < 4) ? a : b;
-        const int dst = (i < 4 ? LDS_A + stage * A_STAGE : LDS_B + stage * B_STAGE) + (q & 31) * 1024;
-        __builtin_amdgcn_global_load_lds((gptr_t)(base + src_off[i] + (uint32_t)kb * 128u),
+    // load t of K block kb into LDS stage `stage`: t < A_LOADS is the activation part, the rest the weight part
+    auto issue_load = [&](int t, int kb, int stage) {
+        const bool is_a = t < A_LOADS;
+        const int q = (is_a ? t : t - A_LOADS) * 8 + wave;
+        const uint8_t* base = is_a ? a : b;
+        const int dst = (is_a ? LDS_A + stage * A_STAGE : LDS_B + stage * B_STAGE) + q * 1024;
+        __builtin_amdgcn_global_load_lds((gptr_t)(base + src_off[t] + (uint32_t)kb * 128u),
                                          (lptr_t)(lds + dst), 16, 0, 0);
-    };
-    auto issue_loads = [&](int kb, int stage) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int q = i * 8 + wave;
-            const uint8_t* base = (i < 4) ? a : b;
-            const int dst = (i < 4 ? LDS_A + stage * A_STAGE : LDS_B + stage * B_STAGE) + (q & 31) * 1024;
-            __builtin_amdgcn_global_load_lds((gptr_t)(base + src_off[i] + (uint32_t)kb * 128u),
-                                             (lptr_t)(lds + dst), 16, 0, 0);
-        }
     };
 
     // ---- fragment read addresses.  A lane reads row (lane&15) of a 16-row sub-tile and the 32 bytes
@@ -144,7 +155,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const int fr = lane & 15, fq = lane >> 4;
     const int fx = swz(fr);                                   // sub-tile bases are multiples of 16 rows
     const int c0 = ((2 * fq) ^ fx) * 16, c1 = ((2 * fq + 1) ^ fx) * 16;
-    // 16-row sub-tile j of this wavefront: 64 consecutive rows in dense mode; in grouped mode the sub-tiles are
+    // 16-row sub-tile j of this wavefront: consecutive rows in dense mode; in grouped mode the sub-tiles are
     // dealt round-robin over the four m-wavefronts, so that a tile with few valid rows (a small expert) leaves
     // every SIMD the same share of work instead of idling two of them
     auto sub_row = [&](int j) { return G ? (j * WAVES_M + wm) * 16 : wm * WM + j * 16; };
@@ -152,12 +163,13 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const int a_rd = LDS_A + (sub_row(0) + fr) * 128;         // + j*A_JSTRIDE + stage*A_STAGE
     const int b_rd = LDS_B + (wn * WN + fr) * 128;            // + i*16*128 + stage*B_STAGE
 
-    // ---- scales.  They take the same route as the tiles: global -> LDS (4 bytes per lane), double buffered,
-    // requested one block ahead, read back after the block's barrier.  An ordinary global load inside the K
+    // ---- scales.  They take the same route as the tiles: global -> LDS (4 bytes per lane), one slot per stage,
+    // requested with the tiles, read back after the block's barrier.  An ordinary global load inside the K
     // loop is not an option: issued behind the wavefront's outstanding direct-to-LDS loads it holds the
     // wavefront until those have returned -- a memory round trip per K block, measured at 30% of the kernel.
-    // Wavefronts 0-3 fetch a_s[row, kb] of 64 tile rows each, wavefront 4 the b_s rows of the two column halves
-    // (wavefronts 5-7 repeat that into slots nobody reads, which keeps the loop free of branches).
+    // Wavefronts 0-3 fetch a_s[row, kb] of 64 tile rows each (rows past the tile repeat its last row), wavefront 4
+    // the b_s rows of the two column halves (wavefronts 5-7 repeat that into slots nobody reads, which keeps the
+    // loop free of branches).
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
     const uint32_t sc_off = wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KB
@@ -167,7 +179,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
                                          (lptr_t)(lds + LDS_SC + stage * SC_STAGE + wave * 256), 4, 0, 0);
     };
     auto lds_as = [&](int j, int stage) { return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (sub_row(j) + fr) * 4); };
-    auto lds_bs = [&](int stage) { return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (BM + wn) * 4); };
+    auto lds_bs = [&](int stage) { return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (256 + wn) * 4); };
 
     v4f acc[SN][SM];
 #pragma unroll
@@ -182,43 +194,56 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     // vector pipe.
     //
     // The workgroup barrier of a K block sits before step kSync = SN-2, not at the block's end: by then every
-    // fragment the block still needs is in registers, so after the barrier the idle LDS stage can be refilled
-    // (block kb+2) and the first fragments of block kb+1 are read from the other stage while the last
+    // fragment the block still needs is in registers, so after the barrier the block's LDS stage can be refilled
+    // (block kb+S) and the first fragments of block kb+1 are read from the next stage while the last
     // 2 x SM MFMAs of block kb run.  The next block then starts with its operands already in registers.
+    //
+    // Loads are issued in program order and retire in order.  Per K block a wavefront issues, after barrier kb:
+    // the activation part and the scales of block kb+S (steps kSync, kSync+1), then the weight part of block kb+S
+    // (steps 0, 1 of block kb+1) -- spread out, because a burst of every wavefront's loads right after the barrier
+    // stalls instruction issue.  At barrier kb the data of block kb+1 must be there; everything issued later
+    // belongs to blocks kb+2 .. kb+S-1, so the wait is vmcnt((S-2) * loads per block).
     constexpr int kSync = SN - 2;
-    // sub-tiles of this wavefront that hold at least one valid row (all four in dense mode; the clamped rows of an
-    // edge tile are computed and dropped there).  The pipeline below is instantiated per count, so a wavefront
+    constexpr int kWaitSync = 0x0f70 | ((S - 2) * C::LOADS);
+    static_assert((S - 2) * C::LOADS < 16, "vmcnt immediate");
+    auto next_stage = [](int st) { return st + 1 == S ? 0 : st + 1; };
+    // sub-tiles of this wavefront that hold at least one valid row (all of them in dense mode; the clamped rows of
+    // an edge tile are computed and dropped there).  The pipeline below is instantiated per count, so a wavefront
     // issues MFMAs and FMAs only for live sub-tiles; one without any only feeds LDS and keeps the barriers.
     const int ja_live = G ? max(0, min(SM, ((rows_here + 15) / 16 - wm + WAVES_M - 1) / WAVES_M)) : SM;
 
 #define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
     auto pipeline = [&](auto ja_tag) {
         constexpr int JA = decltype(ja_tag)::value;
-        issue_loads(0, 0);
+        // prologue: block 0 completely, wait, barrier; then the blocks the steady state expects to be in flight:
+        // 1 .. S-2 completely and the activation part + scales of block S-1
+#pragma unroll
+        for (int t = 0; t < A_LOADS + B_LOADS; ++t) issue_load(t, 0, 0);
         issue_scales(0, 0);
+        __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
+        wg_barrier();
+#pragma unroll
+        for (int blk = 1; blk < S; ++blk) {
+#pragma unroll
+            for (int t = 0; t < (blk < S - 1 ? A_LOADS + B_LOADS : A_LOADS); ++t) issue_load(t, min(blk, KB - 1), blk);
+            issue_scales(min(blk, KB - 1), blk);
+        }
         if constexpr (JA == 0) {
-            __builtin_amdgcn_s_waitcnt(0x0f70);
-            __syncthreads();
-#pragma unroll
-            for (int t = 0; t < 4; ++t) issue_load(t, min(1, KB - 1), 1);
-            issue_scales(min(1, KB - 1), 1);
+            int st = 0;
             for (int kb = 0; kb < KB; ++kb) {
+                const int st_prev = st == 0 ? S - 1 : st - 1;
 #pragma unroll
-                for (int t = 4; t < 8; ++t) issue_load(t, min(kb + 1, KB - 1), (kb & 1) ^ 1);
-                __builtin_amdgcn_s_waitcnt(0x0f70);
-                __syncthreads();
+                for (int t = A_LOADS; t < A_LOADS + B_LOADS; ++t) issue_load(t, min(kb - 1 + S, KB - 1), st_prev);
+                __builtin_amdgcn_s_waitcnt(kWaitSync);
+                wg_barrier();
 #pragma unroll
-                for (int t = 0; t < 4; ++t) issue_load(t, min(kb + 2, KB - 1), kb & 1);
-                issue_scales(min(kb + 2, KB - 1), kb & 1);
+                for (int t = 0; t < A_LOADS; ++t) issue_load(t, min(kb + S, KB - 1), st);
+                issue_scales(min(kb + S, KB - 1), st);
+                st = next_stage(st);
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);
         } else {
         float sc[JA], sc_nxt[JA];
-        __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
-        __syncthreads();
-#pragma unroll
-        for (int t = 0; t < 4; ++t) issue_load(t, min(1, KB - 1), 1);
-        issue_scales(min(1, KB - 1), 1);
         {
             const float bs = lds_bs(0);
 #pragma unroll
@@ -238,14 +263,15 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
             nf1 = join(*(const v4i*)(bs_base + 2048 + c0), *(const v4i*)(bs_base + 2048 + c1));
         }
 
+        int stage = 0;                        // LDS stage of block kb
         for (int kb = 0; kb < KB; ++kb) {
-            const int stage = kb & 1;
+            const int st_next = next_stage(stage), st_prev = stage == 0 ? S - 1 : stage - 1;
             const uint8_t* bs_base = lds + b_rd + stage * B_STAGE;
-            const uint8_t* as_next = lds + a_rd + (stage ^ 1) * A_STAGE;
-            const uint8_t* bs_next = lds + b_rd + (stage ^ 1) * B_STAGE;
+            const uint8_t* as_next = lds + a_rd + st_next * A_STAGE;
+            const uint8_t* bs_next = lds + b_rd + st_next * B_STAGE;
 
-            // branch-free: past the end the loop re-fetches the last block into a stage nobody reads again
-            const int kn1 = min(kb + 1, KB - 1), kn2 = min(kb + 2, KB - 1);
+            // branch-free: past the end the loop re-fetches the last block into stages nobody reads again
+            const int kb_w = min(kb - 1 + S, KB - 1), kb_a = min(kb + S, KB - 1);
 
             // fold the tile left over from the previous K block with that block's scale, then switch scales
 #pragma unroll
@@ -257,16 +283,16 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 #pragma unroll
             for (int i = 0; i < SN; ++i) {
                 if (i == kSync) {
-                    // every LDS read of this stage has returned and this wavefront's share of the other stage
+                    // every LDS read of this stage has returned and this wavefront's share of the next stage
                     // (tiles and scales of block kb+1) has landed
-                    __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
-                    __syncthreads();
+                    __builtin_amdgcn_s_waitcnt(kWaitSync);
+                    wg_barrier();
                     {
-                        const float bs = lds_bs(stage ^ 1);
+                        const float bs = lds_bs(st_next);
 #pragma unroll
-                        for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, stage ^ 1) * bs;
+                        for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, st_next) * bs;
                     }
-                    issue_scales(kn2, stage);
+                    issue_scales(kb_a, stage);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // weight rows are streamed two steps ahead; the last two steps fetch steps 0 and 1 of the next block
@@ -290,16 +316,15 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 #pragma unroll
                     for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(p[j - 1][e], sc[j - 1], acc[i][j - 1][e]);
                 }
-                // Refill of the stage that the barrier freed, spread over four steps so that the address unit sees
-                // two loads per wavefront at a time and not a burst of eight from every wavefront at once: the
-                // activation half of block kb+2 now, the weight half of block kb+1 in the first two steps.
+                // refill, see above: activation part of block kb+S after the barrier, weight part of block kb-1+S
+                // at the start of the block
                 if (i >= kSync) {
-                    issue_load((i - kSync) * 2, kn2, stage);
-                    issue_load((i - kSync) * 2 + 1, kn2, stage);
+#pragma unroll
+                    for (int t = 0; t < A_LOADS / 2; ++t) issue_load((i - kSync) * (A_LOADS / 2) + t, kb_a, stage);
                 }
                 if (i < 2) {
-                    issue_load(4 + i * 2, kn1, stage ^ 1);
-                    issue_load(5 + i * 2, kn1, stage ^ 1);
+#pragma unroll
+                    for (int t = 0; t < B_LOADS / 2; ++t) issue_load(A_LOADS + i * (B_LOADS / 2) + t, kb_w, st_prev);
                 }
                 pend = p[JA - 1];
                 nf0 = nf1;
@@ -316,15 +341,17 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
+            stage = st_next;
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[SN - 1][JA - 1][e] = __builtin_fmaf(pend[e], sc[JA - 1], acc[SN - 1][JA - 1][e]);
-        __builtin_amdgcn_s_waitcnt(0x0f70);             // the clamped refills of the last two blocks are still in flight
+        __builtin_amdgcn_s_waitcnt(0x0f70);             // the clamped refills of the last blocks are still in flight
         }
     };
-    if (!G || ja_live == 4) pipeline(std::integral_constant<int, 4>{});
-    else if (ja_live == 3)  pipeline(std::integral_constant<int, 3>{});
-    else if (ja_live == 2)  pipeline(std::integral_constant<int, 2>{});
+    static_assert(SM == 4 || SM == 2, "dispatch below");
+    if (!G || ja_live == SM) pipeline(std::integral_constant<int, SM>{});
+    else if (SM == 4 && ja_live == 3) pipeline(std::integral_constant<int, (SM == 4 ? 3 : 1)>{});
+    else if (SM == 4 && ja_live == 2) pipeline(std::integral_constant<int, (SM == 4 ? 2 : 1)>{});
     else if (ja_live == 1)  pipeline(std::integral_constant<int, 1>{});
     else { pipeline(std::integral_constant<int, 0>{}); return; }
 #undef DSV3_SGB
@@ -367,13 +394,14 @@ bool prefill_supported(int64_t m, int64_t n, int64_t k) {
 }
 
 namespace {
-template <int CD, bool G>
+template <int CD, bool G, int TM, int S>
 int launch_kernel(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                   int64_t m, int64_t n, int64_t k, int64_t tm, prefill::GroupTable g, hipStream_t stream) {
     using namespace prefill;
+    constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
     const int64_t tn = (n + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
-    auto kern = fp8_gemm_prefill_kernel<CD, G>;
+    auto kern = fp8_gemm_prefill_kernel<CD, G, TM, S>;
     static bool granted[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
@@ -387,17 +415,17 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
                        (int)m, (int)n, (int)k, (int)tm, (int)tn, g);
     return launch_status();
 }
+constexpr int kGroupedTileRows = 128;
 }  // namespace
 
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, hipStream_t stream) {
-    return launch_kernel<CD, false>(a, a_s, b, b_s, c, m, n, k, (m + prefill::BM - 1) / prefill::BM,
-                                    prefill::GroupTable{}, stream);
+    return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, (m + 255) / 256, prefill::GroupTable{}, stream);
 }
 
 // Rows per tile slot of the grouped kernel: the caller's tile table is built for this height.
-int grouped_tile_rows() { return prefill::BM; }
+int grouped_tile_rows() { return kGroupedTileRows; }
 
 // a: [a_num_rows, k] fp8 with scales a_s; c: [m, n]; group tables as described at GroupTable.  Byte offsets of a
 // and of one group's weights must fit 32 bits.
@@ -410,7 +438,7 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
                    int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
                    const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream) {
     prefill::GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
-    return launch_kernel<CD, true>(a, a_s, b, b_s, c, m, n, k, num_tiles, g, stream);
+    return launch_kernel<CD, true, kGroupedTileRows, 3>(a, a_s, b, b_s, c, m, n, k, num_tiles, g, stream);
 }
 
 #define DSV3_INST(CD) \
