@@ -18,6 +18,7 @@
 // 16-byte chunks of one row in a permuted order p = c ^ f(row), which leaves the
 // later ds_read_b128 fragment reads (16 consecutive rows, same chunk) free of
 // bank conflicts.
+#include <cstdlib>
 #include <type_traits>
 #include "common.hpp"
 
@@ -416,11 +417,21 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
     return launch_status();
 }
 constexpr int kGroupedTileRows = 128;
+inline int env_tile_rows() { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }
 }  // namespace
 
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, hipStream_t stream) {
+    // Two tile heights.  A round of 256-row tiles over the 256 compute units takes about 1.64x as long as a round
+    // of 128-row tiles (measured, K = 7168), and the last round is rarely full: pick whichever needs less time in
+    // whole rounds.  (M = 4096 x N = 18432: 5 rounds of 256-row tiles beat 9 of 128-row ones; M = 1024: 3 short
+    // rounds beat 2 long ones; below ~400 rows the 128-row tile always wins.)
+    const int64_t tn = (n + prefill::BN - 1) / prefill::BN;
+    const int64_t r256 = ((m + 255) / 256 * tn + 255) / 256, r128 = ((m + 127) / 128 * tn + 255) / 256;
+    const int forced = env_tile_rows();
+    if (forced == 128 || (forced != 256 && 100 * r128 <= 164 * r256))
+        return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, (m + 127) / 128, prefill::GroupTable{}, stream);
     return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, (m + 255) / 256, prefill::GroupTable{}, stream);
 }
 

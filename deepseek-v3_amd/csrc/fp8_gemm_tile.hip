@@ -297,7 +297,7 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
     }
     const Plan p = make_plan(m, n, k);
     if (p.splits == 1) {
-        if (prefill_supported(m, n, k) && m > 64 && (force == 2 || (force == 0 && m >= 192)))
+        if (prefill_supported(m, n, k) && m > 64 && force != 1)
             return launch_prefill<CD>(a, a_s, b, b_s, c, m, n, k, st);
         if (p.bm == 32) return launch_cfg<32, 128, 32, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
         if (p.bm == 64) return launch_cfg<64, 128, 64, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
