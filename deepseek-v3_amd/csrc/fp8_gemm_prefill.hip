@@ -84,7 +84,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
-        int M, int N, int K, int tiles_m, int tiles_n, GroupTable g) {
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, GroupTable g) {
     using C = Cfg<TM, S>;
     constexpr int WM = C::WM, SM = C::SM, A_LOADS = C::A_LOADS, B_LOADS = C::B_LOADS;
     constexpr int A_STAGE = C::A_STAGE, B_STAGE = C::B_STAGE, LDS_A = C::LDS_A, LDS_B = C::LDS_B, LDS_SC = C::LDS_SC;
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         if (grp < 0) return;            // uniform over the workgroup, before any barrier
         m0 = g.tile_row0[tm];
         rows_here = g.tile_rows[tm];
-        n0 = tn * BN;
+        n0 = (tn_first + tn) * BN;
         b += (size_t)grp * g.b_stride;
         b_s += (size_t)grp * g.bs_stride;
     } else {
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const int in_band = pid - band * GROUP_M * tiles_n;
         const int tm = band * GROUP_M + in_band % band_rows;
         const int tn = in_band / band_rows;
-        m0 = tm * TM; n0 = tn * BN;
+        m0 = tm * TM; n0 = (tn_first + tn) * BN;
         rows_here = min(TM, M - m0);
     }
     // row of a behind row r of the tile; rows past the tile's end repeat its last row (their results are dropped)
@@ -395,13 +395,15 @@ bool prefill_supported(int64_t m, int64_t n, int64_t k) {
 }
 
 namespace {
+// Launches the column tiles [tn_first, tn_first + tn_count) of every row tile.
 template <int CD, bool G, int TM, int S>
 int launch_kernel(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
-                  int64_t m, int64_t n, int64_t k, int64_t tm, prefill::GroupTable g, hipStream_t stream) {
+                  int64_t m, int64_t n, int64_t k, int64_t tm, int64_t tn_first, int64_t tn_count,
+                  prefill::GroupTable g, hipStream_t stream) {
     using namespace prefill;
     constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
-    const int64_t tn = (n + BN - 1) / BN;
-    if (tm * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (tm * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (tm * tn_count == 0) return DSV3_OK;
     auto kern = fp8_gemm_prefill_kernel<CD, G, TM, S>;
     static bool granted[64] = {};
     int dev = 0;
@@ -411,12 +413,13 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
             return DSV3_ERR_LAUNCH;
         granted[dev] = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(THREADS), LDS_BYTES, stream,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn_count)), dim3(THREADS), LDS_BYTES, stream,
                        (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c,
-                       (int)m, (int)n, (int)k, (int)tm, (int)tn, g);
+                       (int)m, (int)n, (int)k, (int)tm, (int)tn_count, (int)tn_first, g);
     return launch_status();
 }
 constexpr int kGroupedTileRows = 128;
+constexpr int64_t kCUs = 256;
 inline int env_tile_rows() { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }
 }  // namespace
 
@@ -424,15 +427,25 @@ template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, hipStream_t stream) {
     // Two tile heights.  A round of 256-row tiles over the 256 compute units takes about 1.64x as long as a round
-    // of 128-row tiles (measured, K = 7168), and the last round is rarely full: pick whichever needs less time in
-    // whole rounds.  (M = 4096 x N = 18432: 5 rounds of 256-row tiles beat 9 of 128-row ones; M = 1024: 3 short
-    // rounds beat 2 long ones; below ~400 rows the 128-row tile always wins.)
+    // of 128-row tiles (measured, K = 7168), and the last round is rarely full.  Three plans, costed in whole
+    // rounds: all tall tiles, all short tiles, or tall tiles for as many column tiles as fill whole rounds and
+    // short tiles for the remaining columns (M = 4096 x N = 18432: 64 column tiles = 4 full rounds of tall tiles,
+    // the last 8 column tiles = exactly one round of short ones, instead of a fifth round that is half empty).
     const int64_t tn = (n + prefill::BN - 1) / prefill::BN;
-    const int64_t r256 = ((m + 255) / 256 * tn + 255) / 256, r128 = ((m + 127) / 128 * tn + 255) / 256;
+    const int64_t tm256 = (m + 255) / 256, tm128 = (m + 127) / 128;
+    auto rounds = [](int64_t tiles) { return (tiles + kCUs - 1) / kCUs; };
+    const int64_t cost_tall = 164 * rounds(tm256 * tn), cost_short = 100 * rounds(tm128 * tn);
+    const int64_t tn_tall = (tm256 * tn / kCUs) * kCUs / tm256;                   // column tiles in whole tall rounds
+    const int64_t cost_mixed = 164 * rounds(tm256 * tn_tall) + 100 * rounds(tm128 * (tn - tn_tall));
     const int forced = env_tile_rows();
-    if (forced == 128 || (forced != 256 && 100 * r128 <= 164 * r256))
-        return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, (m + 127) / 128, prefill::GroupTable{}, stream);
-    return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, (m + 255) / 256, prefill::GroupTable{}, stream);
+    const prefill::GroupTable none{};
+    if (forced == 128 || (forced == 0 && cost_short <= cost_tall && cost_short <= cost_mixed))
+        return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, tm128, 0, tn, none, stream);
+    if (forced == 256 || cost_tall <= cost_mixed || tn_tall == 0)
+        return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, tm256, 0, tn, none, stream);
+    const int rc = launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, tm256, 0, tn_tall, none, stream);
+    if (rc != DSV3_OK) return rc;
+    return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, tm128, tn_tall, tn - tn_tall, none, stream);
 }
 
 // Rows per tile slot of the grouped kernel: the caller's tile table is built for this height.
@@ -449,7 +462,8 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
                    int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
                    const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream) {
     prefill::GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
-    return launch_kernel<CD, true, kGroupedTileRows, 3>(a, a_s, b, b_s, c, m, n, k, num_tiles, g, stream);
+    return launch_kernel<CD, true, kGroupedTileRows, 3>(a, a_s, b, b_s, c, m, n, k, num_tiles, 0,
+                                                          (n + prefill::BN - 1) / prefill::BN, g, stream);
 }
 
 #define DSV3_INST(CD) \
