@@ -6,6 +6,9 @@
 //   moe_combine    y[t] = (sum over the token's experts, ascending expert index, of out * weight) + shared,
 //                  every step rounded to bf16 exactly where model.py:689-693 rounds
 //   group_tiles    per-group row counts -> the tile table the grouped GEMM reads (no host round trip)
+//   moe_route      expert indices of every token -> per-expert counts, expert-sorted token list, and for every
+//                  token its rows in that list in ascending expert order (what torch.where / bincount / the loop
+//                  order of model.py:683-689 determine), in four small launches and without a sort
 #include "common.hpp"
 
 namespace dsv3 {
@@ -112,7 +115,8 @@ __global__ __launch_bounds__(kThreads) void moe_combine_kernel(
 // ceil(count / tile_rows) each; slots past the last one are marked unused.  One workgroup, any group count.
 __global__ __launch_bounds__(kThreads) void group_tiles_kernel(
         const int* __restrict__ counts, int groups, int tile_rows, int max_tiles,
-        int* __restrict__ tile_group, int* __restrict__ tile_row0, int* __restrict__ tile_nrows) {
+        int* __restrict__ tile_group, int* __restrict__ tile_row0, int* __restrict__ tile_nrows,
+        int* __restrict__ offsets) {           // optional: first row of every group
     __shared__ int tile_base[kThreads + 1], row_base[kThreads + 1];
     int done_tiles = 0, done_rows = 0;
     for (int g0 = 0; g0 < groups; g0 += kThreads) {
@@ -131,6 +135,7 @@ __global__ __launch_bounds__(kThreads) void group_tiles_kernel(
             __syncthreads();
         }
         const int t0 = done_tiles + tile_base[threadIdx.x], r0 = done_rows + row_base[threadIdx.x];
+        if (offsets && g < groups) offsets[g] = r0;
         for (int i = 0; i < nt; ++i) {
             if (t0 + i < max_tiles) {
                 tile_group[t0 + i] = g;
@@ -146,7 +151,86 @@ __global__ __launch_bounds__(kThreads) void group_tiles_kernel(
     }
 }
 
+__global__ __launch_bounds__(kThreads) void fill_zero_kernel(int* __restrict__ p, int n) {
+    const int i = blockIdx.x * kThreads + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// counts[e] += number of (token, slot) pairs routed to expert e; a workgroup first adds up its pairs in LDS
+__global__ __launch_bounds__(kThreads) void route_count_kernel(
+        const int64_t* __restrict__ indices, int64_t pairs, int experts, int* __restrict__ counts) {
+    extern __shared__ int bins[];
+    for (int e = threadIdx.x; e < experts; e += kThreads) bins[e] = 0;
+    __syncthreads();
+    for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < pairs; p += (int64_t)gridDim.x * kThreads) {
+        const int64_t e = indices[p];
+        if (e >= 0 && e < experts) atomicAdd(&bins[e], 1);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += kThreads)
+        if (bins[e]) atomicAdd(&counts[e], bins[e]);
+}
+
+// One thread per token: its experts in ascending order get the next free row of their group.  The order of rows
+// inside a group depends on the order in which threads arrive, which is harmless: a row of the grouped GEMM does
+// not depend on its position, and `rows` records where each pair went.
+template <int MAXK>
+__global__ __launch_bounds__(kThreads) void route_scatter_kernel(
+        const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int tokens, int topk, int experts,
+        const int* __restrict__ offsets, int* __restrict__ cursor,
+        int* __restrict__ a_rows, int* __restrict__ rows, uint16_t* __restrict__ w_sorted) {
+    const int t = blockIdx.x * kThreads + threadIdx.x;
+    if (t >= tokens) return;
+    int e[MAXK], slot[MAXK];
+#pragma unroll
+    for (int j = 0; j < MAXK; ++j) {
+        e[j] = j < topk ? (int)indices[(int64_t)t * topk + j] : 0x7fffffff;
+        slot[j] = j;
+    }
+    // insertion sort by expert index (stable; the reference's top-k never repeats an expert for a token)
+#pragma unroll
+    for (int i = 1; i < MAXK; ++i) {
+#pragma unroll
+        for (int j = i; j > 0; --j) {
+            if (e[j] < e[j - 1]) {
+                const int te = e[j]; e[j] = e[j - 1]; e[j - 1] = te;
+                const int ts = slot[j]; slot[j] = slot[j - 1]; slot[j - 1] = ts;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < MAXK; ++j) {
+        if (j < topk) {
+            int pos = 0;
+            if (e[j] >= 0 && e[j] < experts) {
+                pos = offsets[e[j]] + atomicAdd(&cursor[e[j]], 1);
+                a_rows[pos] = t;
+            }
+            rows[(int64_t)t * topk + j] = pos;
+            w_sorted[(int64_t)t * topk + j] = weights[(int64_t)t * topk + slot[j]];
+        }
+    }
+}
+
 }  // namespace
+
+int launch_moe_route(const int64_t* indices, const void* weights, int64_t tokens, int topk, int experts,
+                     int max_tiles, int tile_rows, int* counts, int* offsets, int* cursor, int* a_rows, int* rows,
+                     void* w_sorted, int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st) {
+    const int64_t pairs = tokens * topk;
+    // counts | offsets | cursor are consecutive thirds of one scratch array; clear it with a kernel (a memset node
+    // recorded into a captured graph has given wrong results on replays)
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((3 * experts + kThreads - 1) / kThreads)), dim3(kThreads), 0, st, counts, 3 * experts);
+    const unsigned cgrid = (unsigned)((pairs + kThreads * 8 - 1) / (kThreads * 8) > 1024 ? 1024 : (pairs + kThreads * 8 - 1) / (kThreads * 8));
+    hipLaunchKernelGGL(route_count_kernel, dim3(cgrid ? cgrid : 1), dim3(kThreads), (size_t)experts * sizeof(int), st,
+                       indices, pairs, experts, counts);
+    hipLaunchKernelGGL(group_tiles_kernel, dim3(1), dim3(kThreads), 0, st,
+                       (const int*)counts, experts, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows, offsets);
+    hipLaunchKernelGGL(route_scatter_kernel<16>, dim3((unsigned)((tokens + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
+                       indices, (const uint16_t*)weights, (int)tokens, topk, experts, (const int*)offsets, cursor,
+                       a_rows, rows, (uint16_t*)w_sorted);
+    return launch_status();
+}
 
 int launch_swiglu_quant(const void* h, void* y, float* s, int64_t rows, int64_t inter, int scale_fmt, hipStream_t st) {
     const int64_t n_chunks = rows * inter / 8;
@@ -171,7 +255,7 @@ int launch_moe_combine(const void* out, const int* rows, const void* w, const vo
 int launch_group_tiles(const int* counts, int groups, int tile_rows, int max_tiles,
                        int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st) {
     hipLaunchKernelGGL(group_tiles_kernel, dim3(1), dim3(kThreads), 0, st,
-                       counts, groups, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows);
+                       counts, groups, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows, (int*)nullptr);
     return launch_status();
 }
 

@@ -244,25 +244,18 @@ class MoE(nn.Module):
         w13, s13, w2, s2 = self._stacked
         tokens, topk = indices.shape
         pairs = tokens * topk
-        flat = indices.reshape(-1)
-        order = torch.argsort(flat, stable=True)                       # expert-sorted row -> (token, slot) pair
-        counts = torch.bincount(flat, minlength=self.n_routed_experts).to(torch.int32)
-        a_rows = (order // topk).to(torch.int32)                       # token behind each expert-sorted row
-        max_tiles = pairs // ops.grouped_tile_rows() + self.n_routed_experts
-        tile_group, tile_row0, tile_rows = torch.ops.dsv3fp8.group_tiles(counts, max_tiles)
+        # counts per expert, expert-sorted token list, each token's rows in ascending expert order (the order in
+        # which the reference's loop adds them, model.py:684-689) and the tile table -- all on the device
+        _, a_rows, rows, w_sorted, tile_group, tile_row0, tile_rows = torch.ops.dsv3fp8.moe_route(
+            indices.contiguous(), weights.contiguous(), self.n_routed_experts)
         fmt = ops._lib.SCALE_FMT_UE8M0 if Linear.scale_fmt == "ue8m0" else ops._lib.SCALE_FMT_NONE
         code = ops.dtype_code(torch.get_default_dtype())
         xq, xs = act_quant(x, block_size, Linear.scale_fmt)           # quantised once: 1x128 blocks are per token
         h = torch.ops.dsv3fp8.fp8_gemm_grouped(xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, code)
         gq, gs = torch.ops.dsv3fp8.swiglu_quant(h, block_size, fmt)
         out = torch.ops.dsv3fp8.fp8_gemm_grouped(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code)
-        # the reference adds a token's expert outputs in ascending expert index (its loop order, model.py:684-689)
-        slot = indices.argsort(dim=1)
-        pos = torch.empty_like(order)
-        pos[order] = torch.arange(pairs, device=order.device)
-        rows = pos.view(tokens, topk).gather(1, slot).to(torch.int32)
         z = self.shared_experts(x)
-        return torch.ops.dsv3fp8.moe_combine(out, rows, weights.gather(1, slot).contiguous(), z.contiguous())
+        return torch.ops.dsv3fp8.moe_combine(out, rows, w_sorted, z.contiguous())
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         shape = x.size()

@@ -133,6 +133,21 @@ int dsv3_group_tiles(const int32_t* counts, int groups, int max_tiles,
                      int32_t* tile_group, int32_t* tile_row0, int32_t* tile_rows, void* stream);
 
 /*
+ * Routing bookkeeping of one MoE forward, on the device (inference/model.py:683-689: bincount, the per-expert
+ * torch.where token lists, and the order in which the loop over experts touches a token):
+ *     indices [tokens, topk] int64 (the router's expert choices), weights [tokens, topk] (2-byte dtype)  ->
+ *     scratch [3*experts] int32: counts per expert, first row per expert, (internal cursor);
+ *     a_rows  [tokens*topk]    : token behind every row of the expert-sorted row list (groups back to back);
+ *     rows    [tokens, topk]   : for every token, its rows in that list in ascending expert order;
+ *     w_sorted[tokens, topk]   : the routing weights in the same order;
+ *     tile_group/tile_row0/tile_rows [max_tiles]: the tile table of dsv3_group_tiles for these counts.
+ * The order of rows inside an expert's group is unspecified (it does not affect any result).  topk <= 16.
+ */
+int dsv3_moe_route(const int64_t* indices, const void* weights, int w_dtype, int64_t tokens, int topk, int experts,
+                   int max_tiles, int32_t* scratch, int32_t* a_rows, int32_t* rows, void* w_sorted,
+                   int32_t* tile_group, int32_t* tile_row0, int32_t* tile_rows, void* stream);
+
+/*
  * Grouped fp8_gemm (inference/kernel.py:145-172 applied per expert as in inference/model.py:684-689):
  *     for every tile slot t with group g = tile_group[t] >= 0, rows r in [tile_row0[t], tile_row0[t]+tile_rows[t]):
  *         c[r, :] = fp8_gemm( a[src(r), :], a_s[src(r), :], b + g*b_group_stride, b_s + g*bs_group_stride )

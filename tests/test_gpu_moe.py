@@ -180,3 +180,34 @@ def test_moe_grouped_matches_expert_loop_and_oracle(K):
         M.MoE.grouped = True
         M.gemm_impl, M.Linear.dtype = old[0], old[2]
         torch.set_default_dtype(old[1])
+
+
+@pytest.mark.parametrize("tokens,topk,experts", [(300, 2, 8), (4096, 8, 256), (1, 4, 16), (33, 1, 5)])
+def test_moe_route(K, tokens, topk, experts):
+    from dsv3fp8 import ops
+    g = torch.Generator().manual_seed(7)
+    scores = torch.rand(tokens, experts, generator=g)
+    scores[:, experts // 2] += 0.3 * (torch.arange(tokens) % 3 == 0)            # a popular expert
+    indices = scores.topk(topk, dim=-1)[1]
+    weights = torch.rand(tokens, topk, generator=g).bfloat16()
+    counts, a_rows, rows, w_sorted, tg, t0, tr = torch.ops.dsv3fp8.moe_route(indices.cuda(), weights.cuda(), experts)
+    counts, a_rows, rows, w_sorted = counts.cpu(), a_rows.cpu(), rows.cpu(), w_sorted.cpu()
+    ref_counts = torch.bincount(indices.flatten(), minlength=experts)
+    assert torch.equal(counts.long(), ref_counts)
+    offsets = torch.cumsum(ref_counts, 0) - ref_counts
+    pairs = tokens * topk
+    assert sorted(rows.flatten().tolist()) == list(range(pairs))               # every row used exactly once
+    for e in range(experts):                                                    # group e = the tokens that chose e
+        grp = a_rows[offsets[e]:offsets[e] + ref_counts[e]].long()
+        assert torch.equal(grp.sort()[0], torch.where((indices == e).any(-1))[0])
+    order = indices.argsort(dim=1)
+    se = indices.gather(1, order)
+    assert torch.equal(w_sorted.view(torch.int16), weights.gather(1, order).view(torch.int16))
+    for j in range(topk):                                                       # rows[t, j] lies in the group of the j-th smallest expert
+        r = rows[:, j].long()
+        assert torch.equal(a_rows[r].long(), torch.arange(tokens))
+        assert ((r >= offsets[se[:, j]]) & (r < offsets[se[:, j]] + ref_counts[se[:, j]])).all()
+    R = ops.grouped_tile_rows()
+    exp_tiles = [(e, int(offsets[e]) + i, min(R, int(ref_counts[e]) - i)) for e in range(experts) for i in range(0, int(ref_counts[e]), R)]
+    got = list(zip(tg.tolist(), t0.tolist(), tr.tolist()))
+    assert got[:len(exp_tiles)] == exp_tiles and all(x[0] == -1 for x in got[len(exp_tiles):])
