@@ -211,3 +211,44 @@ def test_moe_route(K, tokens, topk, experts):
     exp_tiles = [(e, int(offsets[e]) + i, min(R, int(ref_counts[e]) - i)) for e in range(experts) for i in range(0, int(ref_counts[e]), R)]
     got = list(zip(tg.tolist(), t0.tolist(), tr.tolist()))
     assert got[:len(exp_tiles)] == exp_tiles and all(x[0] == -1 for x in got[len(exp_tiles):])
+
+
+def test_moe_forward_is_graph_capturable(K):
+    """The grouped path issues no host synchronisation (the reference's loop needs bincount(...).tolist()): one
+    forward can be captured in a HIP graph and replayed, with eager work between the replays."""
+    from dsv3fp8 import model as M
+    old = (M.gemm_impl, torch.get_default_dtype(), M.Linear.dtype)
+    torch.set_default_dtype(torch.bfloat16)
+    M.Linear.dtype = FP8
+    M.gemm_impl = "fp8"
+    try:
+        args = M.ModelArgs(dim=256, inter_dim=512, moe_inter_dim=128, n_routed_experts=8, n_shared_experts=1,
+                           n_activated_experts=2, n_expert_groups=2, n_limited_groups=1, route_scale=2.5)
+        with torch.device("cuda"):
+            moe = M.MoE(args)
+        g = torch.Generator(device="cuda").manual_seed(11)
+        with torch.no_grad():
+            moe.gate.weight.copy_(torch.randn(8, 256, generator=g, device="cuda") * 0.05)
+            for lin in [l for ex in list(moe.experts) + [moe.shared_experts] for l in (ex.w1, ex.w2, ex.w3)]:
+                w8, s = oracle.block_quant_weight((torch.randn(lin.out_features, lin.in_features) * 0.05).bfloat16())
+                lin.weight.copy_(w8.cuda()); lin.scale.copy_(s.cuda())
+        moe.stack_experts()
+        x = torch.randn(200, 256, generator=g, device="cuda").bfloat16()
+        static_x = x.clone()
+        with torch.inference_mode():
+            eager = moe(x).clone()
+            moe(static_x)                                   # warm-up outside capture (workspaces, attributes)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_y = moe(static_x)
+            for rep in range(3):
+                x2 = torch.randn(200, 256, generator=g, device="cuda").bfloat16() if rep else x
+                static_x.copy_(x2)
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(static_y, moe(x2)), rep      # eager work between replays, every replay checked
+        assert torch.equal(eager, moe(x))
+    finally:
+        M.gemm_impl, M.Linear.dtype = old[0], old[2]
+        torch.set_default_dtype(old[1])
