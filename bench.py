@@ -137,7 +137,7 @@ def run_extras(K, W):
 
 
 def run_moe(K, W, tokens: int = 4096):
-    """BASELINE config 5: one MoE layer (256 routed + 1 shared SwiGLU experts, 7168 -> 2048 -> 7168, fp8
+    """The MoE-layer configuration: one MoE layer (256 routed + 1 shared SwiGLU experts, 7168 -> 2048 -> 7168, fp8
     block-scaled weights generated on the device), T tokens, sigmoid gate with bias over random logits'
     weights, 8 groups / top-4 groups / top-8 experts, route_scale 2.5.  Timed twice: the grouped path
     (device-side token lists, two grouped GEMMs, fused SwiGLU + re-quantisation, ordered combine) and the
@@ -208,7 +208,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is built and measured on ONE GPU (one GPU's share of the work at its real "
-                 "shape); --gpus must be 1. Sharding is described in DESIGN.md.")
+                 "shape); --gpus must be 1.")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback.")
 

@@ -241,7 +241,7 @@ def test_fp8_gemm_close_to_unquantised_product():
 
 
 def test_cfg1_cpu_plumbing():
-    """BASELINE config 1: x [16,7168], wq_a-shaped weight [1536,7168], seed 0."""
+    """The CPU-plumbing configuration: x [16,7168], wq_a-shaped weight [1536,7168], seed 0."""
     from dsv3fp8 import workloads
     x, w8, ws = workloads.cfg1_cpu_plumbing()
     assert ws.shape == (12, 56)
