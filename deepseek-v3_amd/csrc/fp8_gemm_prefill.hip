@@ -427,25 +427,17 @@ template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, hipStream_t stream) {
     // Two tile heights.  A round of 256-row tiles over the 256 compute units takes about 1.64x as long as a round
-    // of 128-row tiles (measured, K = 7168), and the last round is rarely full.  Three plans, costed in whole
-    // rounds: all tall tiles, all short tiles, or tall tiles for as many column tiles as fill whole rounds and
-    // short tiles for the remaining columns (M = 4096 x N = 18432: 64 column tiles = 4 full rounds of tall tiles,
-    // the last 8 column tiles = exactly one round of short ones, instead of a fifth round that is half empty).
+    // of 128-row tiles (measured, K = 7168), and the last round is rarely full: pick whichever needs less time in
+    // whole rounds.  (M = 4096 x N = 18432: 5 rounds of tall tiles beat 9 of short ones; M = 1024: 3 short rounds
+    // beat 2 tall ones; below ~400 rows the short tile always wins.)
     const int64_t tn = (n + prefill::BN - 1) / prefill::BN;
     const int64_t tm256 = (m + 255) / 256, tm128 = (m + 127) / 128;
     auto rounds = [](int64_t tiles) { return (tiles + kCUs - 1) / kCUs; };
-    const int64_t cost_tall = 164 * rounds(tm256 * tn), cost_short = 100 * rounds(tm128 * tn);
-    const int64_t tn_tall = (tm256 * tn / kCUs) * kCUs / tm256;                   // column tiles in whole tall rounds
-    const int64_t cost_mixed = 164 * rounds(tm256 * tn_tall) + 100 * rounds(tm128 * (tn - tn_tall));
     const int forced = env_tile_rows();
     const prefill::GroupTable none{};
-    if (forced == 128 || (forced == 0 && cost_short <= cost_tall && cost_short <= cost_mixed))
+    if (forced == 128 || (forced != 256 && 100 * rounds(tm128 * tn) <= 164 * rounds(tm256 * tn)))
         return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, tm128, 0, tn, none, stream);
-    if (forced == 256 || cost_tall <= cost_mixed || tn_tall == 0)
-        return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, tm256, 0, tn, none, stream);
-    const int rc = launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, tm256, 0, tn_tall, none, stream);
-    if (rc != DSV3_OK) return rc;
-    return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, tm128, tn_tall, tn - tn_tall, none, stream);
+    return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, tm256, 0, tn, none, stream);
 }
 
 // Rows per tile slot of the grouped kernel: the caller's tile table is built for this height.
