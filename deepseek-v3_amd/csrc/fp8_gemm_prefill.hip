@@ -90,25 +90,30 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     constexpr int A_STAGE = C::A_STAGE, B_STAGE = C::B_STAGE, LDS_A = C::LDS_A, LDS_B = C::LDS_B, LDS_SC = C::LDS_SC;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
-    // ---- workgroup -> tile: contiguous run of tiles per XCD; dense mode walks bands of GROUP_M tile rows,
-    // grouped mode keeps the column tiles of one row tile together (they share the gathered rows of a)
-    const int T = tiles_m * tiles_n;
-    int pid = blockIdx.x;
-    {
-        const int q = T / 8, r = T % 8, x = pid % 8;
-        pid = x * q + (x < r ? x : r) + pid / 8;
-    }
+    // ---- workgroup -> tile.  Consecutive workgroup ids go to consecutive XCDs (8 of them, each with its own L2).
+    // Dense mode gives every XCD a contiguous run of tiles and walks it in bands of GROUP_M tile rows.  Grouped
+    // mode deals the row tiles round-robin over the XCDs -- the live ones sit at the front of the tile table, and a
+    // contiguous split would leave the XCDs that get the unused tail idle -- and keeps the column tiles of a row
+    // tile on one XCD (they share the gathered rows of a).
     int m0, n0, rows_here;              // first row of the tile in c, first column, valid rows
     if (G) {
-        const int tm = pid / tiles_n, tn = pid - tm * tiles_n;
+        const int x = blockIdx.x % 8, idx = blockIdx.x / 8;
+        const int tm = (idx / tiles_n) * 8 + x, tn = idx - (idx / tiles_n) * tiles_n;
+        if (tm >= tiles_m) return;      // uniform over the workgroup, before any barrier
         const int grp = g.tile_group[tm];
-        if (grp < 0) return;            // uniform over the workgroup, before any barrier
+        if (grp < 0) return;
         m0 = g.tile_row0[tm];
         rows_here = g.tile_rows[tm];
         n0 = (tn_first + tn) * BN;
         b += (size_t)grp * g.b_stride;
         b_s += (size_t)grp * g.bs_stride;
     } else {
+        const int T = tiles_m * tiles_n;
+        int pid = blockIdx.x;
+        {
+            const int q = T / 8, r = T % 8, x = pid % 8;
+            pid = x * q + (x < r ? x : r) + pid / 8;
+        }
         constexpr int GROUP_M = 4;
         const int band = pid / (GROUP_M * tiles_n);
         const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
@@ -402,7 +407,7 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
                   prefill::GroupTable g, hipStream_t stream) {
     using namespace prefill;
     constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
-    if (tm * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if ((tm + 8) * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (tm * tn_count == 0) return DSV3_OK;
     auto kern = fp8_gemm_prefill_kernel<CD, G, TM, S>;
     static bool granted[64] = {};
@@ -413,7 +418,8 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
             return DSV3_ERR_LAUNCH;
         granted[dev] = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn_count)), dim3(THREADS), LDS_BYTES, stream,
+    const int64_t grid = (G ? (tm + 7) / 8 * 8 : tm) * tn_count;       // grouped: row tiles are dealt over the 8 XCDs
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream,
                        (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c,
                        (int)m, (int)n, (int)k, (int)tm, (int)tn_count, (int)tn_first, g);
     return launch_status();
