@@ -67,6 +67,20 @@ def test_mid_m(K, m):
     _check(K, x, w8, ws)
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (100, 300, 128),      # one K block: the pipeline's prologue and clamped refills only (short tiles, 3 LDS stages)
+    (130, 256, 256),      # two K blocks, two short row tiles, the second with 2 rows
+    (2048, 8192, 128),    # one full round of tall tiles (256 rows, 2 LDS stages), one K block
+    (2050, 8192, 384),    # tall tiles with a 2-row edge tile, odd number of K blocks
+    (1024, 18432, 256),   # short tiles chosen for a large problem (3 rounds of short beat 2 of tall)
+])
+def test_large_m_tile_heights_and_short_k(K, m, n, k):
+    from dsv3fp8 import workloads
+    x = workloads.activations(m, k, seed=m)
+    w8, ws = workloads.weight(n, k, seed=n % 89)
+    _check(K, x, w8, ws)
+
+
 @pytest.mark.parametrize("n", [1, 15, 16, 100, 129, 576, 577, 1000])
 def test_ragged_n(K, n):
     from dsv3fp8 import workloads
