@@ -190,7 +190,7 @@ inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
     p.mt = (int)((m + 15) / 16);
     if (p.mt == 3) p.mt = 4;                                    // 3 sub-tiles run as 4 (chunk size stays a power of two)
     const int64_t kb = k / 128, groups = (n + 63) / 64;
-    if (groups < 96) return p;                                  // too few workgroups: the in-workgroup split-K kernels do better
+    if (groups < 4) return p;                                   // a handful of rows: not worth a streaming plan
     const int64_t capacity = 256 * 3;                           // resident workgroups (3 per CU)
     // K blocks per workgroup: a divisor of kb that is a multiple of the ring depth; take the split count that
     // fills one round best
