@@ -149,4 +149,23 @@ int dsv3_moe_combine(const void* expert_out, int dtype, const int32_t* rows, con
     return launch_moe_combine(expert_out, rows, weights, shared, y, tokens, topk, dim, (hipStream_t)stream);
 }
 
+int dsv3_wkv_b_absorb(const void* x, int64_t x_token_stride, int64_t x_head_stride,
+                      const void* wkv_b, const float* wkv_b_scale, void* y, int dtype, int side,
+                      int64_t tokens, int heads, int nope_dim, int v_dim, int64_t kv_rank, int block_size,
+                      void* stream) {
+    if (dtype != DSV3_BF16) return DSV3_ERR_BAD_DTYPE;
+    if (block_size != 128) return DSV3_ERR_BAD_BLOCK;
+    if (side != DSV3_ABSORB_Q && side != DSV3_ABSORB_V) return DSV3_ERR_BAD_SHAPE;
+    if (tokens < 0 || heads < 0 || heads > 65535 || tokens > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (!wkv_b_absorb_supported(side, nope_dim, v_dim, kv_rank)) return DSV3_ERR_BAD_SHAPE;
+    const int64_t in_dim = side == DSV3_ABSORB_Q ? nope_dim : kv_rank;
+    if (x_token_stride < 0 || x_head_stride < in_dim || x_token_stride % 8 != 0 || x_head_stride % 8 != 0)
+        return DSV3_ERR_BAD_SHAPE;
+    if (tokens == 0 || heads == 0) return DSV3_OK;
+    if (!x || !wkv_b || !wkv_b_scale || !y) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(x, 16) || !aligned(wkv_b, 16) || !aligned(y, 16) || !aligned(wkv_b_scale, 4)) return DSV3_ERR_MISALIGNED;
+    return launch_wkv_b_absorb(x, x_token_stride, x_head_stride, wkv_b, wkv_b_scale, y, side, tokens, heads,
+                               nope_dim, v_dim, kv_rank, (hipStream_t)stream);
+}
+
 }  // extern "C"

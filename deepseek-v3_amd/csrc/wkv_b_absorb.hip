@@ -1,0 +1,272 @@
+// The two per-head products of the absorbed MLA attention with the block-scaled fp8 weight wkv_b, without
+// materialising weight_dequant(wkv_b) (reference: inference/model.py:481-483 and :495).
+//
+//   wkv_b : fp8 [heads * (nope + v), C], scales fp32 [ceil(rows/128), C/128]; head h owns rows h*(nope+v) ...
+//   W     : bf16( f32(wkv_b) * scale )        -- exactly what weight_dequant would have written (kernel.py:83-86)
+//   side Q: y[m, h, c] = sum_d x[m, h, d] * W[h*(nope+v) + d,        c]     d < nope   ("bshd,hdc->bshc")
+//   side V: y[m, h, d] = sum_c x[m, h, c] * W[h*(nope+v) + nope + d, c]     d < v      ("bshc,hdc->bshd")
+//
+// Both are weight-stationary: a wavefront dequantises one slab of one head's weight ONCE into MFMA operand
+// registers (128 VGPRs of bf16: 128 x 128 for side Q, 32 x 512 for side V), then streams 16-token sub-tiles
+// past it with v_mfma_f32_16x16x32_bf16.  Operand roles are picked per side so that a lane ends up with
+// consecutive output features of a token and writes them with 16-byte stores.  Which output feature sits in
+// which MFMA row, and which K index sits in which operand slot, is free as long as both operands agree; the maps
+// below are chosen so that every global access of a lane is one aligned 8- or 16-byte piece:
+//
+//   side Q  (K = d runs over weight ROWS, features c are contiguous in memory)
+//     wave slab: 128 features c0 .. c0+127, 8 MFMA sub-tiles t; MFMA row i of sub-tile t is feature c0 + 8*i + t.
+//     lane (i = lane%16, g = lane/16) reads, for each of its 8 K rows of a 32-row step, the 8 bytes
+//     [c0 + 8*i, +8) -> byte t belongs to sub-tile t.  Side Q issues the activation as the A operand instead, so
+//     the lane owns features c0 + 8*i + [0, 8) of the four tokens 4*g .. 4*g+3 and a group of 16 lanes writes 256
+//     contiguous bytes of one token.
+//   side V  (K = c is contiguous in memory, features d are weight rows)
+//     wave slab: 32 features d0 .. d0+31, 2 sub-tiles; MFMA row i of sub-tile t is feature d0 + 8*(i/4) + 4*t + i%4.
+//     Within a 128-wide K block lane group g takes the 32 consecutive K values [32*g, +32) (four MFMA steps), so
+//     a lane reads 32 contiguous weight bytes and 64 contiguous activation bytes per K block, all inside one scale
+//     block.  It owns output features d0 + 8*g + [0, 8) of token i.
+//
+// HBM traffic: the weight slab once per workgroup (8.4 MB per side for the 671B shape), the activations once
+// (the four wavefronts of a workgroup share their reads through the L1), the output once.
+#include "common.hpp"
+
+namespace dsv3 {
+namespace {
+
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ v4f mfma_bf16(v4u a, v4u b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+}
+
+struct AbsorbArgs {
+    const uint16_t* x;      // bf16 activations
+    int64_t x_ts, x_hs;     // token / head stride of x in elements
+    const uint8_t* w;       // fp8 wkv_b
+    const float* ws;        // its block scales
+    int64_t w_cols;         // C
+    int ws_cols;            // C / 128
+    uint16_t* y;            // bf16 [tokens, heads, n_out]
+    int64_t tokens;
+    int heads, head_rows, nope, n_out;
+    int slabs;              // feature slabs per head (side Q: C/128, side V: v/32)
+    int subtiles;           // ceil(tokens / 16)
+};
+
+// 8 fp8 bytes -> 8 binary32
+__device__ __forceinline__ void cvt8(v2u p, float (&f)[8]) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        v2f lo = fp8x2_lo_to_f32(p[q]), hi = fp8x2_hi_to_f32(p[q]);
+        f[4 * q] = lo.x; f[4 * q + 1] = lo.y; f[4 * q + 2] = hi.x; f[4 * q + 3] = hi.y;
+    }
+}
+
+// side Q; KS = nope / 32 MFMA K steps
+template <int KS>
+__global__ __launch_bounds__(256) void absorb_q_kernel(AbsorbArgs p) {
+    const int lane = threadIdx.x & 63;
+    const int slab = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (slab >= p.slabs) return;
+    const int h = blockIdx.y, i = lane & 15, g = lane >> 4;
+    const int c0 = slab * 128;
+    const int64_t row0 = (int64_t)h * p.head_rows;
+
+    v4u A[KS][8];
+    {
+        v2u raw[KS][8];
+        float sc[KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const int64_t r = row0 + s * 32 + g * 8;       // 8 rows r .. r+7 lie in one scale block
+            sc[s] = p.ws[(r >> 7) * p.ws_cols + slab];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) raw[s][e] = *(const v2u*)(p.w + (r + e) * p.w_cols + c0 + i * 8);
+        }
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int e2 = 0; e2 < 4; ++e2) {
+                float f0[8], f1[8];
+                cvt8(raw[s][2 * e2], f0);
+                cvt8(raw[s][2 * e2 + 1], f1);
+#pragma unroll
+                for (int t = 0; t < 8; ++t) A[s][t][e2] = pack_bf16(f0[t] * sc[s], f1[t] * sc[s]);
+            }
+    }
+
+    // The token loop has no branches besides its back edge: rows past the end are clamped to the last token (they
+    // load, compute and store that token's values again) and the prefetch past the last sub-tile repeats it, so
+    // the compiler can count the stores that follow each prefetch instead of draining them (s_waitcnt vmcnt(4)).
+    const uint16_t* xh = p.x + (int64_t)h * p.x_hs + g * 8;
+    const int64_t last = p.tokens - 1;
+    auto load_b = [&](int ms, v4u (&b)[KS]) {
+        ms = ms < p.subtiles ? ms : p.subtiles - 1;
+        int64_t tok = (int64_t)ms * 16 + i;
+        tok = tok < last ? tok : last;
+        const uint16_t* src = xh + tok * p.x_ts;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) b[s] = *(const v4u*)(src + s * 32);
+    };
+
+    v4u bn[KS];
+    load_b(blockIdx.z, bn);
+    for (int ms = blockIdx.z; ms < p.subtiles; ms += gridDim.z) {
+        v4u b[KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) b[s] = bn[s];
+        load_b(ms + gridDim.z, bn);
+        // activations are the MFMA A operand here: the lane gets feature column i of sub-tile t (feature
+        // c0 + 8*i + t) for the four tokens 4*g + j, i.e. 8 consecutive features per token, and the 16 lanes of a
+        // group write one token's 128 features of this slab as 256 contiguous bytes
+        v4f acc[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc[t] = mfma_bf16(b[s], A[s][t], acc[t]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int64_t tok = (int64_t)ms * 16 + g * 4 + j;
+            tok = tok < last ? tok : last;
+            v4u o;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) o[q] = pack_bf16(acc[2 * q][j], acc[2 * q + 1][j]);
+            *(v4u*)(p.y + (tok * p.heads + h) * p.n_out + c0 + i * 8) = o;
+        }
+    }
+}
+
+// side V; KB = C / 128 scale blocks along K
+template <int KB>
+__global__ __launch_bounds__(256) void absorb_v_kernel(AbsorbArgs p) {
+    const int lane = threadIdx.x & 63;
+    const int slab = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (slab >= p.slabs) return;
+    const int h = blockIdx.y, i = lane & 15, g = lane >> 4;
+    const int d0 = slab * 32;
+    const int64_t row0 = (int64_t)h * p.head_rows + p.nope + d0;
+
+    v4u A[2][KB][4];
+    {
+        v4u raw[2][KB][2];
+        float sc[2][KB];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int64_t r = row0 + (i >> 2) * 8 + t * 4 + (i & 3);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                sc[t][kb] = p.ws[(r >> 7) * p.ws_cols + kb];
+                const v4u* src = (const v4u*)(p.w + r * p.w_cols + kb * 128 + g * 32);
+                raw[t][kb][0] = src[0];
+                raw[t][kb][1] = src[1];
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    // K values 8*s .. 8*s+7 of the lane's 32: dwords 2*s and 2*s+1 of the 32 bytes
+                    float f[8];
+                    cvt8(v2u{raw[t][kb][s >> 1][2 * (s & 1)], raw[t][kb][s >> 1][2 * (s & 1) + 1]}, f);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        A[t][kb][s][q] = pack_bf16(f[2 * q] * sc[t][kb], f[2 * q + 1] * sc[t][kb]);
+                }
+    }
+
+    // The token loop has no branches besides its back edge (see side Q).  A sub-tile is consumed in NS steps of KH
+    // K blocks; while one step's activations feed the MFMAs the next step's are in flight.
+    constexpr int NS = KB >= 2 ? 2 : 1, KH = KB / NS;
+    const uint16_t* xh = p.x + (int64_t)h * p.x_hs + g * 32;
+    const int64_t last = p.tokens - 1;
+    auto load_b = [&](int ms, int step, v4u (&b)[KH][4]) {
+        ms = ms < p.subtiles ? ms : p.subtiles - 1;
+        int64_t tok = (int64_t)ms * 16 + i;
+        tok = tok < last ? tok : last;
+        const uint16_t* src = xh + tok * p.x_ts + step * (KH * 128);
+#pragma unroll
+        for (int kb = 0; kb < KH; ++kb)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) b[kb][s] = *(const v4u*)(src + kb * 128 + s * 8);
+    };
+
+    v4u bn[KH][4];
+    load_b(blockIdx.z, 0, bn);
+    for (int ms = blockIdx.z; ms < p.subtiles; ms += gridDim.z) {
+        // two accumulators per sub-tile (even / odd K steps) keep four independent MFMA chains in flight
+        v4f acc[2][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) acc[t][0] = acc[t][1] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int step = 0; step < NS; ++step) {
+            v4u b[KH][4];
+#pragma unroll
+            for (int kb = 0; kb < KH; ++kb)
+#pragma unroll
+                for (int s = 0; s < 4; ++s) b[kb][s] = bn[kb][s];
+            if (step + 1 < NS) load_b(ms, step + 1, bn);
+            else load_b(ms + gridDim.z, 0, bn);
+#pragma unroll
+            for (int kb = 0; kb < KH; ++kb)
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                        acc[t][s & 1] = mfma_bf16(A[t][step * KH + kb][s], b[kb][s], acc[t][s & 1]);
+        }
+        int64_t tok = (int64_t)ms * 16 + i;
+        tok = tok < last ? tok : last;            // clamped rows rewrite the last token's values
+        v4u o;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const v4f r = acc[t][0] + acc[t][1];
+            o[2 * t] = pack_bf16(r[0], r[1]);
+            o[2 * t + 1] = pack_bf16(r[2], r[3]);
+        }
+        *(v4u*)(p.y + (tok * p.heads + h) * p.n_out + d0 + g * 8) = o;
+    }
+}
+
+}  // namespace
+
+bool wkv_b_absorb_supported(int side, int nope, int v, int64_t kv_rank) {
+    if (kv_rank <= 0 || kv_rank % 128 != 0 || nope % 32 != 0 || v % 32 != 0 || nope <= 0 || v <= 0) return false;
+    if (side == DSV3_ABSORB_Q) return nope == 64 || nope == 128;
+    return kv_rank == 128 || kv_rank == 256 || kv_rank == 512;
+}
+
+int launch_wkv_b_absorb(const void* x, int64_t x_ts, int64_t x_hs, const void* w, const float* ws, void* y, int side,
+                        int64_t tokens, int heads, int nope, int v, int64_t kv_rank, hipStream_t st) {
+    AbsorbArgs p;
+    p.x = (const uint16_t*)x; p.x_ts = x_ts; p.x_hs = x_hs;
+    p.w = (const uint8_t*)w; p.ws = ws; p.w_cols = kv_rank; p.ws_cols = (int)(kv_rank / 128);
+    p.y = (uint16_t*)y; p.tokens = tokens; p.heads = heads; p.head_rows = nope + v; p.nope = nope;
+    p.subtiles = (int)((tokens + 15) / 16);
+    const bool q = side == DSV3_ABSORB_Q;
+    p.n_out = q ? (int)kv_rank : v;
+    p.slabs = q ? (int)(kv_rank / 128) : v / 32;
+    // few tokens: one wavefront per workgroup spreads the weight reads over every CU; many tokens: the wavefronts
+    // of a workgroup take different slabs of the same head and share the activation reads
+    const int waves = p.subtiles > 4 ? 4 : 1;
+    const int gx = (p.slabs + waves - 1) / waves;
+    // token sub-tiles are dealt over gridDim.z so that about two workgroups per CU are resident
+    int gz = 512 / (gx * heads > 0 ? gx * heads : 1);
+    gz = gz < 1 ? 1 : gz;
+    gz = gz > p.subtiles ? p.subtiles : gz;
+    gz = gz > 65535 ? 65535 : gz;
+    const dim3 grid(gx, heads, gz), block(64 * waves);
+    if (q) {
+        if (nope == 128) hipLaunchKernelGGL(absorb_q_kernel<4>, grid, block, 0, st, p);
+        else hipLaunchKernelGGL(absorb_q_kernel<2>, grid, block, 0, st, p);
+    } else {
+        if (kv_rank == 512) hipLaunchKernelGGL(absorb_v_kernel<4>, grid, block, 0, st, p);
+        else if (kv_rank == 256) hipLaunchKernelGGL(absorb_v_kernel<2>, grid, block, 0, st, p);
+        else hipLaunchKernelGGL(absorb_v_kernel<1>, grid, block, 0, st, p);
+    }
+    return launch_status();
+}
+
+}  // namespace dsv3

@@ -14,6 +14,7 @@ LIB_PATH = Path(__file__).resolve().parent.parent / "lib" / "libdsv3fp8.so"
 # enum dsv3_dtype / dsv3_scale_fmt / dsv3_status (include/dsv3_fp8.h)
 BF16, F16, F32 = 0, 1, 2
 SCALE_FMT_NONE, SCALE_FMT_UE8M0 = 0, 1
+ABSORB_Q, ABSORB_V = 0, 1
 OK = 0
 
 EXPORTS = {
@@ -34,6 +35,8 @@ EXPORTS = {
     "dsv3_swiglu_quant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]),
     "dsv3_moe_combine": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int64, c_int, c_int64, c_void_p]),
+    "dsv3_wkv_b_absorb": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                  c_int64, c_int, c_int, c_int, c_int64, c_int, c_void_p]),
 }
 
 

@@ -1,9 +1,10 @@
 """Host-side callers of the FP8 kernels, mirroring the part of the reference's
 ``inference/model.py`` that sits directly on top of them: the ``linear()``
 dispatch (model.py:131-163), ``Linear`` and its column/row parallel variants
-(model.py:166-267), and the SwiGLU / routing modules that issue the FP8 linears
+(model.py:166-267), the SwiGLU / routing modules that issue the FP8 linears
 of the MoE layer (``MLP`` :500-532, ``Gate`` :535-598, ``Expert`` :601-633,
-``MoE`` :636-693).  Names, constructor arguments, the ``weight.scale``
+``MoE`` :636-693), and the attention layer ``MLA`` (:395-497) whose absorbed
+form multiplies with the FP8 weight ``wkv_b`` directly.  Names, constructor arguments, the ``weight.scale``
 convention and the module-level switches (``gemm_impl``, ``block_size``) follow
 the reference so that code written against it runs unchanged.
 
@@ -12,6 +13,7 @@ variants reduce to plain ``Linear`` and no collective is issued.
 """
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 from typing import Literal, Optional, Tuple
 
@@ -26,6 +28,7 @@ world_size = 1
 rank = 0
 block_size = 128
 gemm_impl: Literal["bf16", "fp8"] = "bf16"     # the reference's default (model.py:16); set to "fp8" for the FP8 GEMM path
+attn_impl: Literal["naive", "absorb"] = "absorb"   # model.py:17
 
 
 @dataclass
@@ -42,6 +45,21 @@ class ModelArgs:
     n_limited_groups: int = 4
     score_func: Literal["softmax", "sigmoid"] = "sigmoid"
     route_scale: float = 2.5
+    # attention (MLA) and its rotary embedding
+    max_batch_size: int = 8
+    max_seq_len: int = 4096 * 4
+    n_heads: int = 128
+    q_lora_rank: int = 1536
+    kv_lora_rank: int = 512
+    qk_nope_head_dim: int = 128
+    qk_rope_head_dim: int = 64
+    v_head_dim: int = 128
+    original_seq_len: int = 4096
+    rope_theta: float = 10000.0
+    rope_factor: float = 40
+    beta_fast: int = 32
+    beta_slow: int = 1
+    mscale: float = 1.
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -113,6 +131,147 @@ class RowParallelLinear(Linear):
         if self.bias is not None:
             y += self.bias
         return y
+
+
+class RMSNorm(nn.Module):
+    """x / rms(x) * weight over the last dimension (model.py:270-291)."""
+
+    def __init__(self, dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.dim = dim
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return F.rms_norm(x, (self.dim,), self.weight, self.eps)
+
+
+def precompute_freqs_cis(args: ModelArgs) -> torch.Tensor:
+    """Rotary phases e^{i * pos * f_j} for every position below ``max_seq_len`` as a complex64
+    ``[max_seq_len, qk_rope_head_dim / 2]`` tensor (model.py:294-372).  Beyond ``original_seq_len`` the
+    frequencies are stretched YaRN-style: pair j keeps its frequency where it completes more than ``beta_fast``
+    turns over the original window, is divided by ``rope_factor`` where it completes fewer than ``beta_slow``,
+    and is blended linearly in between."""
+    dim, base = args.qk_rope_head_dim, args.rope_theta
+    freqs = base ** (-torch.arange(0, dim, 2, dtype=torch.float32) / dim)
+    if args.max_seq_len > args.original_seq_len:
+        def pair_index(turns: float) -> float:     # the (fractional) pair that makes `turns` rotations in the window
+            return dim * math.log(args.original_seq_len / (turns * 2 * math.pi)) / (2 * math.log(base))
+        lo = max(math.floor(pair_index(args.beta_fast)), 0)
+        hi = min(math.ceil(pair_index(args.beta_slow)), dim - 1)
+        span = (hi - lo) if hi != lo else 0.001
+        stretched = ((torch.arange(dim // 2, dtype=torch.float32) - lo) / span).clamp(0, 1)   # 0: keep, 1: stretch
+        freqs = freqs / args.rope_factor * stretched + freqs * (1 - stretched)
+    angles = torch.outer(torch.arange(args.max_seq_len), freqs)
+    return torch.polar(torch.ones_like(angles), angles)
+
+
+def apply_rotary_emb(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
+    """Rotate consecutive pairs of the last dimension of ``x`` ``[b, s, h, r]`` by the phases of positions
+    ``[s, r/2]``, in binary32, and return the dtype of ``x`` (model.py:375-392)."""
+    pairs = x.float().unflatten(-1, (-1, 2))
+    re, im = pairs[..., 0], pairs[..., 1]
+    cos = freqs_cis.real.view(1, x.size(1), 1, -1)
+    sin = freqs_cis.imag.view(1, x.size(1), 1, -1)
+    return torch.stack((re * cos - im * sin, re * sin + im * cos), dim=-1).flatten(-2).to(x.dtype)
+
+
+class MLA(nn.Module):
+    """Multi-head latent attention (model.py:395-497) with the reference's two cache layouts.
+
+    ``attn_impl == "absorb"`` keeps the compressed latent (``kv_cache`` [b, t, kv_lora_rank]) and the shared
+    rotary key (``pe_cache``), and folds the up-projection ``wkv_b`` into the query and the output:
+    ``q_nope @ wkv_b[:, :nope]`` before the scores and ``@ wkv_b[:, -v:]^T`` after the weighted sum.  When
+    ``wkv_b`` is stored in FP8 the reference dequantises the whole weight on every call (model.py:481); here the
+    two products read the FP8 weight and its block scales directly (``torch.ops.dsv3fp8.wkv_b_absorb``), with
+    the same bf16 rounding of every dequantised weight.  ``MLA.fused = False`` selects the dequantise-then-einsum
+    sequence of the reference instead.  The score / softmax / weighted-sum einsums are bf16 torch operations as
+    in the reference: they do not touch FP8 data.
+    """
+
+    fused: bool = True
+
+    def __init__(self, args: ModelArgs):
+        super().__init__()
+        self.dim = args.dim
+        self.n_heads = args.n_heads
+        self.n_local_heads = args.n_heads // world_size
+        self.q_lora_rank = args.q_lora_rank
+        self.kv_lora_rank = args.kv_lora_rank
+        self.qk_nope_head_dim = args.qk_nope_head_dim
+        self.qk_rope_head_dim = args.qk_rope_head_dim
+        self.qk_head_dim = args.qk_nope_head_dim + args.qk_rope_head_dim
+        self.v_head_dim = args.v_head_dim
+        if self.q_lora_rank == 0:
+            self.wq = ColumnParallelLinear(self.dim, self.n_heads * self.qk_head_dim)
+        else:
+            self.wq_a = Linear(self.dim, self.q_lora_rank)
+            self.q_norm = RMSNorm(self.q_lora_rank)
+            self.wq_b = ColumnParallelLinear(self.q_lora_rank, self.n_heads * self.qk_head_dim)
+        self.wkv_a = Linear(self.dim, self.kv_lora_rank + self.qk_rope_head_dim)
+        self.kv_norm = RMSNorm(self.kv_lora_rank)
+        self.wkv_b = ColumnParallelLinear(self.kv_lora_rank, self.n_heads * (self.qk_nope_head_dim + self.v_head_dim))
+        self.wo = RowParallelLinear(self.n_heads * self.v_head_dim, self.dim)
+        self.softmax_scale = self.qk_head_dim ** -0.5
+        if args.max_seq_len > args.original_seq_len:
+            mscale = 0.1 * args.mscale * math.log(args.rope_factor) + 1.0
+            self.softmax_scale = self.softmax_scale * mscale * mscale
+        b, t, h = args.max_batch_size, args.max_seq_len, self.n_local_heads
+        if attn_impl == "naive":
+            self.register_buffer("k_cache", torch.zeros(b, t, h, self.qk_head_dim), persistent=False)
+            self.register_buffer("v_cache", torch.zeros(b, t, h, self.v_head_dim), persistent=False)
+        else:
+            self.register_buffer("kv_cache", torch.zeros(b, t, self.kv_lora_rank), persistent=False)
+            self.register_buffer("pe_cache", torch.zeros(b, t, self.qk_rope_head_dim), persistent=False)
+
+    def _absorb(self, x: torch.Tensor, side: int, wkv_b: Optional[torch.Tensor]) -> torch.Tensor:
+        """One of the two wkv_b products.  ``wkv_b`` is the [h, nope+v, c] bf16 weight for the einsum path, or
+        None to read the FP8 weight in place."""
+        if wkv_b is None:
+            return torch.ops.dsv3fp8.wkv_b_absorb(x, self.wkv_b.weight, self.wkv_b.scale, side,
+                                                  self.qk_nope_head_dim, self.v_head_dim)
+        if side == ops._lib.ABSORB_Q:
+            return torch.einsum("bshd,hdc->bshc", x, wkv_b[:, :self.qk_nope_head_dim])
+        return torch.einsum("bshc,hdc->bshd", x, wkv_b[:, -self.v_head_dim:])
+
+    def forward(self, x: torch.Tensor, start_pos: int, freqs_cis: torch.Tensor, mask: Optional[torch.Tensor]):
+        bsz, seqlen, _ = x.size()
+        end_pos = start_pos + seqlen
+        q = self.wq(x) if self.q_lora_rank == 0 else self.wq_b(self.q_norm(self.wq_a(x)))
+        q = q.view(bsz, seqlen, self.n_local_heads, self.qk_head_dim)
+        q_nope, q_pe = torch.split(q, [self.qk_nope_head_dim, self.qk_rope_head_dim], dim=-1)
+        q_pe = apply_rotary_emb(q_pe, freqs_cis)
+        kv, k_pe = torch.split(self.wkv_a(x), [self.kv_lora_rank, self.qk_rope_head_dim], dim=-1)
+        k_pe = apply_rotary_emb(k_pe.unsqueeze(2), freqs_cis)
+        if attn_impl == "naive":
+            q = torch.cat([q_nope, q_pe], dim=-1)
+            kv = self.wkv_b(self.kv_norm(kv)).view(bsz, seqlen, self.n_local_heads, self.qk_nope_head_dim + self.v_head_dim)
+            k_nope, v = torch.split(kv, [self.qk_nope_head_dim, self.v_head_dim], dim=-1)
+            self.k_cache[:bsz, start_pos:end_pos] = torch.cat([k_nope, k_pe.expand(-1, -1, self.n_local_heads, -1)], dim=-1)
+            self.v_cache[:bsz, start_pos:end_pos] = v
+            scores = torch.einsum("bshd,bthd->bsht", q, self.k_cache[:bsz, :end_pos]) * self.softmax_scale
+        else:
+            w = self.wkv_b.weight
+            if w.element_size() > 1:
+                wkv_b = w.view(self.n_local_heads, -1, self.kv_lora_rank)
+            elif self.fused and x.is_cuda and x.dtype == torch.bfloat16:
+                wkv_b = None
+            else:
+                wkv_b = weight_dequant(w, self.wkv_b.scale, block_size).view(self.n_local_heads, -1, self.kv_lora_rank)
+            q_nope = self._absorb(q_nope, ops._lib.ABSORB_Q, wkv_b)
+            self.kv_cache[:bsz, start_pos:end_pos] = self.kv_norm(kv)
+            self.pe_cache[:bsz, start_pos:end_pos] = k_pe.squeeze(2)
+            scores = (torch.einsum("bshc,btc->bsht", q_nope, self.kv_cache[:bsz, :end_pos]) +
+                      torch.einsum("bshr,btr->bsht", q_pe, self.pe_cache[:bsz, :end_pos])) * self.softmax_scale
+        if mask is not None:
+            scores += mask.unsqueeze(1)
+        scores = scores.softmax(dim=-1, dtype=torch.float32).type_as(x)
+        if attn_impl == "naive":
+            x = torch.einsum("bsht,bthd->bshd", scores, self.v_cache[:bsz, :end_pos])
+        else:
+            x = torch.einsum("bsht,btc->bshc", scores, self.kv_cache[:bsz, :end_pos])
+            x = self._absorb(x, ops._lib.ABSORB_V, wkv_b)
+        return self.wo(x.flatten(2))
 
 
 class MLP(nn.Module):

@@ -1,8 +1,8 @@
 """PyTorch-ROCm custom ops over the C ABI.
 
 ``torch.ops.dsv3fp8.{act_quant, weight_dequant, fp8_gemm}`` and the grouped
-mixture-of-experts ops ``{group_tiles, fp8_gemm_grouped, swiglu_quant, moe_combine}``
-take and return torch tensors; the device implementations hand raw device pointers and the
+mixture-of-experts ops ``{group_tiles, moe_route, fp8_gemm_grouped, swiglu_quant, moe_combine}`` and the
+attention op ``wkv_b_absorb`` take and return torch tensors; the device implementations hand raw device pointers and the
 current HIP stream of the tensors' device to libdsv3fp8.so.  Only a device
 ("CUDA" dispatch key, which is HIP on ROCm) implementation and a shape-only Meta
 implementation are registered: calling an op on CPU tensors raises.
@@ -29,6 +29,7 @@ _libdef.define("fp8_gemm_grouped(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b,
                "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int out_dtype) -> Tensor")
 _libdef.define("swiglu_quant(Tensor h, int block_size, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("moe_combine(Tensor expert_out, Tensor rows, Tensor weights, Tensor? shared) -> Tensor")
+_libdef.define("wkv_b_absorb(Tensor x, Tensor wkv_b, Tensor scale, int side, int nope_dim, int v_dim) -> Tensor")
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -213,8 +214,35 @@ def _moe_combine_meta(expert_out, rows, weights, shared):
     return expert_out.new_empty(rows.size(0), expert_out.size(1))
 
 
+def _absorb_out_dim(wkv_b, side: int, v_dim: int) -> int:
+    return wkv_b.size(1) if side == _lib.ABSORB_Q else v_dim
+
+
+def _wkv_b_absorb_dev(x, wkv_b, scale, side: int, nope_dim: int, v_dim: int):
+    # x: [..., heads, in] bf16, innermost dimension contiguous, leading dimensions collapsible into one token axis
+    # (the q_nope slice of q is such a view); wkv_b: [heads*(nope_dim+v_dim), kv_rank] fp8 with its block scales
+    assert x.dim() >= 2 and x.stride(-1) == 1 and x.dtype == torch.bfloat16
+    assert wkv_b.dim() == 2 and wkv_b.is_contiguous() and scale.is_contiguous() and wkv_b.element_size() == 1
+    heads = x.size(-2)
+    assert wkv_b.size(0) == heads * (nope_dim + v_dim), "wkv_b rows must be heads * (nope_dim + v_dim)"
+    assert x.size(-1) == (nope_dim if side == _lib.ABSORB_Q else wkv_b.size(1))
+    xt = x.view(-1, heads, x.size(-1))
+    y = x.new_empty(*x.size()[:-1], _absorb_out_dim(wkv_b, side, v_dim))
+    with torch.cuda.device(x.device):
+        rc = _lib.lib.dsv3_wkv_b_absorb(xt.data_ptr(), xt.stride(0), xt.stride(1), wkv_b.data_ptr(), scale.data_ptr(),
+                                        y.data_ptr(), _lib.BF16, side, xt.size(0), heads, nope_dim, v_dim,
+                                        wkv_b.size(1), 128, _stream(x))
+    _lib.check(rc, "dsv3_wkv_b_absorb")
+    return y
+
+
+def _wkv_b_absorb_meta(x, wkv_b, scale, side, nope_dim, v_dim):
+    return x.new_empty(*x.size()[:-1], _absorb_out_dim(wkv_b, side, v_dim))
+
+
 _libimpl = torch.library.Library("dsv3fp8", "IMPL")
-for _name, _dev, _meta in (("group_tiles", _group_tiles_dev, _group_tiles_meta),
+for _name, _dev, _meta in (("wkv_b_absorb", _wkv_b_absorb_dev, _wkv_b_absorb_meta),
+                           ("group_tiles", _group_tiles_dev, _group_tiles_meta),
                            ("moe_route", _moe_route_dev, _moe_route_meta),
                            ("fp8_gemm_grouped", _fp8_gemm_grouped_dev, _fp8_gemm_grouped_meta),
                            ("swiglu_quant", _swiglu_quant_dev, _swiglu_quant_meta),

@@ -55,6 +55,12 @@ typedef enum dsv3_scale_fmt {
     DSV3_SCALE_FMT_UE8M0 = 1
 } dsv3_scale_fmt;
 
+/* Which of the two wkv_b products of the absorbed attention dsv3_wkv_b_absorb computes. */
+typedef enum dsv3_absorb_side {
+    DSV3_ABSORB_Q = 0,   /* "bshd,hdc->bshc" with wkv_b[:, :nope]   (inference/model.py:483) */
+    DSV3_ABSORB_V = 1    /* "bshc,hdc->bshd" with wkv_b[:, -v:]     (inference/model.py:495) */
+} dsv3_absorb_side;
+
 /* Library version: major*10000 + minor*100 + patch. */
 int dsv3_version(void);
 
@@ -183,6 +189,24 @@ int dsv3_swiglu_quant(const void* h, int h_dtype, void* y, float* s, int64_t row
  */
 int dsv3_moe_combine(const void* expert_out, int dtype, const int32_t* rows, const void* weights,
                      const void* shared, void* y, int64_t tokens, int topk, int64_t dim, void* stream);
+
+/*
+ * The two per-head products of the absorbed MLA attention with the fp8 weight wkv_b, dequantised in flight
+ * instead of through a weight_dequant call per step (inference/model.py:481-483 and :495):
+ *     W = bf16( f32(wkv_b) * scale[row/128, col/128] )        (what weight_dequant would write, kernel.py:83-86)
+ *     side DSV3_ABSORB_Q:  y[t, h, c] = sum_{d < nope_dim} x[t, h, d] * W[h*(nope_dim+v_dim) + d, c]
+ *     side DSV3_ABSORB_V:  y[t, h, d] = sum_{c < kv_rank}  x[t, h, c] * W[h*(nope_dim+v_dim) + nope_dim + d, c]
+ * accumulated in binary32 and rounded once to `dtype` (DSV3_BF16 only).
+ * x: bf16, element (t, h, j) at x[t*x_token_stride + h*x_head_stride + j] (strides in elements, multiples of 8;
+ * this takes the q_nope view of q without a copy); wkv_b: [heads*(nope_dim+v_dim), kv_rank] e4m3, row-major;
+ * wkv_b_scale: [ceil(rows/128), kv_rank/128]; y: contiguous [tokens, heads, kv_rank] (Q) or [tokens, heads, v_dim] (V).
+ * block_size must be 128; kv_rank % 128 == 0, nope_dim and v_dim multiples of 32; side Q implements nope_dim
+ * 64 and 128, side V kv_rank 128, 256 and 512 (DSV3_ERR_BAD_SHAPE otherwise).  x, wkv_b and y 16-byte aligned.
+ */
+int dsv3_wkv_b_absorb(const void* x, int64_t x_token_stride, int64_t x_head_stride,
+                      const void* wkv_b, const float* wkv_b_scale, void* y, int dtype, int side,
+                      int64_t tokens, int heads, int nope_dim, int v_dim, int64_t kv_rank, int block_size,
+                      void* stream);
 
 #ifdef __cplusplus
 }

@@ -14,10 +14,13 @@ reference checkout).  All arithmetic is IEEE binary32 on the CPU:
 * ``gate``           inference/model.py:566-598
 * ``mlp`` / ``moe``  inference/model.py:532, 633, 669-693
 * ``block_quant_weight`` README_WEIGHTS.md:83-92 (zero padding of ragged blocks)
+* ``wkv_b_absorb``   inference/model.py:481-483, 495 (the two wkv_b products of the absorbed attention)
+* ``rms_norm`` / ``rotary`` / ``mla``  inference/model.py:270-291, 375-392, 456-497
 
 Pinning (see tests/test_oracle_*.py): the conversions and all three kernels are
 checked against the independent plain-C restatement in ``dsv3_oracle.c`` and
-against closed-form known answers; nothing here is "parity unpinned" except the
+against closed-form known answers; ``wkv_b_absorb`` against a scalar triple loop,
+one-hot inputs that read single dequantised weights and exact integer cases; nothing here is "parity unpinned" except the
 choice among equal scores in ``gate`` (torch.topk leaves ties unspecified; the
 workloads are generated without ties).
 """
@@ -180,3 +183,67 @@ def moe(x, weights, indices, experts, shared, scale_fmt=None) -> torch.Tensor:
         y[idx] += mlp(x[idx], *ex, scale_fmt=scale_fmt) * weights[idx, top, None]
     z = mlp(x, *shared)   # the shared expert is an MLP of Column/RowParallelLinear: no scale_fmt (model.py:233,262)
     return (y + z).view(shape)
+
+
+def wkv_b_absorb_f32(x: torch.Tensor, wkv_b: torch.Tensor, scale: torch.Tensor, side: str,
+                     nope_dim: int, v_dim: int) -> torch.Tensor:
+    """model.py:481-483 and :495 with the result left in binary32.  The weight is dequantised to bf16 first
+    (model.py:481, kernel.py:83-86) and viewed as [heads, nope+v, c] (model.py:482);
+    side "q": "bshd,hdc->bshc" with wkv_b[:, :nope]; side "v": "bshc,hdc->bshd" with wkv_b[:, -v:].
+    ``x`` is [..., heads, d or c]."""
+    heads = x.size(-2)
+    w = weight_dequant(wkv_b, scale).float().view(heads, nope_dim + v_dim, wkv_b.size(1))
+    if side == "q":
+        return torch.einsum("...hd,hdc->...hc", x.float(), w[:, :nope_dim])
+    return torch.einsum("...hc,hdc->...hd", x.float(), w[:, -v_dim:])
+
+
+def wkv_b_absorb(x, wkv_b, scale, side: str, nope_dim: int, v_dim: int) -> torch.Tensor:
+    """The bf16 einsum of the reference: binary32 accumulation, one rounding to the dtype of ``x``."""
+    return wkv_b_absorb_f32(x, wkv_b, scale, side, nope_dim, v_dim).to(x.dtype)
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """model.py:291 (F.rms_norm): x * rsqrt(mean(x^2) + eps) * weight, evaluated in binary32."""
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(x.dtype)
+
+
+def rotary(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
+    """model.py:375-392: consecutive pairs of the last dimension times e^{i theta} of the position."""
+    xc = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2))
+    y = torch.view_as_real(xc * freqs_cis.view(1, x.size(1), 1, xc.size(-1))).flatten(3)
+    return y.to(x.dtype)
+
+
+def _bf16_einsum(eq: str, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    return torch.einsum(eq, a.float(), b.float()).to(a.dtype)
+
+
+def mla(x, start_pos: int, freqs_cis, mask, p: dict, kv_cache, pe_cache, n_heads: int, nope_dim: int,
+        rope_dim: int, v_dim: int, kv_rank: int, softmax_scale: float, scale_fmt=None) -> torch.Tensor:
+    """model.py:456-497, the "absorb" branch with a low-rank query (q_lora_rank > 0), at world_size 1.
+    ``p`` maps a layer name to (weight, scale) for the five linears and to the weight for the two norms;
+    the caches are updated in place like the reference's buffers.  Every einsum is a bf16 matmul: binary32
+    accumulation, one rounding."""
+    bsz, seqlen, _ = x.shape
+    end_pos = start_pos + seqlen
+    lin = lambda name, t, fmt=None: linear(t, p[name][0], scale=p[name][1], scale_fmt=fmt)
+    # wq_a and wkv_a are plain Linear layers and take scale_fmt; wq_b, wkv_b, wo are parallel layers and do not
+    q = lin("wq_b", rms_norm(lin("wq_a", x, scale_fmt), p["q_norm"]))
+    q = q.view(bsz, seqlen, n_heads, nope_dim + rope_dim)
+    q_nope, q_pe = torch.split(q, [nope_dim, rope_dim], dim=-1)
+    q_pe = rotary(q_pe, freqs_cis)
+    kv, k_pe = torch.split(lin("wkv_a", x, scale_fmt), [kv_rank, rope_dim], dim=-1)
+    k_pe = rotary(k_pe.unsqueeze(2), freqs_cis)
+    q_nope = wkv_b_absorb(q_nope, p["wkv_b"][0], p["wkv_b"][1], "q", nope_dim, v_dim)
+    kv_cache[:bsz, start_pos:end_pos] = rms_norm(kv, p["kv_norm"])
+    pe_cache[:bsz, start_pos:end_pos] = k_pe.squeeze(2)
+    scores = (_bf16_einsum("bshc,btc->bsht", q_nope, kv_cache[:bsz, :end_pos]) +
+              _bf16_einsum("bshr,btr->bsht", q_pe, pe_cache[:bsz, :end_pos])) * softmax_scale
+    if mask is not None:
+        scores = scores + mask.unsqueeze(1)
+    scores = scores.softmax(dim=-1, dtype=torch.float32).type_as(x)
+    o = _bf16_einsum("bsht,btc->bshc", scores, kv_cache[:bsz, :end_pos])
+    o = wkv_b_absorb(o, p["wkv_b"][0], p["wkv_b"][1], "v", nope_dim, v_dim)
+    return lin("wo", o.flatten(2))

@@ -164,3 +164,27 @@ def test_moe_route_validation(L):
     assert call(2, L.F32) == 5
     assert call(4, 0) == 2 and call(4, 17) == 2 and call(5, 0) == 2 and call(3, -1) == 2
     assert call(0, A16 + 4) == 4
+
+
+def test_wkv_b_absorb_validation(L):
+    f = L.lib.dsv3_wkv_b_absorb
+    #     x    ts        hs   w    ws   y    dtype   side tokens heads nope v   kv_rank block stream
+    ok = [A16, 128 * 192, 192, A16, A16, A16, L.BF16, 0,   4,     128,  128, 128, 512,   128,  None]
+
+    def call(i=None, v=None):
+        a = list(ok)
+        if i is not None:
+            a[i] = v
+        return f(*a)
+    assert call(0, None) == 1 and call(3, None) == 1 and call(4, None) == 1 and call(5, None) == 1
+    assert call(6, L.F32) == 5
+    assert call(13, 64) == 3
+    assert call(7, 2) == 2                         # neither side
+    assert call(10, 32) == 2 and call(10, 96) == 2  # side Q implements nope_dim 64 and 128
+    assert call(12, 500) == 2 and call(11, 100) == 2
+    assert call(2, 100) == 2 and call(1, 12) == 2   # head stride shorter than the row / strides not multiples of 8
+    assert call(0, A16 + 8) == 4 and call(5, A16 + 2) == 4
+    assert call(8, -1) == 2 and call(9, 70000) == 2
+    assert call(8, 0) == 0                           # nothing to do: no launch, no dereference
+    v = list(ok); v[7] = 1; v[12] = 384
+    assert f(*v) == 2                               # side V implements kv_rank 128, 256, 512
