@@ -133,7 +133,37 @@ def run_extras(K, W):
         del wqs
     out["decode"] = dec
     out["moe_layer_T4096"] = run_moe(K, W)
+    out["wkv_b_absorb"] = run_absorb(K, W)
     return out
+
+
+def run_absorb(K, W):
+    """The two wkv_b products of the absorbed attention on the fp8 weight (128 heads, 128 + 128 rows each, rank
+    512), per token count: microseconds of the fused kernels (rotating weight copies, HIP graph) beside the
+    reference's sequence on the same device -- weight_dequant of the whole weight, then two bf16 einsums."""
+    heads, nope, v, c = 128, 128, 128, 512
+    copies = 24                                                # 24 x 16.8 MB > Infinity Cache
+    w8, sc = W.random_fp8_weight(heads * (nope + v), c, 7, "cuda")
+    w8s = [w8.clone() for _ in range(copies)]
+    wd = K.weight_dequant(w8, sc).view(heads, nope + v, c)
+    op = torch.ops.dsv3fp8.wkv_b_absorb
+    res = {}
+    for tokens in (1, 16, 64, 128, 4096):
+        g = torch.Generator(device="cuda").manual_seed(tokens)
+        q = torch.randn(tokens, heads, nope + 64, generator=g, device="cuda").bfloat16()[..., :nope]
+        o = torch.randn(tokens, heads, c, generator=g, device="cuda").bfloat16()
+        n = copies if tokens < 1024 else 6
+        us_q = time_graph([(lambda t=t: op(q, t, sc, 0, nope, v)) for t in w8s[:n]])
+        us_v = time_graph([(lambda t=t: op(o, t, sc, 1, nope, v)) for t in w8s[:n]])
+        us_d = time_graph([(lambda t=t: K.weight_dequant(t, sc)) for t in w8s[:n]])
+        us_e = time_graph([lambda: torch.einsum("mhd,hdc->mhc", q, wd[:, :nope]),
+                           lambda: torch.einsum("mhc,hdc->mhd", o, wd[:, nope:])] * 3) * 2
+        wbytes = heads * 128 * c
+        res[f"T{tokens}"] = {"q_us": round(us_q, 2), "v_us": round(us_v, 2),
+                             "q_GBps": round((wbytes + tokens * heads * (nope + c) * 2) / us_q / 1e3, 1),
+                             "v_GBps": round((wbytes + tokens * heads * (c + v) * 2) / us_v / 1e3, 1),
+                             "dequant_then_einsums_us": round(us_d + us_e, 2)}
+    return res
 
 
 def run_moe(K, W, tokens: int = 4096):

@@ -61,8 +61,9 @@ __device__ __forceinline__ void cvt8(v2u p, float (&f)[8]) {
     }
 }
 
-// side Q; KS = nope / 32 MFMA K steps
-template <int KS>
+// side Q; KS = nope / 32 MFMA K steps; NT: write the output with non-temporal stores (outputs far larger than the
+// last-level cache, which the next kernel could not find there anyway)
+template <int KS, bool NT>
 __global__ __launch_bounds__(256) void absorb_q_kernel(AbsorbArgs p) {
     const int lane = threadIdx.x & 63;
     const int slab = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -132,7 +133,9 @@ __global__ __launch_bounds__(256) void absorb_q_kernel(AbsorbArgs p) {
             v4u o;
 #pragma unroll
             for (int q = 0; q < 4; ++q) o[q] = pack_bf16(acc[2 * q][j], acc[2 * q + 1][j]);
-            *(v4u*)(p.y + (tok * p.heads + h) * p.n_out + c0 + i * 8) = o;
+            v4u* dst = (v4u*)(p.y + (tok * p.heads + h) * p.n_out + c0 + i * 8);
+            if (NT) __builtin_nontemporal_store(o, dst);
+            else *dst = o;
         }
     }
 }
@@ -230,6 +233,141 @@ __global__ __launch_bounds__(256) void absorb_v_kernel(AbsorbArgs p) {
     }
 }
 
+
+// side V for more than 64 tokens, C == 512, v % 128 == 0: same weight slabs and MFMA maps as absorb_v_kernel, but the
+// activations reach the MFMAs through LDS.  Read straight from global memory, a B fragment is 64 pieces of 16
+// bytes from 16 different token rows per load instruction, and each of the four wavefronts of a workgroup
+// fetches the whole 1 KiB row of a token again; that pattern, not HBM, bounds absorb_v_kernel once the weights
+// are amortised.  Here a wavefront's load instruction moves one whole token row (64 lanes x 16 bytes, contiguous)
+// with global_load_lds_dwordx4, each row is fetched once per workgroup, and the fragments come from LDS.
+//
+// LDS: S stages of 16 rows x 1 KiB.  The 16-byte chunk c of row r is stored at chunk position c ^ (r & 15)
+// (the permutation is applied to the global address a lane loads from, since the LDS side of the load is fixed
+// to lane order), which spreads the 16 rows of a ds_read_b128 over all banks.
+//
+// Pipeline per workgroup iteration: wait for the oldest stage's loads (own vmcnt; loads and stores retire in
+// issue order, so the later ones are simply counted), barrier, refill the stage everybody finished reading one
+// iteration ago, read fragments, multiply, store.
+constexpr int kStagedRows = 16, kStagedRowBytes = 1024, kStagedStage = kStagedRows * kStagedRowBytes;
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+__device__ __forceinline__ void wg_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int S>
+__global__ __launch_bounds__(256) void absorb_v_staged_kernel(AbsorbArgs p) {
+    constexpr int KB = 4;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slab = blockIdx.x * 4 + wave;                 // slabs is a multiple of 4 here
+    const int h = blockIdx.y, i = lane & 15, g = lane >> 4;
+    const int d0 = slab * 32;
+    const int64_t row0 = (int64_t)h * p.head_rows + p.nope + d0;
+
+    v4u A[2][KB][4];
+    {
+        v4u raw[2][KB][2];
+        float sc[2][KB];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int64_t r = row0 + (i >> 2) * 8 + t * 4 + (i & 3);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                sc[t][kb] = p.ws[(r >> 7) * p.ws_cols + kb];
+                const v4u* src = (const v4u*)(p.w + r * p.w_cols + kb * 128 + g * 32);
+                raw[t][kb][0] = src[0];
+                raw[t][kb][1] = src[1];
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    float f[8];
+                    cvt8(v2u{raw[t][kb][s >> 1][2 * (s & 1)], raw[t][kb][s >> 1][2 * (s & 1) + 1]}, f);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        A[t][kb][s][q] = pack_bf16(f[2 * q] * sc[t][kb], f[2 * q + 1] * sc[t][kb]);
+                }
+    }
+    // the weight loads above must not be counted among the loads the pipeline waits for
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+
+    const int64_t last = p.tokens - 1;
+    const int gz = gridDim.z;
+    const uint16_t* xh = p.x + (int64_t)h * p.x_hs;
+    // wavefront `wave` moves rows wave, wave+4, wave+8, wave+12 of a tile (one instruction each)
+    auto issue_tile = [&](int ms, int stage) {
+        ms = ms < p.subtiles ? ms : p.subtiles - 1;
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+            const int r = n * 4 + wave;
+            int64_t tok = (int64_t)ms * 16 + r;
+            tok = tok < last ? tok : last;
+            const uint16_t* src = xh + tok * p.x_ts + ((lane ^ r) << 3);      // r < 16: permutes the low 4 chunk bits
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + stage * kStagedStage + r * kStagedRowBytes),
+                                             16, 0, 0);
+        }
+    };
+    // fragment (kb, s) of the lane: row i, chunk kb*16 + g*4 + s
+    const uint8_t* frag = lds + i * kStagedRowBytes;
+    int frag_off[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) frag_off[s] = (((g * 4 + s) ^ i) << 4);
+
+    int ms = blockIdx.z;
+#pragma unroll
+    for (int t = 0; t < S - 1; ++t) issue_tile(ms + t * gz, t);
+    int stage = 0;
+    for (int it = 0; ms < p.subtiles; ms += gz, ++it) {
+        // outstanding after the loads of this tile: the loads of the S-2 tiles behind it, and (once the
+        // pipeline runs) one store per iteration since they were issued
+        if (it < S - 1) __builtin_amdgcn_s_waitcnt(0x0f70 | (4 * (S - 2)));
+        else            __builtin_amdgcn_s_waitcnt(0x0f70 | (4 * (S - 2) + (S - 1)));
+        wg_barrier();
+        issue_tile(ms + (S - 1) * gz, stage == 0 ? S - 1 : stage - 1);
+        const uint8_t* st = frag + stage * kStagedStage;
+        v4f acc[2][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) acc[t][0] = acc[t][1] = v4f{0.f, 0.f, 0.f, 0.f};
+        v4u b[2][4];                                  // K block kb+1 is read while kb feeds the MFMAs
+#pragma unroll
+        for (int s = 0; s < 4; ++s) b[0][s] = *(const v4u*)(st + frag_off[s]);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            if (kb + 1 < KB) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) b[(kb + 1) & 1][s] = *(const v4u*)(st + (kb + 1) * 256 + frag_off[s]);
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) acc[t][s & 1] = mfma_bf16(A[t][kb][s], b[kb & 1][s], acc[t][s & 1]);
+        }
+        // keep the order written above (the scheduler otherwise sinks every read next to its use and waits for
+        // each pair): 4 reads ahead, then per K block the next 4 reads followed by its 8 MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            if (kb + 1 < KB) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        }
+        int64_t tok = (int64_t)ms * 16 + i;
+        tok = tok < last ? tok : last;
+        v4u o;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const v4f r = acc[t][0] + acc[t][1];
+            o[2 * t] = pack_bf16(r[0], r[1]);
+            o[2 * t + 1] = pack_bf16(r[2], r[3]);
+        }
+        *(v4u*)(p.y + (tok * p.heads + h) * p.n_out + d0 + g * 8) = o;
+        stage = stage + 1 == S ? 0 : stage + 1;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);     // the clamped refills of the last iterations still write LDS
+}
+
 }  // namespace
 
 bool wkv_b_absorb_supported(int side, int nope, int v, int64_t kv_rank) {
@@ -258,9 +396,26 @@ int launch_wkv_b_absorb(const void* x, int64_t x_ts, int64_t x_hs, const void* w
     gz = gz > p.subtiles ? p.subtiles : gz;
     gz = gz > 65535 ? 65535 : gz;
     const dim3 grid(gx, heads, gz), block(64 * waves);
+    if (!q && kv_rank == 512 && v % 128 == 0 && waves == 4) {
+        constexpr int S = 4;
+        static bool granted[64];                 // 64 KiB of dynamic LDS needs the opt-in once per device
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
+        if (!granted[dev]) {
+            if (hipFuncSetAttribute((const void*)absorb_v_staged_kernel<S>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    S * kStagedStage) != hipSuccess)
+                return DSV3_ERR_LAUNCH;
+            granted[dev] = true;
+        }
+        hipLaunchKernelGGL(absorb_v_staged_kernel<S>, grid, block, S * kStagedStage, st, p);
+        return launch_status();
+    }
     if (q) {
-        if (nope == 128) hipLaunchKernelGGL(absorb_q_kernel<4>, grid, block, 0, st, p);
-        else hipLaunchKernelGGL(absorb_q_kernel<2>, grid, block, 0, st, p);
+        const bool nt = tokens * heads * kv_rank * 2 > (int64_t)256 << 20;
+        if (nope == 128 && nt) hipLaunchKernelGGL((absorb_q_kernel<4, true>), grid, block, 0, st, p);
+        else if (nope == 128) hipLaunchKernelGGL((absorb_q_kernel<4, false>), grid, block, 0, st, p);
+        else if (nt) hipLaunchKernelGGL((absorb_q_kernel<2, true>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((absorb_q_kernel<2, false>), grid, block, 0, st, p);
     } else {
         if (kv_rank == 512) hipLaunchKernelGGL(absorb_v_kernel<4>, grid, block, 0, st, p);
         else if (kv_rank == 256) hipLaunchKernelGGL(absorb_v_kernel<2>, grid, block, 0, st, p);

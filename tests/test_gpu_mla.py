@@ -55,7 +55,8 @@ def test_absorb_671b_shape(K, tokens, side):
     _check(y, x, w8, s, side, nope, v)
 
 
-@pytest.mark.parametrize("heads,nope,v,c", [(3, 64, 32, 128), (5, 64, 64, 256), (2, 128, 32, 512), (1, 128, 96, 384)])
+@pytest.mark.parametrize("heads,nope,v,c", [(3, 64, 32, 128), (5, 64, 64, 256), (2, 128, 32, 512), (1, 128, 96, 384),
+                                             (3, 64, 128, 512)])
 def test_absorb_other_shapes(K, heads, nope, v, c):
     """Heads whose row ranges straddle 128-row scale blocks (nope + v not a multiple of 128)."""
     w8, s = _wkv_b(heads, nope, v, c, 11)
