@@ -137,7 +137,7 @@ def run_extras(K, W):
     return out
 
 
-def run_absorb(K, W):
+def run_absorb(K, W, token_counts=(1, 16, 64, 128, 4096)):
     """The two wkv_b products of the absorbed attention on the fp8 weight (128 heads, 128 + 128 rows each, rank
     512), per token count: microseconds of the fused kernels (rotating weight copies, HIP graph) beside the
     reference's sequence on the same device -- weight_dequant of the whole weight, then two bf16 einsums."""
@@ -148,7 +148,7 @@ def run_absorb(K, W):
     wd = K.weight_dequant(w8, sc).view(heads, nope + v, c)
     op = torch.ops.dsv3fp8.wkv_b_absorb
     res = {}
-    for tokens in (1, 16, 64, 128, 4096):
+    for tokens in token_counts:
         g = torch.Generator(device="cuda").manual_seed(tokens)
         q = torch.randn(tokens, heads, nope + 64, generator=g, device="cuda").bfloat16()[..., :nope]
         o = torch.randn(tokens, heads, c, generator=g, device="cuda").bfloat16()
@@ -232,6 +232,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only-absorb", type=int, default=0, metavar="TOKENS",
+                    help="profiling aid: run only the wkv_b_absorb leg at this token count and print its JSON")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known HBM traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled")
@@ -246,6 +248,13 @@ def main():
     from dsv3fp8 import workloads as W
     torch.set_default_dtype(torch.bfloat16)  # as the reference's caller does (generate.py:109)
     torch.cuda.set_device(0)
+    if args.only_absorb:
+        if args.copy_calibration:
+            src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+            torch.empty_like(src).copy_(src)
+            torch.cuda.synchronize()
+        print(json.dumps({"wkv_b_absorb": run_absorb(K, W, (args.only_absorb,))}), flush=True)
+        return
 
     M = W.PREFILL_M
     k, n = W.PREFILL_SHAPES["w1"]
