@@ -216,12 +216,16 @@ def cpu_baseline(W, rows: int = 1024):
     x = W.activations(rows, 7168, 0, "cpu")
     w8, ws = W.weight(18432, 7168, 1, "cpu")
     oracle.linear(x[:64], w8, scale=ws)                      # warm-up
-    t0 = time.perf_counter()
-    oracle.linear(x, w8, scale=ws)
-    dt = time.perf_counter() - t0
-    return {"value": round(2 * rows * 18432 * 7168 / dt / 1e12, 4), "unit": "TFLOP/s",
+    passes, t0 = 0, time.perf_counter()
+    while True:                                              # whole passes over the sample until >= 10 s of CPU work
+        oracle.linear(x, w8, scale=ws)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt >= 10.0 or passes >= 8:
+            break
+    return {"value": round(2 * rows * passes * 18432 * 7168 / dt / 1e12, 4), "unit": "TFLOP/s",
             "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"oracle.linear() (act_quant + fp8_gemm, fp32 torch-CPU) on {rows} of 4096 rows, "
+            "sample": f"oracle.linear() (act_quant + fp8_gemm, fp32 torch-CPU), {passes} passes over {rows} of 4096 rows, "
                       f"K=7168 -> N=18432, {dt:.2f} s"}
 
 

@@ -149,6 +149,23 @@ int dsv3_moe_combine(const void* expert_out, int dtype, const int32_t* rows, con
     return launch_moe_combine(expert_out, rows, weights, shared, y, tokens, topk, dim, (hipStream_t)stream);
 }
 
+int dsv3_gate_route(const void* logits, int dtype, const float* bias, void* weights, int64_t* indices,
+                    int64_t tokens, int experts, int topk, int n_groups, int topk_groups, int score_func,
+                    float route_scale, void* stream) {
+    if (dtype != DSV3_BF16) return DSV3_ERR_BAD_DTYPE;
+    if (score_func != DSV3_SCORE_SOFTMAX && score_func != DSV3_SCORE_SIGMOID) return DSV3_ERR_BAD_DTYPE;
+    if (tokens < 0 || tokens > 0x7fffffff || experts < 1 || experts > 512 || topk < 1 || topk > 64 || topk > experts)
+        return DSV3_ERR_BAD_SHAPE;
+    if (n_groups < 1 || n_groups > 64 || experts % n_groups != 0 || topk_groups < 1 || topk_groups > n_groups ||
+        (int64_t)topk_groups * (experts / n_groups) < topk)
+        return DSV3_ERR_BAD_SHAPE;
+    if (tokens == 0) return DSV3_OK;
+    if (!logits || !weights || !indices) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(logits, 2) || !aligned(weights, 2) || !aligned(indices, 8) || !aligned(bias, 4)) return DSV3_ERR_MISALIGNED;
+    return launch_gate_route(logits, bias, weights, indices, tokens, experts, topk, n_groups, topk_groups, score_func,
+                             route_scale, (hipStream_t)stream);
+}
+
 int dsv3_wkv_b_absorb(const void* x, int64_t x_token_stride, int64_t x_head_stride,
                       const void* wkv_b, const float* wkv_b_scale, void* y, int dtype, int side,
                       int64_t tokens, int heads, int nope_dim, int v_dim, int64_t kv_rank, int block_size,

@@ -97,6 +97,9 @@ int launch_moe_route(const int64_t* indices, const void* weights, int64_t tokens
                      void* w_sorted, int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st);
 int launch_group_tiles(const int* counts, int groups, int tile_rows, int max_tiles,
                        int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st);
+int launch_gate_route(const void* logits, const float* bias, void* weights, int64_t* indices, int64_t tokens,
+                      int experts, int topk, int n_groups, int topk_groups, int score_func, float route_scale,
+                      hipStream_t st);
 bool wkv_b_absorb_supported(int side, int nope, int v, int64_t kv_rank);
 int launch_wkv_b_absorb(const void* x, int64_t x_ts, int64_t x_hs, const void* w, const float* ws, void* y, int side,
                         int64_t tokens, int heads, int nope, int v, int64_t kv_rank, hipStream_t st);

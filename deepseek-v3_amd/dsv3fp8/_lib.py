@@ -6,7 +6,7 @@ has not been built the import fails with the command that builds it.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent.parent / "lib" / "libdsv3fp8.so"
@@ -15,6 +15,7 @@ LIB_PATH = Path(__file__).resolve().parent.parent / "lib" / "libdsv3fp8.so"
 BF16, F16, F32 = 0, 1, 2
 SCALE_FMT_NONE, SCALE_FMT_UE8M0 = 0, 1
 ABSORB_Q, ABSORB_V = 0, 1
+SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
 OK = 0
 
 EXPORTS = {
@@ -35,6 +36,8 @@ EXPORTS = {
     "dsv3_swiglu_quant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]),
     "dsv3_moe_combine": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int64, c_int, c_int64, c_void_p]),
+    "dsv3_gate_route": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
+                                c_int, c_float, c_void_p]),
     "dsv3_wkv_b_absorb": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                   c_int64, c_int, c_int, c_int, c_int64, c_int, c_void_p]),
 }

@@ -303,8 +303,21 @@ class Gate(nn.Module):
         self.weight = nn.Parameter(torch.empty(args.n_routed_experts, args.dim))
         self.bias = nn.Parameter(torch.empty(args.n_routed_experts, dtype=torch.float32)) if self.dim == 7168 else None
 
+    fused: bool = True
+
+    def _fused_ok(self, scores: torch.Tensor) -> bool:
+        experts = scores.size(-1)
+        return (self.fused and scores.is_cuda and scores.dtype == torch.bfloat16 and experts <= 512
+                and self.topk <= min(64, experts) and self.n_groups <= 64 and experts % self.n_groups == 0
+                and self.topk <= self.topk_groups * (experts // self.n_groups))
+
     def forward(self, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         scores = linear(x, self.weight)
+        if self._fused_ok(scores):
+            # everything after the linear layer in one launch (the tensor-op sequence below is what it computes)
+            func = ops._lib.SCORE_SOFTMAX if self.score_func == "softmax" else ops._lib.SCORE_SIGMOID
+            return torch.ops.dsv3fp8.gate_route(scores.contiguous(), self.bias, self.topk, self.n_groups,
+                                                self.topk_groups, func, float(self.route_scale))
         scores = scores.softmax(dim=-1, dtype=torch.float32) if self.score_func == "softmax" else scores.sigmoid()
         unbiased = scores
         if self.bias is not None:

@@ -1,7 +1,7 @@
 """PyTorch-ROCm custom ops over the C ABI.
 
 ``torch.ops.dsv3fp8.{act_quant, weight_dequant, fp8_gemm}`` and the grouped
-mixture-of-experts ops ``{group_tiles, moe_route, fp8_gemm_grouped, swiglu_quant, moe_combine}`` and the
+mixture-of-experts ops ``{gate_route, group_tiles, moe_route, fp8_gemm_grouped, swiglu_quant, moe_combine}`` and the
 attention op ``wkv_b_absorb`` take and return torch tensors; the device implementations hand raw device pointers and the
 current HIP stream of the tensors' device to libdsv3fp8.so.  Only a device
 ("CUDA" dispatch key, which is HIP on ROCm) implementation and a shape-only Meta
@@ -29,6 +29,8 @@ _libdef.define("fp8_gemm_grouped(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b,
                "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int out_dtype) -> Tensor")
 _libdef.define("swiglu_quant(Tensor h, int block_size, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("moe_combine(Tensor expert_out, Tensor rows, Tensor weights, Tensor? shared) -> Tensor")
+_libdef.define("gate_route(Tensor logits, Tensor? bias, int topk, int n_groups, int topk_groups, int score_func, "
+               "float route_scale) -> (Tensor, Tensor)")
 _libdef.define("wkv_b_absorb(Tensor x, Tensor wkv_b, Tensor scale, int side, int nope_dim, int v_dim) -> Tensor")
 
 
@@ -214,6 +216,24 @@ def _moe_combine_meta(expert_out, rows, weights, shared):
     return expert_out.new_empty(rows.size(0), expert_out.size(1))
 
 
+def _gate_route_dev(logits, bias, topk: int, n_groups: int, topk_groups: int, score_func: int, route_scale: float):
+    assert logits.dim() == 2 and logits.is_contiguous() and logits.dtype == torch.bfloat16
+    assert bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == logits.size(1))
+    tokens, experts = logits.shape
+    weights = logits.new_empty(tokens, topk)
+    indices = torch.empty(tokens, topk, dtype=torch.int64, device=logits.device)
+    with torch.cuda.device(logits.device):
+        rc = _lib.lib.dsv3_gate_route(logits.data_ptr(), _lib.BF16, bias.data_ptr() if bias is not None else None,
+                                      weights.data_ptr(), indices.data_ptr(), tokens, experts, topk, n_groups,
+                                      topk_groups, score_func, route_scale, _stream(logits))
+    _lib.check(rc, "dsv3_gate_route")
+    return weights, indices
+
+
+def _gate_route_meta(logits, bias, topk, n_groups, topk_groups, score_func, route_scale):
+    return logits.new_empty(logits.size(0), topk), logits.new_empty(logits.size(0), topk, dtype=torch.int64)
+
+
 def _absorb_out_dim(wkv_b, side: int, v_dim: int) -> int:
     return wkv_b.size(1) if side == _lib.ABSORB_Q else v_dim
 
@@ -242,6 +262,7 @@ def _wkv_b_absorb_meta(x, wkv_b, scale, side, nope_dim, v_dim):
 
 _libimpl = torch.library.Library("dsv3fp8", "IMPL")
 for _name, _dev, _meta in (("wkv_b_absorb", _wkv_b_absorb_dev, _wkv_b_absorb_meta),
+                           ("gate_route", _gate_route_dev, _gate_route_meta),
                            ("group_tiles", _group_tiles_dev, _group_tiles_meta),
                            ("moe_route", _moe_route_dev, _moe_route_meta),
                            ("fp8_gemm_grouped", _fp8_gemm_grouped_dev, _fp8_gemm_grouped_meta),

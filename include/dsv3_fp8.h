@@ -61,6 +61,12 @@ typedef enum dsv3_absorb_side {
     DSV3_ABSORB_V = 1    /* "bshc,hdc->bshd" with wkv_b[:, -v:]     (inference/model.py:495) */
 } dsv3_absorb_side;
 
+/* score_func of the router (inference/model.py:578-581). */
+typedef enum dsv3_score_func {
+    DSV3_SCORE_SOFTMAX = 0,
+    DSV3_SCORE_SIGMOID = 1
+} dsv3_score_func;
+
 /* Library version: major*10000 + minor*100 + patch. */
 int dsv3_version(void);
 
@@ -189,6 +195,22 @@ int dsv3_swiglu_quant(const void* h, int h_dtype, void* y, float* s, int64_t row
  */
 int dsv3_moe_combine(const void* expert_out, int dtype, const int32_t* rows, const void* weights,
                      const void* shared, void* y, int64_t tokens, int topk, int64_t dim, void* stream);
+
+/*
+ * Expert selection of the router, everything after its linear layer (inference/model.py:577-598):
+ *     s = sigmoid(logits) rounded to bf16, or softmax(logits) in binary32;   sel = s + bias (binary32, bias optional)
+ *     n_groups > 1: a group scores the sum of its two largest sel (with bias) or its largest (without); experts
+ *                   outside the topk_groups best groups are masked to -inf
+ *     indices = the topk largest sel in descending order (ties: lower index);   w = s[indices]
+ *     sigmoid: w = bf16(w / bf16(sum w));   weights = bf16(w * route_scale)
+ * logits: [tokens, experts] of `dtype` (DSV3_BF16 only), the output of the router's linear layer; bias: fp32
+ * [experts] or NULL; weights: bf16 [tokens, topk]; indices: int64 [tokens, topk].
+ * 1 <= topk <= 64, topk <= experts <= 512, experts % n_groups == 0, n_groups <= 64,
+ * topk <= topk_groups * (experts / n_groups).
+ */
+int dsv3_gate_route(const void* logits, int dtype, const float* bias, void* weights, int64_t* indices,
+                    int64_t tokens, int experts, int topk, int n_groups, int topk_groups, int score_func,
+                    float route_scale, void* stream);
 
 /*
  * The two per-head products of the absorbed MLA attention with the fp8 weight wkv_b, dequantised in flight

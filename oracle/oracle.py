@@ -141,10 +141,10 @@ def mlp(x, w1, s1, w2, s2, w3, s3, scale_fmt=None) -> torch.Tensor:
     return linear(h, w2, scale=s2, scale_fmt=scale_fmt)
 
 
-def gate(x, gate_weight, gate_bias, topk: int, n_groups: int, topk_groups: int,
-         route_scale: float, score_func: str = "sigmoid"):
-    """model.py:576-598."""
-    scores = F.linear(x, gate_weight)
+def gate_route(scores, gate_bias, topk: int, n_groups: int, topk_groups: int,
+               route_scale: float, score_func: str = "sigmoid"):
+    """model.py:577-598: everything after the router's linear layer.  ``scores`` is its output [tokens, experts]."""
+    tokens = scores.size(0)
     if score_func == "softmax":
         scores = scores.softmax(dim=-1, dtype=torch.float32)
     else:
@@ -153,19 +153,27 @@ def gate(x, gate_weight, gate_bias, topk: int, n_groups: int, topk_groups: int,
     if gate_bias is not None:
         scores = scores + gate_bias
     if n_groups > 1:
-        scores = scores.view(x.size(0), n_groups, -1)
+        scores = scores.view(tokens, n_groups, -1)
         if gate_bias is None:
             group_scores = scores.amax(dim=-1)
         else:
             group_scores = scores.topk(2, dim=-1)[0].sum(dim=-1)
         idx = group_scores.topk(topk_groups, dim=-1)[1]
-        mask = torch.ones(x.size(0), n_groups, dtype=torch.bool).scatter_(1, idx, False)
+        mask = torch.ones(tokens, n_groups, dtype=torch.bool).scatter_(1, idx, False)
         scores = scores.masked_fill(mask.unsqueeze(-1), float("-inf")).flatten(1)
     indices = torch.topk(scores, topk, dim=-1)[1]
     weights = original.gather(1, indices)
     if score_func == "sigmoid":
         weights = weights / weights.sum(dim=-1, keepdim=True)
     weights = weights * route_scale
+    return weights, indices
+
+
+def gate(x, gate_weight, gate_bias, topk: int, n_groups: int, topk_groups: int,
+         route_scale: float, score_func: str = "sigmoid"):
+    """model.py:576-598."""
+    weights, indices = gate_route(F.linear(x, gate_weight), gate_bias, topk, n_groups, topk_groups, route_scale,
+                                  score_func)
     return weights.type_as(x), indices
 
 

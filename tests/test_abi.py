@@ -188,3 +188,24 @@ def test_wkv_b_absorb_validation(L):
     assert call(8, 0) == 0                           # nothing to do: no launch, no dereference
     v = list(ok); v[7] = 1; v[12] = 384
     assert f(*v) == 2                               # side V implements kv_rank 128, 256, 512
+
+
+def test_gate_route_validation(L):
+    f = L.lib.dsv3_gate_route
+    #     logits dtype   bias  w    idx  tokens experts topk groups topk_groups func scale stream
+    ok = [A16,   L.BF16, None, A16, A16, 4,     256,    8,   8,     4,          1,   2.5,  None]
+
+    def call(i=None, v=None):
+        a = list(ok)
+        if i is not None:
+            a[i] = v
+        return f(*a)
+    assert call(0, None) == 1 and call(3, None) == 1 and call(4, None) == 1
+    assert call(1, L.F32) == 5 and call(10, 2) == 5
+    assert call(6, 513) == 2 and call(7, 0) == 2 and call(7, 65) == 2 and call(5, -1) == 2
+    assert call(8, 7) == 2                          # experts not divisible by the number of groups
+    assert call(9, 9) == 2 and call(9, 0) == 2
+    a = list(ok); a[8], a[9], a[7] = 64, 1, 8       # one group of 4 experts cannot supply 8
+    assert f(*a) == 2
+    assert call(0, A16 + 1) == 4 and call(4, A16 + 4) == 4
+    assert call(5, 0) == 0
