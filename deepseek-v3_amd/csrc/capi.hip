@@ -90,16 +90,18 @@ int dsv3_group_tiles(const int32_t* counts, int groups, int max_tiles,
 }
 
 int dsv3_moe_route(const int64_t* indices, const void* weights, int w_dtype, int64_t tokens, int topk, int experts,
-                   int max_tiles, int32_t* scratch, int32_t* a_rows, int32_t* rows, void* w_sorted,
+                   int shared_group, int max_tiles, int32_t* scratch, int32_t* a_rows, int32_t* rows, void* w_sorted,
                    int32_t* tile_group, int32_t* tile_row0, int32_t* tile_rows, void* stream) {
     if (w_dtype != DSV3_BF16 && w_dtype != DSV3_F16) return DSV3_ERR_BAD_DTYPE;       // any 2-byte type: values are only moved
     if (tokens < 0 || topk < 1 || topk > 16 || experts < 1 || experts > 8192 || max_tiles < 0) return DSV3_ERR_BAD_SHAPE;
-    if (tokens * topk > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (tokens * (topk + 1) > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (!scratch || (max_tiles > 0 && (!tile_group || !tile_row0 || !tile_rows))) return DSV3_ERR_NULL_POINTER;
     if (tokens > 0 && (!indices || !weights || !a_rows || !rows || !w_sorted)) return DSV3_ERR_NULL_POINTER;
     if (!aligned(indices, 8) || !aligned(weights, 2) || !aligned(w_sorted, 2)) return DSV3_ERR_MISALIGNED;
-    return launch_moe_route(indices, weights, tokens, topk, experts, max_tiles, grouped_tile_rows(),
-                            scratch, scratch + experts, scratch + 2 * (int64_t)experts, a_rows, rows, w_sorted,
+    const int groups = experts + (shared_group ? 1 : 0);
+    const int one = shared_group ? (w_dtype == DSV3_BF16 ? 0x3F80 : 0x3C00) : 0;     // 1.0 in the weights' type
+    return launch_moe_route(indices, weights, tokens, topk, experts, one, max_tiles, grouped_tile_rows(),
+                            scratch, scratch + groups, scratch + 2 * (int64_t)groups, a_rows, rows, w_sorted,
                             tile_group, tile_row0, tile_rows, (hipStream_t)stream);
 }
 

@@ -93,8 +93,8 @@ int launch_swiglu_quant(const void* h, void* y, float* s, int64_t rows, int64_t 
 int launch_moe_combine(const void* out, const int* rows, const void* w, const void* shared, void* y,
                        int64_t tokens, int topk, int64_t dim, hipStream_t st);
 int launch_moe_route(const int64_t* indices, const void* weights, int64_t tokens, int topk, int experts,
-                     int max_tiles, int tile_rows, int* counts, int* offsets, int* cursor, int* a_rows, int* rows,
-                     void* w_sorted, int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st);
+                     int shared_one, int max_tiles, int tile_rows, int* counts, int* offsets, int* cursor, int* a_rows,
+                     int* rows, void* w_sorted, int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st);
 int launch_group_tiles(const int* counts, int groups, int tile_rows, int max_tiles,
                        int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st);
 int launch_gate_route(const void* logits, const float* bias, void* weights, int64_t* indices, int64_t tokens,

@@ -14,31 +14,40 @@
 namespace dsv3 {
 namespace {
 
-struct Best { float v; int i; };
-
-__device__ __forceinline__ Best better(Best a, Best b) {
-    return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
+// Wavefront-wide reductions that leave the result in every lane: four DPP steps inside each row of 16 lanes
+// (no LDS traffic), then two cross-row exchanges.
+template <int CTRL> __device__ __forceinline__ int dpp_mov(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
 }
-// largest value over the wavefront, lowest index among equals; every lane gets the result
-__device__ __forceinline__ Best wave_argmax(Best x) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        Best o;
-        o.v = __shfl_xor(x.v, d, 64);
-        o.i = __shfl_xor(x.i, d, 64);
-        x = better(x, o);
-    }
-    return x;
-}
-__device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) x += __shfl_xor(x, d, 64);
-    return x;
+template <class Op> __device__ __forceinline__ int wave_reduce(int v, Op op) {
+    v = op(v, dpp_mov<0xB1>(v));      // quad_perm [1,0,3,2]
+    v = op(v, dpp_mov<0x4E>(v));      // quad_perm [2,3,0,1]
+    v = op(v, dpp_mov<0x141>(v));     // row_half_mirror
+    v = op(v, dpp_mov<0x140>(v));     // row_mirror
+    v = op(v, __shfl_xor(v, 16, 64));
+    v = op(v, __shfl_xor(v, 32, 64));
+    return v;
 }
 __device__ __forceinline__ float wave_max(float x) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) x = fmaxf(x, __shfl_xor(x, d, 64));
-    return x;
+    return __builtin_bit_cast(float, wave_reduce(__builtin_bit_cast(int, x), [](int a, int b) {
+        return __builtin_bit_cast(int, fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b))); }));
+}
+__device__ __forceinline__ float wave_sum(float x) {
+    return __builtin_bit_cast(float, wave_reduce(__builtin_bit_cast(int, x), [](int a, int b) {
+        return __builtin_bit_cast(int, __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b)); }));
+}
+__device__ __forceinline__ int wave_min(int x) { return wave_reduce(x, [](int a, int b) { return a < b ? a : b; }); }
+
+struct Best { float v; int i; };
+// largest value over the wavefront, lowest index among equals; every lane gets the result
+__device__ __forceinline__ Best wave_argmax(Best x) {
+    Best r;
+    r.v = wave_max(x.v);
+    r.i = wave_min(x.v == r.v ? x.i : 0x7fffffff);
+    return r;
+}
+__device__ __forceinline__ Best better(Best a, Best b) {
+    return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
 }
 __device__ __forceinline__ float round_bf16(float x) { return bf16lo_to_f32(pack_bf16(x, 0.f) & 0xffffu); }
 
@@ -120,13 +129,15 @@ __global__ __launch_bounds__(64 * kTokensPerWg) void gate_route_kernel(
             if (e < experts) loc = better(loc, Best{ sel[s], e });
         }
         const Best b = wave_argmax(loc);
-        float w = 0.f;
+        // the winner's unbiased score: slot b.i / 64 of lane b.i % 64, fetched with a lane read (b is uniform)
+        const int win = __builtin_amdgcn_readfirstlane(b.i);
+        float cand = 0.f;
 #pragma unroll
-        for (int s = 0; s < EPL; ++s)
-            if (s * 64 + lane == b.i) { w = orig[s]; sel[s] = ninf; }
-        // the owner holds w, every other lane 0: the sum is a broadcast.  A winner at -inf (fewer finite
-        // candidates than topk) was cleared before and is returned again, like any tie.
-        w = wave_sum(w);
+        for (int s = 0; s < EPL; ++s) {
+            if (s == (win >> 6)) cand = orig[s];
+            if (s * 64 + lane == win) sel[s] = ninf;
+        }
+        const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cand), win & 63));
         if (lane == t) my_w = w;
         if (lane == 0) idx_out[(int64_t)token * topk + t] = b.i;
     }

@@ -76,47 +76,61 @@ __global__ __launch_bounds__(kThreads) void swiglu_quant_kernel(
     }
 }
 
-// One workgroup per token.  rows[t, k] is the row of `out` holding the token's k-th expert output in ascending
-// expert order, w[t, k] the matching routing weight (bf16).
+// One thread per 16-byte chunk of a token's output row (grid: tokens x chunk blocks).  rows[t, k] is the row of
+// `out` holding the token's k-th expert output in ascending expert order, w[t, k] the matching routing weight
+// (bf16).  The additions are a dependent chain of bf16 roundings, the loads are not: four experts' chunks are
+// fetched before they are added.
 __global__ __launch_bounds__(kThreads) void moe_combine_kernel(
         const v4u* __restrict__ out, const int* __restrict__ rows, const uint16_t* __restrict__ w,
         const v4u* __restrict__ shared, v4u* __restrict__ y, int topk, int chunks_per_row) {
     const int t = blockIdx.x;
-    for (int c = threadIdx.x; c < chunks_per_row; c += kThreads) {
-        float acc[8];
+    const int c = blockIdx.y * kThreads + threadIdx.x;
+    if (c >= chunks_per_row) return;
+    float acc[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-        for (int k = 0; k < topk; ++k) {
-            const int r = rows[t * topk + k];
-            const float wk = bf16lo_to_f32(w[t * topk + k]);
-            const v4u v = out[(int64_t)r * chunks_per_row + c];
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    v4u z = {0u, 0u, 0u, 0u};
+    if (shared) z = shared[(int64_t)t * chunks_per_row + c];
+    for (int k0 = 0; k0 < topk; k0 += 4) {
+        v4u v[4];
+        float wk[4];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float x = (i & 1) ? bf16hi_to_f32(v[i >> 1]) : bf16lo_to_f32(v[i >> 1]);
-                acc[i] = round_bf16(acc[i] + round_bf16(x * wk));       // y[idx] += expert_out * weight
+        for (int u = 0; u < 4; ++u) {
+            const int k = min(k0 + u, topk - 1);
+            wk[u] = bf16lo_to_f32(w[t * topk + k]);
+            v[u] = out[(int64_t)rows[t * topk + k] * chunks_per_row + c];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (k0 + u < topk) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float x = (i & 1) ? bf16hi_to_f32(v[u][i >> 1]) : bf16lo_to_f32(v[u][i >> 1]);
+                    acc[i] = round_bf16(acc[i] + round_bf16(x * wk[u]));       // y[idx] += expert_out * weight
+                }
             }
         }
-        if (shared) {
-            const v4u z = shared[(int64_t)t * chunks_per_row + c];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float x = (i & 1) ? bf16hi_to_f32(z[i >> 1]) : bf16lo_to_f32(z[i >> 1]);
-                acc[i] = round_bf16(acc[i] + x);                         // y + z
-            }
-        }
-        v4u o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = pack_bf16(acc[2 * i], acc[2 * i + 1]);
-        y[(int64_t)t * chunks_per_row + c] = o;
     }
+    if (shared) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float x = (i & 1) ? bf16hi_to_f32(z[i >> 1]) : bf16lo_to_f32(z[i >> 1]);
+            acc[i] = round_bf16(acc[i] + x);                                     // y + z
+        }
+    }
+    v4u o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = pack_bf16(acc[2 * i], acc[2 * i + 1]);
+    y[(int64_t)t * chunks_per_row + c] = o;
 }
 
 // counts[g] rows per group, groups laid out back to back in c.  Tile slots are handed out group by group,
-// ceil(count / tile_rows) each; slots past the last one are marked unused.  One workgroup, any group count.
-__global__ __launch_bounds__(kThreads) void group_tiles_kernel(
-        const int* __restrict__ counts, int groups, int tile_rows, int max_tiles,
+// ceil(count / tile_rows) each; slots past the last one are marked unused.  Called by every thread of ONE workgroup
+// of kThreads threads; counts and offsets may live in LDS or in global memory.
+__device__ __forceinline__ void tiles_from_counts(
+        const int* counts, int groups, int tile_rows, int max_tiles,
         int* __restrict__ tile_group, int* __restrict__ tile_row0, int* __restrict__ tile_nrows,
-        int* __restrict__ offsets) {           // optional: first row of every group
+        int* offsets) {                        // optional: first row of every group
     __shared__ int tile_base[kThreads + 1], row_base[kThreads + 1];
     int done_tiles = 0, done_rows = 0;
     for (int g0 = 0; g0 < groups; g0 += kThreads) {
@@ -151,6 +165,13 @@ __global__ __launch_bounds__(kThreads) void group_tiles_kernel(
     }
 }
 
+__global__ __launch_bounds__(kThreads) void group_tiles_kernel(
+        const int* __restrict__ counts, int groups, int tile_rows, int max_tiles,
+        int* __restrict__ tile_group, int* __restrict__ tile_row0, int* __restrict__ tile_nrows,
+        int* __restrict__ offsets) {
+    tiles_from_counts(counts, groups, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows, offsets);
+}
+
 __global__ __launch_bounds__(kThreads) void fill_zero_kernel(int* __restrict__ p, int n) {
     const int i = blockIdx.x * kThreads + threadIdx.x;
     if (i < n) p[i] = 0;
@@ -158,8 +179,9 @@ __global__ __launch_bounds__(kThreads) void fill_zero_kernel(int* __restrict__ p
 
 // counts[e] += number of (token, slot) pairs routed to expert e; a workgroup first adds up its pairs in LDS
 __global__ __launch_bounds__(kThreads) void route_count_kernel(
-        const int64_t* __restrict__ indices, int64_t pairs, int experts, int* __restrict__ counts) {
+        const int64_t* __restrict__ indices, int64_t pairs, int experts, int* __restrict__ counts, int shared_rows) {
     extern __shared__ int bins[];
+    if (shared_rows && blockIdx.x == 0 && threadIdx.x == 0) counts[experts] = shared_rows;   // nobody else adds to it
     for (int e = threadIdx.x; e < experts; e += kThreads) bins[e] = 0;
     __syncthreads();
     for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < pairs; p += (int64_t)gridDim.x * kThreads) {
@@ -173,14 +195,15 @@ __global__ __launch_bounds__(kThreads) void route_count_kernel(
 
 // One thread per token: its experts in ascending order get the next free row of their group.  The order of rows
 // inside a group depends on the order in which threads arrive, which is harmless: a row of the grouped GEMM does
-// not depend on its position, and `rows` records where each pair went.
+// not depend on its position, and `rows` records where each pair went.  With `shared_one` != 0 every token also
+// takes row t of one more group (index `experts`, rows in token order) as its last entry, with that 16-bit
+// pattern (1.0 in the weights' type) as its weight: the outputs then have topk + 1 columns.
 template <int MAXK>
-__global__ __launch_bounds__(kThreads) void route_scatter_kernel(
-        const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int tokens, int topk, int experts,
-        const int* __restrict__ offsets, int* __restrict__ cursor,
-        int* __restrict__ a_rows, int* __restrict__ rows, uint16_t* __restrict__ w_sorted) {
-    const int t = blockIdx.x * kThreads + threadIdx.x;
-    if (t >= tokens) return;
+__device__ __forceinline__ void scatter_token(
+        int t, const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int topk, int experts,
+        const int* offsets, int* cursor, int* __restrict__ a_rows, int* __restrict__ rows,
+        uint16_t* __restrict__ w_sorted, int shared_one) {
+    const int cols = topk + (shared_one ? 1 : 0);
     int e[MAXK], slot[MAXK];
 #pragma unroll
     for (int j = 0; j < MAXK; ++j) {
@@ -206,29 +229,81 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
                 pos = offsets[e[j]] + atomicAdd(&cursor[e[j]], 1);
                 a_rows[pos] = t;
             }
-            rows[(int64_t)t * topk + j] = pos;
-            w_sorted[(int64_t)t * topk + j] = weights[(int64_t)t * topk + slot[j]];
+            rows[(int64_t)t * cols + j] = pos;
+            w_sorted[(int64_t)t * cols + j] = weights[(int64_t)t * topk + slot[j]];
         }
     }
+    if (shared_one) {
+        const int pos = offsets[experts] + t;
+        a_rows[pos] = t;
+        rows[(int64_t)t * cols + topk] = pos;
+        w_sorted[(int64_t)t * cols + topk] = (uint16_t)shared_one;
+    }
+}
+
+template <int MAXK>
+__global__ __launch_bounds__(kThreads) void route_scatter_kernel(
+        const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int tokens, int topk, int experts,
+        const int* __restrict__ offsets, int* __restrict__ cursor,
+        int* __restrict__ a_rows, int* __restrict__ rows, uint16_t* __restrict__ w_sorted, int shared_one) {
+    const int t = blockIdx.x * kThreads + threadIdx.x;
+    if (t >= tokens) return;
+    scatter_token<MAXK>(t, indices, weights, topk, experts, offsets, cursor, a_rows, rows, w_sorted, shared_one);
+}
+
+// The whole bookkeeping in one workgroup, for token counts up to kThreads (decode steps): counts, offsets and
+// cursors stay in LDS; only the counts are also written out.
+template <int MAXK>
+__global__ __launch_bounds__(kThreads) void route_small_kernel(
+        const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int tokens, int topk, int experts,
+        int groups, int tile_rows, int max_tiles, int* __restrict__ counts_out, int* __restrict__ offsets_out,
+        int* __restrict__ a_rows, int* __restrict__ rows, uint16_t* __restrict__ w_sorted,
+        int* __restrict__ tile_group, int* __restrict__ tile_row0, int* __restrict__ tile_nrows, int shared_one) {
+    extern __shared__ int lds_i[];
+    int* bins = lds_i; int* offs = lds_i + groups; int* cur = lds_i + 2 * groups;
+    for (int g = threadIdx.x; g < 3 * groups; g += kThreads) lds_i[g] = 0;
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < tokens) {
+        for (int j = 0; j < topk; ++j) {
+            const int64_t e = indices[(int64_t)t * topk + j];
+            if (e >= 0 && e < experts) atomicAdd(&bins[e], 1);
+        }
+    }
+    if (shared_one && t == 0) bins[experts] = tokens;
+    __syncthreads();
+    for (int g = threadIdx.x; g < groups; g += kThreads) counts_out[g] = bins[g];
+    tiles_from_counts(bins, groups, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows, offs);
+    __syncthreads();
+    for (int g = threadIdx.x; g < groups; g += kThreads) offsets_out[g] = offs[g];
+    if (t < tokens)
+        scatter_token<MAXK>(t, indices, weights, topk, experts, offs, cur, a_rows, rows, w_sorted, shared_one);
 }
 
 }  // namespace
 
 int launch_moe_route(const int64_t* indices, const void* weights, int64_t tokens, int topk, int experts,
-                     int max_tiles, int tile_rows, int* counts, int* offsets, int* cursor, int* a_rows, int* rows,
-                     void* w_sorted, int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st) {
+                     int shared_one, int max_tiles, int tile_rows, int* counts, int* offsets, int* cursor, int* a_rows,
+                     int* rows, void* w_sorted, int* tile_group, int* tile_row0, int* tile_nrows, hipStream_t st) {
     const int64_t pairs = tokens * topk;
+    const int groups = experts + (shared_one ? 1 : 0);
+    if (tokens <= kThreads && groups <= 4096) {
+        hipLaunchKernelGGL(route_small_kernel<16>, dim3(1), dim3(kThreads), (size_t)3 * groups * sizeof(int), st,
+                           indices, (const uint16_t*)weights, (int)tokens, topk, experts, groups, tile_rows, max_tiles,
+                           counts, offsets, a_rows, rows, (uint16_t*)w_sorted, tile_group, tile_row0, tile_nrows, shared_one);
+        return launch_status();
+    }
     // counts | offsets | cursor are consecutive thirds of one scratch array; clear it with a kernel (a memset node
     // recorded into a captured graph has given wrong results on replays)
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((3 * experts + kThreads - 1) / kThreads)), dim3(kThreads), 0, st, counts, 3 * experts);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((3 * groups + kThreads - 1) / kThreads)), dim3(kThreads), 0, st, counts, 3 * groups);
     const unsigned cgrid = (unsigned)((pairs + kThreads * 8 - 1) / (kThreads * 8) > 1024 ? 1024 : (pairs + kThreads * 8 - 1) / (kThreads * 8));
     hipLaunchKernelGGL(route_count_kernel, dim3(cgrid ? cgrid : 1), dim3(kThreads), (size_t)experts * sizeof(int), st,
-                       indices, pairs, experts, counts);
+                       indices, pairs, experts, counts, shared_one ? (int)tokens : 0);
     hipLaunchKernelGGL(group_tiles_kernel, dim3(1), dim3(kThreads), 0, st,
-                       (const int*)counts, experts, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows, offsets);
+                       (const int*)counts, groups, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows, offsets);
     hipLaunchKernelGGL(route_scatter_kernel<16>, dim3((unsigned)((tokens + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
                        indices, (const uint16_t*)weights, (int)tokens, topk, experts, (const int*)offsets, cursor,
-                       a_rows, rows, (uint16_t*)w_sorted);
+                       a_rows, rows, (uint16_t*)w_sorted, shared_one);
     return launch_status();
 }
 
@@ -247,7 +322,8 @@ int launch_swiglu_quant(const void* h, void* y, float* s, int64_t rows, int64_t 
 
 int launch_moe_combine(const void* out, const int* rows, const void* w, const void* shared, void* y,
                        int64_t tokens, int topk, int64_t dim, hipStream_t st) {
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)tokens), dim3(kThreads), 0, st,
+    const unsigned chunk_blocks = (unsigned)((dim / 8 + kThreads - 1) / kThreads);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)tokens, chunk_blocks), dim3(kThreads), 0, st,
                        (const v4u*)out, rows, (const uint16_t*)w, (const v4u*)shared, (v4u*)y, topk, (int)(dim / 8));
     return launch_status();
 }

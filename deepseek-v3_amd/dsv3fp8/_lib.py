@@ -28,7 +28,7 @@ EXPORTS = {
     "dsv3_fp8_gemm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "dsv3_fp8_gemm_grouped_tile_rows": (c_int, []),
     "dsv3_group_tiles": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
-    "dsv3_moe_route": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+    "dsv3_moe_route": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "dsv3_fp8_gemm_grouped": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64,
                                       c_void_p, c_int, c_int64, c_int64, c_int64,

@@ -361,6 +361,7 @@ class MoE(nn.Module):
     """
 
     grouped: bool = True
+    fold_shared_max_tokens: int = 512
 
     def __init__(self, args: ModelArgs):
         super().__init__()
@@ -381,13 +382,20 @@ class MoE(nn.Module):
     def stack_experts(self) -> None:
         """Move the routed experts' weights into two contiguous buffers, [E, 2*inter, dim] (w1 over w3) and
         [E, dim, inter] (w2), with their scales alongside; each expert's parameters become views of them, so
-        ``load_model``-style in-place copies and the expert-by-expert path keep working on the same memory."""
+        ``load_model``-style in-place copies and the expert-by-expert path keep working on the same memory.
+        A shared expert of the same shape (``n_shared_experts == 1``) is stacked behind them as entry E, so the
+        grouped GEMMs can run it as one more group."""
         if self._stacked is not None:
             return
         exs = list(self.experts)
         inter, dim = exs[0].w1.out_features, self.dim
         assert inter % block_size == 0 and dim % block_size == 0
         dev, fp8 = exs[0].w1.weight.device, exs[0].w1.weight.dtype
+        sh = self.shared_experts
+        self._shared_stacked = (sh.w1.out_features == inter and sh.w1.weight.dtype == fp8
+                                and sh.w1.weight.device == dev)
+        if self._shared_stacked:
+            exs.append(sh)
         n = len(exs)
         ib, db = inter // block_size, dim // block_size
         with torch.no_grad():
@@ -414,20 +422,28 @@ class MoE(nn.Module):
     def _forward_grouped(self, x: torch.Tensor, weights: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
         self.stack_experts()
         w13, s13, w2, s2 = self._stacked
-        tokens, topk = indices.shape
-        pairs = tokens * topk
+        # Few tokens: the shared expert rides along as group E that every token selects with weight 1 -- it has the
+        # highest index, so the ordered combine adds it last, bf16(y + bf16(z * 1)) = bf16(y + z), exactly where
+        # the reference adds z.  That saves its three separate GEMM + quantise launches; with many tokens the dense
+        # large-M kernel runs it faster than 128-row groups do.  Its linears never take scale_fmt (model.py:233,
+        # 262), so the shortcut needs the routed experts to use none either.
+        fold = (self._shared_stacked and Linear.scale_fmt is None and indices.size(0) <= self.fold_shared_max_tokens
+                and indices.size(1) < 16)
+        if not fold:
+            w13, s13, w2, s2 = (t[:self.n_routed_experts] for t in self._stacked)
         # counts per expert, expert-sorted token list, each token's rows in ascending expert order (the order in
         # which the reference's loop adds them, model.py:684-689) and the tile table -- all on the device
         _, a_rows, rows, w_sorted, tile_group, tile_row0, tile_rows = torch.ops.dsv3fp8.moe_route(
-            indices.contiguous(), weights.contiguous(), self.n_routed_experts)
+            indices.contiguous(), weights.contiguous(), self.n_routed_experts, fold)
+        pairs = rows.numel()
         fmt = ops._lib.SCALE_FMT_UE8M0 if Linear.scale_fmt == "ue8m0" else ops._lib.SCALE_FMT_NONE
         code = ops.dtype_code(torch.get_default_dtype())
         xq, xs = act_quant(x, block_size, Linear.scale_fmt)           # quantised once: 1x128 blocks are per token
         h = torch.ops.dsv3fp8.fp8_gemm_grouped(xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, code)
         gq, gs = torch.ops.dsv3fp8.swiglu_quant(h, block_size, fmt)
         out = torch.ops.dsv3fp8.fp8_gemm_grouped(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code)
-        z = self.shared_experts(x)
-        return torch.ops.dsv3fp8.moe_combine(out, rows, w_sorted, z.contiguous())
+        z = None if fold else self.shared_experts(x).contiguous()
+        return torch.ops.dsv3fp8.moe_combine(out, rows, w_sorted, z)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         shape = x.size()

@@ -24,7 +24,7 @@ _libdef.define("act_quant(Tensor x, int block_size, int scale_fmt) -> (Tensor, T
 _libdef.define("weight_dequant(Tensor x, Tensor s, int block_size, int out_dtype) -> Tensor")
 _libdef.define("fp8_gemm(Tensor a, Tensor a_s, Tensor b, Tensor b_s, int out_dtype) -> Tensor")
 _libdef.define("group_tiles(Tensor counts, int max_tiles) -> (Tensor, Tensor, Tensor)")
-_libdef.define("moe_route(Tensor indices, Tensor weights, int experts) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)")
+_libdef.define("moe_route(Tensor indices, Tensor weights, int experts, bool shared_group) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)")
 _libdef.define("fp8_gemm_grouped(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b, Tensor b_s, int rows, "
                "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int out_dtype) -> Tensor")
 _libdef.define("swiglu_quant(Tensor h, int block_size, int scale_fmt) -> (Tensor, Tensor)")
@@ -126,34 +126,38 @@ def _group_tiles_meta(counts, max_tiles):
     return tuple(counts.new_empty(max_tiles, dtype=torch.int32) for _ in range(3))
 
 
-def _moe_route_dev(indices: torch.Tensor, weights: torch.Tensor, experts: int):
-    """-> counts [experts], a_rows [tokens*topk], rows [tokens, topk], w_sorted [tokens, topk], tile_group,
-    tile_row0, tile_rows (see dsv3_moe_route in include/dsv3_fp8.h)."""
+def _moe_route_dev(indices: torch.Tensor, weights: torch.Tensor, experts: int, shared_group: bool):
+    """-> counts [groups], a_rows [tokens*cols], rows [tokens, cols], w_sorted [tokens, cols], tile_group,
+    tile_row0, tile_rows, with groups = experts (+1) and cols = topk (+1 with shared_group); see dsv3_moe_route
+    in include/dsv3_fp8.h."""
     assert indices.dtype == torch.int64 and indices.dim() == 2 and indices.is_contiguous()
     assert weights.shape == indices.shape and weights.is_contiguous() and weights.element_size() == 2
     tokens, topk = indices.shape
-    pairs = tokens * topk
-    max_tiles = pairs // grouped_tile_rows() + experts
+    groups, cols = experts + int(shared_group), topk + int(shared_group)
+    pairs = tokens * cols
+    max_tiles = pairs // grouped_tile_rows() + groups
     dev = indices.device
-    ints = torch.empty(3 * experts + pairs + pairs + 3 * max_tiles, dtype=torch.int32, device=dev)
-    scratch, a_rows, rows, tiles = ints.split([3 * experts, pairs, pairs, 3 * max_tiles])
+    ints = torch.empty(3 * groups + pairs + pairs + 3 * max_tiles, dtype=torch.int32, device=dev)
+    scratch, a_rows, rows, tiles = ints.split([3 * groups, pairs, pairs, 3 * max_tiles])
     tiles = tiles.view(3, max_tiles)
-    w_sorted = torch.empty_like(weights)
+    w_sorted = weights.new_empty(tokens, cols)
     with torch.cuda.device(dev):
         rc = _lib.lib.dsv3_moe_route(indices.data_ptr(), weights.data_ptr(), dtype_code(weights.dtype), tokens, topk,
-                                     experts, max_tiles, scratch.data_ptr(), a_rows.data_ptr(), rows.data_ptr(),
-                                     w_sorted.data_ptr(), tiles[0].data_ptr(), tiles[1].data_ptr(), tiles[2].data_ptr(),
-                                     _stream(indices))
+                                     experts, int(shared_group), max_tiles, scratch.data_ptr(), a_rows.data_ptr(),
+                                     rows.data_ptr(), w_sorted.data_ptr(), tiles[0].data_ptr(), tiles[1].data_ptr(),
+                                     tiles[2].data_ptr(), _stream(indices))
     _lib.check(rc, "dsv3_moe_route")
-    return scratch[:experts], a_rows, rows.view(tokens, topk), w_sorted, tiles[0], tiles[1], tiles[2]
+    return scratch[:groups], a_rows, rows.view(tokens, cols), w_sorted, tiles[0], tiles[1], tiles[2]
 
 
-def _moe_route_meta(indices, weights, experts):
+def _moe_route_meta(indices, weights, experts, shared_group):
     tokens, topk = indices.shape
-    pairs = tokens * topk
-    max_tiles = pairs // grouped_tile_rows() + experts
+    groups, cols = experts + int(shared_group), topk + int(shared_group)
+    pairs = tokens * cols
+    max_tiles = pairs // grouped_tile_rows() + groups
     i32 = lambda *shape: indices.new_empty(*shape, dtype=torch.int32)
-    return i32(experts), i32(pairs), i32(tokens, topk), torch.empty_like(weights), i32(max_tiles), i32(max_tiles), i32(max_tiles)
+    return (i32(groups), i32(pairs), i32(tokens, cols), weights.new_empty(tokens, cols), i32(max_tiles), i32(max_tiles),
+            i32(max_tiles))
 
 
 def _fp8_gemm_grouped_dev(a, a_s, a_rows, b, b_s, rows: int, tile_group, tile_row0, tile_rows, out_dtype: int):

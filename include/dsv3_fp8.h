@@ -154,9 +154,13 @@ int dsv3_group_tiles(const int32_t* counts, int groups, int max_tiles,
  *     w_sorted[tokens, topk]   : the routing weights in the same order;
  *     tile_group/tile_row0/tile_rows [max_tiles]: the tile table of dsv3_group_tiles for these counts.
  * The order of rows inside an expert's group is unspecified (it does not affect any result).  topk <= 16.
+ * shared_group != 0 appends one more group, index `experts`, that EVERY token selects with weight 1.0 as its last
+ * entry (its rows are in token order): the shared expert of inference/model.py:690 run as one more group of the
+ * grouped GEMMs; adding it last with weight 1 is the reference's `y + z`.  Then scratch has 3*(experts+1) entries,
+ * a_rows tokens*(topk+1), and rows / w_sorted have topk+1 columns.
  */
 int dsv3_moe_route(const int64_t* indices, const void* weights, int w_dtype, int64_t tokens, int topk, int experts,
-                   int max_tiles, int32_t* scratch, int32_t* a_rows, int32_t* rows, void* w_sorted,
+                   int shared_group, int max_tiles, int32_t* scratch, int32_t* a_rows, int32_t* rows, void* w_sorted,
                    int32_t* tile_group, int32_t* tile_row0, int32_t* tile_rows, void* stream);
 
 /*

@@ -153,14 +153,15 @@ def test_moe_combine_validation(L):
 
 def test_moe_route_validation(L):
     f = L.lib.dsv3_moe_route
-    ok = [A16, A16, L.BF16, 4, 2, 8, 12, A16, A16, A16, A16, A16, A16, A16, None]
+    #     idx  w    dtype   tok topk exp shared max_tiles scratch a_rows rows w_sorted tile tables    stream
+    ok = [A16, A16, L.BF16, 4,  2,   8,  0,     12,       A16,    A16,   A16, A16,     A16, A16, A16, None]
 
     def call(i=None, v=None):
         a = list(ok)
         if i is not None:
             a[i] = v
         return f(*a)
-    assert call(0, None) == 1 and call(7, None) == 1 and call(11, None) == 1
+    assert call(0, None) == 1 and call(8, None) == 1 and call(12, None) == 1
     assert call(2, L.F32) == 5
     assert call(4, 0) == 2 and call(4, 17) == 2 and call(5, 0) == 2 and call(3, -1) == 2
     assert call(0, A16 + 4) == 4

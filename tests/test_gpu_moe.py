@@ -166,8 +166,13 @@ def test_moe_grouped_matches_expert_loop_and_oracle(K):
         x = torch.randn(300, 256, generator=g).bfloat16()
         with torch.inference_mode():
             M.MoE.grouped = True
-            y_grouped = moe(x.cuda())
+            y_grouped = moe(x.cuda())                   # 300 tokens: the shared expert rides along as group 8
             assert moe._stacked is not None and moe.experts[3].w1.weight.data_ptr() == moe._stacked[0][3].data_ptr()
+            assert moe._shared_stacked and moe.shared_experts.w2.weight.data_ptr() == moe._stacked[2][8].data_ptr()
+            moe.fold_shared_max_tokens = 0              # the shared expert as three dense linears instead
+            y_unfolded = moe(x.cuda())
+            del moe.fold_shared_max_tokens
+            assert (y_grouped.float() - y_unfolded.float()).abs().max().item() <= 2e-2 * y_unfolded.float().pow(2).mean().sqrt().item()
             M.MoE.grouped = False
             y_loop = moe(x.cuda())                      # the reference's loop on the (now stacked) expert weights
             wts, idx = moe.gate(x.cuda())
@@ -182,24 +187,35 @@ def test_moe_grouped_matches_expert_loop_and_oracle(K):
         torch.set_default_dtype(old[1])
 
 
-@pytest.mark.parametrize("tokens,topk,experts", [(300, 2, 8), (4096, 8, 256), (1, 4, 16), (33, 1, 5)])
-def test_moe_route(K, tokens, topk, experts):
+@pytest.mark.parametrize("shared", [False, True])
+@pytest.mark.parametrize("tokens,topk,experts", [(300, 2, 8), (4096, 8, 256), (1, 4, 16), (33, 1, 5), (256, 8, 256),
+                                                 (257, 8, 256)])
+def test_moe_route(K, tokens, topk, experts, shared):
+    """Both routes of the bookkeeping (one workgroup up to 256 tokens, four kernels above), with and without the
+    extra group that every token selects last with weight 1."""
     from dsv3fp8 import ops
     g = torch.Generator().manual_seed(7)
     scores = torch.rand(tokens, experts, generator=g)
     scores[:, experts // 2] += 0.3 * (torch.arange(tokens) % 3 == 0)            # a popular expert
     indices = scores.topk(topk, dim=-1)[1]
     weights = torch.rand(tokens, topk, generator=g).bfloat16()
-    counts, a_rows, rows, w_sorted, tg, t0, tr = torch.ops.dsv3fp8.moe_route(indices.cuda(), weights.cuda(), experts)
+    counts, a_rows, rows, w_sorted, tg, t0, tr = torch.ops.dsv3fp8.moe_route(indices.cuda(), weights.cuda(), experts, shared)
     counts, a_rows, rows, w_sorted = counts.cpu(), a_rows.cpu(), rows.cpu(), w_sorted.cpu()
+    if shared:                                                                   # the reference view of the same thing
+        indices = torch.cat([indices, torch.full((tokens, 1), experts)], dim=1)
+        weights = torch.cat([weights, torch.ones(tokens, 1, dtype=torch.bfloat16)], dim=1)
+        experts, topk = experts + 1, topk + 1
     ref_counts = torch.bincount(indices.flatten(), minlength=experts)
     assert torch.equal(counts.long(), ref_counts)
     offsets = torch.cumsum(ref_counts, 0) - ref_counts
     pairs = tokens * topk
+    assert rows.shape == (tokens, topk) and a_rows.numel() == pairs
     assert sorted(rows.flatten().tolist()) == list(range(pairs))               # every row used exactly once
     for e in range(experts):                                                    # group e = the tokens that chose e
         grp = a_rows[offsets[e]:offsets[e] + ref_counts[e]].long()
         assert torch.equal(grp.sort()[0], torch.where((indices == e).any(-1))[0])
+    if shared:                                                                   # the extra group is in token order
+        assert torch.equal(a_rows[offsets[-1]:].long(), torch.arange(tokens))
     order = indices.argsort(dim=1)
     se = indices.gather(1, order)
     assert torch.equal(w_sorted.view(torch.int16), weights.gather(1, order).view(torch.int16))
@@ -207,10 +223,11 @@ def test_moe_route(K, tokens, topk, experts):
         r = rows[:, j].long()
         assert torch.equal(a_rows[r].long(), torch.arange(tokens))
         assert ((r >= offsets[se[:, j]]) & (r < offsets[se[:, j]] + ref_counts[se[:, j]])).all()
+    # the tile table covers every group's rows in order
     R = ops.grouped_tile_rows()
-    exp_tiles = [(e, int(offsets[e]) + i, min(R, int(ref_counts[e]) - i)) for e in range(experts) for i in range(0, int(ref_counts[e]), R)]
+    exp = [(e, int(offsets[e]) + i, min(R, int(ref_counts[e]) - i)) for e in range(experts) for i in range(0, int(ref_counts[e]), R)]
     got = list(zip(tg.tolist(), t0.tolist(), tr.tolist()))
-    assert got[:len(exp_tiles)] == exp_tiles and all(x[0] == -1 for x in got[len(exp_tiles):])
+    assert got[:len(exp)] == exp and all(x[0] == -1 for x in got[len(exp):])
 
 
 def test_moe_forward_is_graph_capturable(K):
