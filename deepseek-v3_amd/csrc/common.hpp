@@ -80,9 +80,10 @@ bool skinny_supported(int64_t m, int64_t n, int64_t k);
 size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t k);
 int launch_skinny(const void* a, const float* a_s, const void* b, const float* b_s, void* c, int c_dtype,
                   int64_t m, int64_t n, int64_t k, void* ws, int* splits_out, hipStream_t st);
+int prefill_splits(int64_t m, int64_t n, int64_t k);
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
-                   int64_t m, int64_t n, int64_t k, hipStream_t stream);
+                   int64_t m, int64_t n, int64_t k, int splits, hipStream_t stream);
 int grouped_tile_rows();
 bool grouped_supported(int64_t a_num_rows, int64_t n, int64_t k);
 template <int CD>

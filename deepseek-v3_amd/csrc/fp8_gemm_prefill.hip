@@ -84,7 +84,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
-        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, GroupTable g) {
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, GroupTable g) {
     using C = Cfg<TM, S>;
     constexpr int WM = C::WM, SM = C::SM, A_LOADS = C::A_LOADS, B_LOADS = C::B_LOADS;
     constexpr int A_STAGE = C::A_STAGE, B_STAGE = C::B_STAGE, LDS_A = C::LDS_A, LDS_B = C::LDS_B, LDS_SC = C::LDS_SC;
@@ -132,7 +132,13 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & (WAVES_M - 1), wn = wave / WAVES_M;
-    const int KB = K / 128;
+    // K blocks of this workgroup: all of them, or slice blockIdx.y of a split over K (dense mode only), whose
+    // partial sums go to slab blockIdx.y of c
+    const int KBT = K / 128;
+    const int kb0 = blockIdx.y * kb_per_split;
+    const int KB = min(kb_per_split, KBT - kb0);
+    c += (size_t)blockIdx.y * (size_t)M * (size_t)N;
+    a += (size_t)kb0 * 128u; b += (size_t)kb0 * 128u;
 
     // ---- global -> LDS copy plan: a stage is TM rows of A, then 256 of B, in 1 KiB wavefront-loads of 8 rows;
     // wavefront w issues A loads t*8 + w (t < A_LOADS) and B loads t*8 + w (t < B_LOADS).
@@ -178,8 +184,8 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     // loop free of branches).
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
-    const uint32_t sc_off = wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KB
-                                     : (uint32_t)min(n0 / 128 + lane, nb_last) * (uint32_t)KB;
+    const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT
+                                      : (uint32_t)min(n0 / 128 + lane, nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
     auto issue_scales = [&](int kb, int stage) {
         __builtin_amdgcn_global_load_lds((gptr_t)(sc_base + sc_off + (uint32_t)kb),
                                          (lptr_t)(lds + LDS_SC + stage * SC_STAGE + wave * 256), 4, 0, 0);
@@ -404,7 +410,7 @@ namespace {
 template <int CD, bool G, int TM, int S>
 int launch_kernel(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                   int64_t m, int64_t n, int64_t k, int64_t tm, int64_t tn_first, int64_t tn_count,
-                  prefill::GroupTable g, hipStream_t stream) {
+                  prefill::GroupTable g, hipStream_t stream, int splits = 1) {
     using namespace prefill;
     constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
     if ((tm + 8) * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
@@ -419,9 +425,11 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
         granted[dev] = true;
     }
     const int64_t grid = (G ? (tm + 7) / 8 * 8 : tm) * tn_count;       // grouped: row tiles are dealt over the 8 XCDs
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream,
-                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c,
-                       (int)m, (int)n, (int)k, (int)tm, (int)tn_count, (int)tn_first, g);
+    const int kb = (int)(k / 128), kb_per_split = (kb + splits - 1) / splits;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)((kb + kb_per_split - 1) / kb_per_split)), dim3(THREADS),
+                       LDS_BYTES, stream, (const uint8_t*)a, a_s, (const uint8_t*)b, b_s,
+                       (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)tm, (int)tn_count, (int)tn_first,
+                       kb_per_split, g);
     return launch_status();
 }
 constexpr int kGroupedTileRows = 128;
@@ -429,9 +437,23 @@ constexpr int64_t kCUs = 256;
 inline int env_tile_rows() { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }
 }  // namespace
 
+// Few row tiles (M up to a few hundred rows) leave most compute units without a tile: the K range is then cut
+// into slices that run as separate workgroups and write binary32 partial sums, which a second kernel adds in a
+// fixed order.  Worth it while the slices still hold 8 K blocks and the workgroup count stays within one round.
+int prefill_splits(int64_t m, int64_t n, int64_t k) {
+    if (m <= 0 || n <= 0 || k < 128) return 1;
+    if (getenv("DSV3_PREFILL_NOSPLIT")) return 1;
+    const int64_t tiles = ((m + 127) / 128) * ((n + prefill::BN - 1) / prefill::BN);
+    int64_t splits = kCUs / tiles;
+    const int64_t kb = k / 128;
+    if (splits > kb / 8) splits = kb / 8;
+    if (splits > 8) splits = 8;
+    return splits < 2 ? 1 : (int)splits;
+}
+
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
-                   int64_t m, int64_t n, int64_t k, hipStream_t stream) {
+                   int64_t m, int64_t n, int64_t k, int splits, hipStream_t stream) {
     // Two tile heights.  A round of 256-row tiles over the 256 compute units takes about 1.64x as long as a round
     // of 128-row tiles (measured, K = 7168), and the last round is rarely full: pick whichever needs less time in
     // whole rounds.  (M = 4096 x N = 18432: 5 rounds of tall tiles beat 9 of short ones; M = 1024: 3 short rounds
@@ -441,8 +463,8 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
     auto rounds = [](int64_t tiles) { return (tiles + kCUs - 1) / kCUs; };
     const int forced = env_tile_rows();
     const prefill::GroupTable none{};
-    if (forced == 128 || (forced != 256 && 100 * rounds(tm128 * tn) <= 164 * rounds(tm256 * tn)))
-        return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, tm128, 0, tn, none, stream);
+    if (splits > 1 || forced == 128 || (forced != 256 && 100 * rounds(tm128 * tn) <= 164 * rounds(tm256 * tn)))
+        return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, tm128, 0, tn, none, stream, splits);
     return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, tm256, 0, tn, none, stream);
 }
 
@@ -465,7 +487,7 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
 }
 
 #define DSV3_INST(CD) \
-    template int launch_prefill<CD>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, hipStream_t); \
+    template int launch_prefill<CD>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, int, hipStream_t); \
     template int launch_grouped<CD>(const void*, const float*, const int*, const void*, const float*, void*, int64_t, int64_t, int64_t, \
                                     int64_t, const int*, const int*, const int*, int64_t, int64_t, hipStream_t);
 DSV3_INST(DSV3_BF16)

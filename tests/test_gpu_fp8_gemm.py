@@ -81,6 +81,24 @@ def test_large_m_tile_heights_and_short_k(K, m, n, k):
     _check(K, x, w8, ws)
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (100, 577, 7168),     # 3 tiles: the K range is cut into 7 slices of 8 blocks; ragged N
+    (130, 4096, 2048),    # two row tiles (one with 2 rows), 2 slices of 8 blocks
+    (128, 18432, 7168),   # 72 tiles, 3 slices of 19 + 19 + 18 blocks
+    (257, 7168, 18432),   # 84 tiles, 3 slices of 48 blocks
+    (65, 1536, 1152),     # 9 K blocks: too short to cut, one slice
+])
+def test_mid_m_split_over_k(K, m, n, k):
+    """Between 65 and a few hundred rows the large-M kernel cuts the K range into slices run by separate
+    workgroups (binary32 partial sums, added in a fixed order by a second kernel)."""
+    from dsv3fp8 import workloads, _lib
+    x = workloads.activations(m, k, seed=m)
+    w8, ws = workloads.weight(n, k, seed=n % 89)
+    _check(K, x, w8, ws)
+    if k >= 2048:
+        assert _lib.lib.dsv3_fp8_gemm_workspace_bytes(m, n, k) >= 2 * m * n * 4
+
+
 @pytest.mark.parametrize("n", [1, 15, 16, 100, 129, 576, 577, 1000])
 def test_ragged_n(K, n):
     from dsv3fp8 import workloads
