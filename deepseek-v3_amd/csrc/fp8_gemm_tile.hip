@@ -293,6 +293,14 @@ int forced_kernel() {
     return v;
 }
 
+// Which problems go to the large-M kernel (K range cut into slices when the tiles do not fill the chip): every M
+// above 64, and M = 17 .. 64 when the weight is large (>= 96 MiB, e.g. 16384 -> 7168: 32 us against 35 - 42 us of
+// the streaming kernel at M = 32 .. 64; for the smaller decode weights the streaming and tile kernels are faster).
+bool to_large_m_kernel(int64_t m, int64_t n, int64_t k) {
+    if (!prefill_supported(m, n, k)) return false;
+    return m > 64 || (m > 16 && n * k >= (96ll << 20));
+}
+
 template <int CD>
 int launch_typed(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                  int64_t m, int64_t n, int64_t k, void* ws, hipStream_t st) {
@@ -303,8 +311,9 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
         return launch_status();
     }
     const int force = forced_kernel();
-    const bool use_stream = force != 1 && stream_supported(m, n, k);
-    if (use_stream || (force != 1 && skinny_supported(m, n, k))) {          // decode shapes: weight-streaming kernels
+    const bool to_prefill = force != 1 && to_large_m_kernel(m, n, k);
+    const bool use_stream = force != 1 && !to_prefill && stream_supported(m, n, k);
+    if (use_stream || (force != 1 && !to_prefill && skinny_supported(m, n, k))) {          // decode shapes: weight-streaming kernels
         int splits = 1;
         const int rc = use_stream ? launch_stream(a, a_s, b, b_s, c, CD, m, n, k, ws, &splits, st)
                                   : launch_skinny(a, a_s, b, b_s, c, CD, m, n, k, ws, &splits, st);
@@ -314,24 +323,24 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
                            (const float*)ws, (typename OutT<CD>::type*)c, mn, splits);
         return launch_status();
     }
+    if (to_prefill) {
+        const int splits = prefill_splits(m, n, k);
+        if (splits == 1) return launch_prefill<CD>(a, a_s, b, b_s, c, m, n, k, 1, st);
+        const int rc = launch_prefill<DSV3_F32>(a, a_s, b, b_s, ws, m, n, k, splits, st);
+        if (rc != DSV3_OK) return rc;
+        const int64_t mn = m * n;
+        const int kb = (int)(k / 128), per = (kb + splits - 1) / splits;
+        const int slabs = (kb + per - 1) / per;
+        if (mn % 4 == 0)
+            hipLaunchKernelGGL((splitk_reduce4_kernel<CD>), dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, st,
+                               (const v4f*)ws, (typename OutT<CD>::type*)c, mn / 4, slabs);
+        else
+            hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
+                               (const float*)ws, (typename OutT<CD>::type*)c, mn, slabs);
+        return launch_status();
+    }
     const Plan p = make_plan(m, n, k);
     if (p.splits == 1) {
-        if (prefill_supported(m, n, k) && m > 64 && force != 1) {
-            const int splits = prefill_splits(m, n, k);
-            if (splits == 1) return launch_prefill<CD>(a, a_s, b, b_s, c, m, n, k, 1, st);
-            const int rc = launch_prefill<DSV3_F32>(a, a_s, b, b_s, ws, m, n, k, splits, st);
-            if (rc != DSV3_OK) return rc;
-            const int64_t mn = m * n;
-            const int kb = (int)(k / 128), per = (kb + splits - 1) / splits;
-            const int slabs = (kb + per - 1) / per;
-            if (mn % 4 == 0)
-                hipLaunchKernelGGL((splitk_reduce4_kernel<CD>), dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, st,
-                                   (const v4f*)ws, (typename OutT<CD>::type*)c, mn / 4, slabs);
-            else
-                hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
-                                   (const float*)ws, (typename OutT<CD>::type*)c, mn, slabs);
-            return launch_status();
-        }
         if (p.bm == 32) return launch_cfg<32, 128, 32, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
         if (p.bm == 64) return launch_cfg<64, 128, 64, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
         return launch_cfg<128, 128, 64, 64, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
@@ -355,7 +364,7 @@ size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
     size_t need = tile_ws;
     if (skinny_supported(m, n, k) && skinny_workspace_bytes(m, n, k) > need) need = skinny_workspace_bytes(m, n, k);
     if (stream_supported(m, n, k) && stream_workspace_bytes(m, n, k) > need) need = stream_workspace_bytes(m, n, k);
-    if (p.splits == 1 && prefill_supported(m, n, k) && m > 64 && prefill_splits(m, n, k) > 1) {
+    if (to_large_m_kernel(m, n, k) && prefill_splits(m, n, k) > 1) {
         const size_t pre = (size_t)prefill_splits(m, n, k) * (size_t)m * (size_t)n * sizeof(float);
         if (pre > need) need = pre;
     }
