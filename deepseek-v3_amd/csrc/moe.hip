@@ -97,8 +97,8 @@ __global__ __launch_bounds__(kThreads) void moe_combine_kernel(
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int k = min(k0 + u, topk - 1);
-            wk[u] = bf16lo_to_f32(w[t * topk + k]);
-            v[u] = out[(int64_t)rows[t * topk + k] * chunks_per_row + c];
+            wk[u] = bf16lo_to_f32(w[(int64_t)t * topk + k]);
+            v[u] = out[(int64_t)rows[(int64_t)t * topk + k] * chunks_per_row + c];
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
