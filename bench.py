@@ -55,7 +55,7 @@ def time_loop(fn, steps: int, warmup: int) -> float:
 
 
 def time_graph(launches, replays: int = 5) -> float:
-    """Average microseconds per launch with the launches captured in one HIP graph, so that
+    """Microseconds per launch (median over the replays) with the launches captured in one HIP graph, so that
     back-to-back kernels are not separated by host launch latency.  `launches` is a list of
     zero-argument callables (typically the same op over rotating buffers)."""
     for fn in launches[: min(3, len(launches))]:
@@ -67,15 +67,15 @@ def time_graph(launches, replays: int = 5) -> float:
             fn()
     g.replay()
     torch.cuda.synchronize()
-    best = float("inf")
+    times = []
     for _ in range(replays):
         e0, e1 = _events(2)
         e0.record()
         g.replay()
         e1.record()
         torch.cuda.synchronize()
-        best = min(best, e0.elapsed_time(e1))
-    return best * 1e3 / len(launches)
+        times.append(e0.elapsed_time(e1))
+    return sorted(times)[len(times) // 2] * 1e3 / len(launches)          # median replay
 
 
 def measured_traffic():
