@@ -132,6 +132,24 @@ def run_extras(K, W):
                                             "hbm_frac": round(gbs / HBM_PEAK_GBS, 3)}
         del wqs
     out["decode"] = dec
+    # linear() at decode sizes: act_quant + fp8_gemm as two launches against the fused single launch
+    lin = {}
+    for name, (k, n) in W.DECODE_SHAPES.items():
+        wq, wsc = W.weight(n, k, 1, "cuda")
+        copies = max(2, min(160, -(-640_000_000 // (n * k))))
+        wqs = [wq.clone() for _ in range(copies)]
+        xa = W.activations(1, k, 1, "cuda")
+
+        def two(t):
+            q, qs = K.act_quant(xa)
+            return K.fp8_gemm(q, qs, t, wsc)
+        l2 = [(lambda t=t: two(t)) for t in wqs]
+        l1 = [(lambda t=t: torch.ops.dsv3fp8.linear_fp8(xa, t, wsc, 0, 0)) for t in wqs]
+        if len(l1) < 40:
+            l1, l2 = l1 * (-(-40 // len(l1))), l2 * (-(-40 // len(l2)))
+        lin[f"{name}_M1"] = {"two_launch_us": round(time_graph(l2), 2), "fused_us": round(time_graph(l1), 2)}
+        del wqs
+    out["linear_decode"] = lin
     out["moe_layer_T4096"] = run_moe(K, W)
     out["wkv_b_absorb"] = run_absorb(K, W)
     return out

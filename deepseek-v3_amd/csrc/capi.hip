@@ -78,6 +78,27 @@ int dsv3_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b
     return launch_fp8_gemm(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+int dsv3_linear_fp8_fused(int64_t m, int64_t n, int64_t k) {
+    return m > 0 && n > 0 && k > 0 && m <= 0x7fffffff && n <= 0x7fffffff && k <= 0x7fffffff && linear_fp8_supported(m, n, k);
+}
+
+int dsv3_linear_fp8(const void* x, int x_dtype, const void* b, const float* b_s, void* c, int c_dtype,
+                    int64_t m, int64_t n, int64_t k, int block_size, int scale_fmt,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+    if (x_dtype != DSV3_BF16 || !valid_dtype(c_dtype)) return DSV3_ERR_BAD_DTYPE;
+    if (scale_fmt != DSV3_SCALE_FMT_NONE && scale_fmt != DSV3_SCALE_FMT_UE8M0) return DSV3_ERR_BAD_DTYPE;
+    if (block_size != 128) return DSV3_ERR_BAD_BLOCK;
+    if (m < 0 || n < 0 || k < 0 || k % 128 != 0) return DSV3_ERR_BAD_SHAPE;
+    if (m == 0 || n == 0) return DSV3_OK;
+    if (!dsv3_linear_fp8_fused(m, n, k)) return DSV3_ERR_BAD_SHAPE;       // ask dsv3_linear_fp8_fused first
+    if (!x || !b || !b_s || !c) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(x, 16) || !aligned(b, 16) || !aligned(b_s, 4) || !aligned(c, c_dtype == DSV3_F32 ? 16 : 8))
+        return DSV3_ERR_MISALIGNED;
+    const size_t need = dsv3_fp8_gemm_workspace_bytes(m, n, k);
+    if (need > 0 && (!workspace || workspace_bytes < need || !aligned(workspace, 256))) return DSV3_ERR_WORKSPACE;
+    return launch_linear_fp8(x, b, b_s, c, c_dtype, m, n, k, scale_fmt, workspace, (hipStream_t)stream);
+}
+
 int dsv3_fp8_gemm_grouped_tile_rows(void) { return grouped_tile_rows(); }
 
 int dsv3_group_tiles(const int32_t* counts, int groups, int max_tiles,

@@ -79,7 +79,10 @@ int launch_stream(const void* a, const float* a_s, const void* b, const float* b
 bool skinny_supported(int64_t m, int64_t n, int64_t k);
 size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t k);
 int launch_skinny(const void* a, const float* a_s, const void* b, const float* b_s, void* c, int c_dtype,
-                  int64_t m, int64_t n, int64_t k, void* ws, int* splits_out, hipStream_t st);
+                  int64_t m, int64_t n, int64_t k, void* ws, int* splits_out, hipStream_t st, int quant_mode = 0);
+int launch_linear_fp8(const void* x, const void* b, const float* b_s, void* c, int c_dtype, int64_t m, int64_t n,
+                      int64_t k, int scale_fmt, void* workspace, hipStream_t stream);
+bool linear_fp8_supported(int64_t m, int64_t n, int64_t k);
 int prefill_splits(int64_t m, int64_t n, int64_t k);
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,

@@ -58,12 +58,21 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 // memory loads retire on different counters, so fetching an activation never drains the weight ring.
 constexpr int kSlabChunks = 4;             // 16-byte activation chunks a thread stages on the way to LDS
 
-template <int MT, int S, int NPF>
+// QF (fused linear, inference/model.py:159-160): `a` holds the bf16 activations themselves and a_s is unused; the
+// workgroup quantises its K range of them on the way into LDS exactly as act_quant would (amax over the 128
+// block, clamp at 1e-4, / 448, optional power-of-two rounding of the scale, correctly rounded quotient, OCP e4m3),
+// so the result equals act_quant followed by this kernel bit for bit and the separate launch disappears.
+template <int CTRL> __device__ __forceinline__ float dpp_max(float v) {
+    int o = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
+    return fmaxf(v, __builtin_bit_cast(float, o));
+}
+
+template <int MT, int S, int NPF, bool QF>
 __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 4))) void fp8_gemm_skinny_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         void* __restrict__ out, int out_dtype,      // out_dtype: dsv3_dtype of `out` (F32 slabs when gridDim.y > 1)
-        int M, int N, int K, int kb_per_wg) {
+        int M, int N, int K, int kb_per_wg, int ue8m0) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -106,16 +115,28 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
     float* act_s = (float*)(lds + (size_t)slab_rows * 128);
     const int chunks = wg_nkb * M * 8;                         // 16-byte chunks to copy (<= kSlabChunks * threads)
     v4i stage[kSlabChunks];
+    v4u raw[QF ? kSlabChunks : 1][2];                          // QF: the 16 bf16 values behind each chunk
+    float stage_q[QF ? kSlabChunks : 1];                       // QF: weight-block scale of the chunk's K block
     float stage_s = 0.f;
 #pragma unroll
     for (int i = 0; i < kSlabChunks; ++i) {
         const int c = tid + i * (int)blockDim.x;
         if (c < chunks) {
             const int ch = c & 7, R = c >> 3, row = R % M, kb = R / M;
-            stage[i] = *(const v4i*)(a + (size_t)row * K + (size_t)(wg_kb0 + kb) * 128 + ch * 16);
+            if (QF) {
+                const v4u* src = (const v4u*)(a + 2 * ((size_t)row * K + (size_t)(wg_kb0 + kb) * 128 + ch * 16));
+                raw[i][0] = src[0];
+                raw[i][1] = src[1];
+                stage_q[i] = b_s[(size_t)min(n0 >> 7, (N - 1) >> 7) * KB + wg_kb0 + kb];
+            } else {
+                stage[i] = *(const v4i*)(a + (size_t)row * K + (size_t)(wg_kb0 + kb) * 128 + ch * 16);
+            }
+        } else if (QF) {
+            raw[i][0] = raw[i][1] = v4u{0u, 0u, 0u, 0u};
+            stage_q[i] = 0.f;
         }
     }
-    if (tid < wg_nkb * M)      // scale of (row, K block) with the weight block's scale already folded in
+    if (!QF && tid < wg_nkb * M)   // scale of (row, K block) with the weight block's scale already folded in
         stage_s = a_s[(size_t)(tid % M) * KB + wg_kb0 + tid / M] * b_s[(size_t)min(n0 >> 7, (N - 1) >> 7) * KB + wg_kb0 + tid / M];
 
     // ---- start the weight stream: the first NPF K blocks of every strip
@@ -131,15 +152,60 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
     for (int p = 0; p < NPF; ++p)
         if (p < nkb) fetch(p, p);
 
+    if (QF) {
+        // the 8 lanes that hold the chunks of one (row, K block) are consecutive and aligned: amax by DPP
 #pragma unroll
-    for (int i = 0; i < kSlabChunks; ++i) {
-        const int c = tid + i * (int)blockDim.x;
-        if (c < chunks) {
-            const int ch = c & 7, R = c >> 3;
-            *(v4i*)(act + R * 128 + ((ch ^ swz(R)) * 16)) = stage[i];
+        for (int i = 0; i < kSlabChunks; ++i) {
+            float f[16];
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    f[8 * h + 2 * e] = bf16lo_to_f32(raw[i][h][e]);
+                    f[8 * h + 2 * e + 1] = bf16hi_to_f32(raw[i][h][e]);
+                }
+            float amax = 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(f[e]));
+            amax = dpp_max<0xB1>(amax);      // quad_perm [1,0,3,2]
+            amax = dpp_max<0x4E>(amax);      // quad_perm [2,3,0,1]
+            amax = dpp_max<0x141>(amax);     // row_half_mirror
+            amax = fmaxf(amax, 1e-4f);
+            float sc = amax / 448.f;
+            if (ue8m0) {
+                uint32_t bits = f32_as_u32(sc);
+                bits = ((bits >> 23) + ((bits & 0x7fffffu) ? 1u : 0u)) << 23;
+                sc = u32_as_f32(bits);
+            }
+            const float r = 1.0f / sc;
+            float q[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {       // x / sc, correctly rounded for bf16 x with |x| <= amax (as act_quant)
+                const float q0 = f[e] * r;
+                const float er = __builtin_fmaf(-q0, sc, f[e]);
+                q[e] = __builtin_copysignf(__builtin_fmaf(er, r, q0), f[e]);
+            }
+            const int c = tid + i * (int)blockDim.x;
+            if (c < chunks) {
+                const int ch = c & 7, R = c >> 3;
+                v4i o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (int)pack_fp8x4(q[4 * e], q[4 * e + 1], q[4 * e + 2], q[4 * e + 3]);
+                *(v4i*)(act + R * 128 + ((ch ^ swz(R)) * 16)) = o;
+                if (ch == 0) act_s[R] = sc * stage_q[i];
+            }
         }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kSlabChunks; ++i) {
+            const int c = tid + i * (int)blockDim.x;
+            if (c < chunks) {
+                const int ch = c & 7, R = c >> 3;
+                *(v4i*)(act + R * 128 + ((ch ^ swz(R)) * 16)) = stage[i];
+            }
+        }
+        if (tid < wg_nkb * M) act_s[tid] = stage_s;
     }
-    if (tid < wg_nkb * M) act_s[tid] = stage_s;
     __syncthreads();
 
     v4f acc[S][MT];
@@ -261,16 +327,16 @@ inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
     return best;
 }
 
-template <int MT, int S>
+template <int MT, int S, bool QF>
 void launch_cfg(const Plan& p, const void* a, const float* a_s, const void* b, const float* b_s,
-                void* out, int out_dtype, int m, int n, int k, hipStream_t st) {
+                void* out, int out_dtype, int m, int n, int k, int ue8m0, hipStream_t st) {
     constexpr int NPF = 8 / S;
     const unsigned groups = (unsigned)((n + 16 * S - 1) / (16 * S));
     const size_t red_bytes = (size_t)p.waves * S * MT * 64 * sizeof(v4f);
     const size_t slab_bytes = ((size_t)p.kb_per_wg * m + 16) * 128 + (size_t)p.kb_per_wg * m * 4;
     const size_t lds = red_bytes > slab_bytes ? red_bytes : slab_bytes;
-    hipLaunchKernelGGL((fp8_gemm_skinny_kernel<MT, S, NPF>), dim3(groups, (unsigned)p.splits), dim3(p.waves * kWave), lds, st,
-                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, out_dtype, m, n, k, p.kb_per_wg);
+    hipLaunchKernelGGL((fp8_gemm_skinny_kernel<MT, S, NPF, QF>), dim3(groups, (unsigned)p.splits), dim3(p.waves * kWave), lds, st,
+                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, out_dtype, m, n, k, p.kb_per_wg, ue8m0);
 }
 
 }  // namespace skinny
@@ -285,15 +351,20 @@ size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t k) {
 }
 
 // Runs the streaming kernel; *splits_out tells the caller how many fp32 slabs were written to `ws`
-// (1 = the result went straight to c).
+// (1 = the result went straight to c).  quant_mode 0: a is fp8 with scales a_s; 1 / 2: a is bf16 and is quantised
+// inside the kernel (scale_fmt none / ue8m0).
 int launch_skinny(const void* a, const float* a_s, const void* b, const float* b_s, void* c, int c_dtype,
-                  int64_t m, int64_t n, int64_t k, void* ws, int* splits_out, hipStream_t st) {
+                  int64_t m, int64_t n, int64_t k, void* ws, int* splits_out, hipStream_t st, int quant_mode) {
     using namespace skinny;
     const Plan p = make_plan(m, n, k);
     void* out = p.splits > 1 ? ws : c;
     const int od = p.splits > 1 ? (int)DSV3_F32 : c_dtype;
     *splits_out = p.splits;
-#define DSV3_CASE(MT_, S_) launch_cfg<MT_, S_>(p, a, a_s, b, b_s, out, od, (int)m, (int)n, (int)k, st); break
+    const int ue = quant_mode == 2;
+#define DSV3_CASE(MT_, S_)                                                                                   \
+    if (quant_mode) launch_cfg<MT_, S_, true>(p, a, a_s, b, b_s, out, od, (int)m, (int)n, (int)k, ue, st);  \
+    else launch_cfg<MT_, S_, false>(p, a, a_s, b, b_s, out, od, (int)m, (int)n, (int)k, 0, st);             \
+    break
     switch (p.mt * 10 + p.s) {
         case 11: DSV3_CASE(1, 1);
         case 12: DSV3_CASE(1, 2);

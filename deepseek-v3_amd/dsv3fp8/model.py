@@ -71,8 +71,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         return F.linear(x, weight, bias)
     if gemm_impl == "bf16":
         return F.linear(x, weight_dequant(weight, weight.scale), bias)
-    xq, xs = act_quant(x, block_size, scale_fmt)
-    y = fp8_gemm(xq, xs, weight, weight.scale)
+    if (x.is_cuda and x.is_contiguous() and weight.is_contiguous() and block_size == 128
+            and x.size(-1) % block_size == 0):
+        # the same two steps behind one op, which runs them as a single launch for few rows (decode)
+        fmt = ops._lib.SCALE_FMT_UE8M0 if scale_fmt == "ue8m0" else ops._lib.SCALE_FMT_NONE
+        y = torch.ops.dsv3fp8.linear_fp8(x, weight, weight.scale, fmt, ops.dtype_code(torch.get_default_dtype()))
+    else:
+        xq, xs = act_quant(x, block_size, scale_fmt)
+        y = fp8_gemm(xq, xs, weight, weight.scale)
     if bias is not None:
         y += bias
     return y

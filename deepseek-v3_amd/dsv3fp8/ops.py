@@ -23,6 +23,7 @@ _libdef = torch.library.Library("dsv3fp8", "DEF")
 _libdef.define("act_quant(Tensor x, int block_size, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("weight_dequant(Tensor x, Tensor s, int block_size, int out_dtype) -> Tensor")
 _libdef.define("fp8_gemm(Tensor a, Tensor a_s, Tensor b, Tensor b_s, int out_dtype) -> Tensor")
+_libdef.define("linear_fp8(Tensor x, Tensor b, Tensor b_s, int scale_fmt, int out_dtype) -> Tensor")
 _libdef.define("group_tiles(Tensor counts, int max_tiles) -> (Tensor, Tensor, Tensor)")
 _libdef.define("moe_route(Tensor indices, Tensor weights, int experts, bool shared_group) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)")
 _libdef.define("fp8_gemm_grouped(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b, Tensor b_s, int rows, "
@@ -106,6 +107,35 @@ def _fp8_gemm_dev(a, a_s, b, b_s, out_dtype: int):
 
 def _fp8_gemm_meta(a, a_s, b, b_s, out_dtype):
     return a.new_empty(*a.size()[:-1], b.size(0), dtype=_CODE_DTYPE[out_dtype])
+
+
+def linear_fp8_fused(m: int, n: int, k: int) -> bool:
+    """Whether act_quant + fp8_gemm of an [m, k] x [n, k] linear run as one launch (dsv3_linear_fp8)."""
+    return bool(_lib.lib.dsv3_linear_fp8_fused(m, n, k))
+
+
+def _linear_fp8_dev(x, b, b_s, scale_fmt: int, out_dtype: int):
+    """act_quant(x, 128, scale_fmt) followed by fp8_gemm, fused where the library implements it, else two calls."""
+    k = x.size(-1)
+    m = x.numel() // k if k else 0
+    n = b.size(0)
+    if not (x.dtype == torch.bfloat16 and linear_fp8_fused(m, n, k)):
+        a, a_s = _act_quant_dev(x, 128, scale_fmt)
+        return _fp8_gemm_dev(a, a_s, b, b_s, out_dtype)
+    c = x.new_empty(*x.size()[:-1], n, dtype=_CODE_DTYPE[out_dtype])
+    with torch.cuda.device(x.device):
+        stream = _stream(x)
+        need = _lib.lib.dsv3_fp8_gemm_workspace_bytes(m, n, k)
+        ws = _workspace(x, need, stream) if need else None
+        rc = _lib.lib.dsv3_linear_fp8(x.data_ptr(), _lib.BF16, b.data_ptr(), b_s.data_ptr(), c.data_ptr(), out_dtype,
+                                      m, n, k, 128, scale_fmt, ws.data_ptr() if ws is not None else None,
+                                      ws.numel() if ws is not None else 0, stream)
+    _lib.check(rc, "dsv3_linear_fp8")
+    return c
+
+
+def _linear_fp8_meta(x, b, b_s, scale_fmt, out_dtype):
+    return x.new_empty(*x.size()[:-1], b.size(0), dtype=_CODE_DTYPE[out_dtype])
 
 
 def grouped_tile_rows() -> int:
@@ -266,6 +296,7 @@ def _wkv_b_absorb_meta(x, wkv_b, scale, side, nope_dim, v_dim):
 
 _libimpl = torch.library.Library("dsv3fp8", "IMPL")
 for _name, _dev, _meta in (("wkv_b_absorb", _wkv_b_absorb_dev, _wkv_b_absorb_meta),
+                           ("linear_fp8", _linear_fp8_dev, _linear_fp8_meta),
                            ("gate_route", _gate_route_dev, _gate_route_meta),
                            ("group_tiles", _group_tiles_dev, _group_tiles_meta),
                            ("moe_route", _moe_route_dev, _moe_route_meta),

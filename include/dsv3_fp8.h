@@ -135,6 +135,18 @@ size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 int dsv3_fp8_gemm_grouped_tile_rows(void);
 
 /*
+ * The FP8 branch of linear() for few rows, act_quant followed by fp8_gemm (inference/model.py:159-160), in one
+ * launch: the weight-streaming kernel quantises the bf16 activations x [m,k] itself, with act_quant's arithmetic
+ * (inference/kernel.py:23-35), so c equals dsv3_act_quant + dsv3_fp8_gemm bit for bit.  Implemented where
+ * dsv3_linear_fp8_fused(m, n, k) returns non-zero (m <= 16 and m*k <= 131072 today); other shapes return DSV3_ERR_BAD_SHAPE and the
+ * caller issues the two calls.  x_dtype must be DSV3_BF16, block_size 128; workspace as for dsv3_fp8_gemm.
+ */
+int dsv3_linear_fp8_fused(int64_t m, int64_t n, int64_t k);
+int dsv3_linear_fp8(const void* x, int x_dtype, const void* b, const float* b_s, void* c, int c_dtype,
+                    int64_t m, int64_t n, int64_t k, int block_size, int scale_fmt,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Tile table for dsv3_fp8_gemm_grouped from per-group row counts (device int32 [groups]; the counts the
  * reference takes from bincount at inference/model.py:683).  Groups are laid out back to back in row order;
  * group g gets ceil(counts[g] / tile_rows) consecutive tile slots.  Writes three device int32 arrays of

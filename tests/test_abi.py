@@ -210,3 +210,25 @@ def test_gate_route_validation(L):
     assert f(*a) == 2
     assert call(0, A16 + 1) == 4 and call(4, A16 + 4) == 4
     assert call(5, 0) == 0
+
+
+def test_linear_fp8_validation(L):
+    f, fused = L.lib.dsv3_linear_fp8, L.lib.dsv3_linear_fp8_fused
+    assert fused(1, 1536, 7168) and fused(8, 7168, 16384) and not fused(16, 7168, 16384) and not fused(17, 1536, 7168)
+    assert not fused(4096, 1536, 7168)
+    assert not fused(4, 1536, 7000) and not fused(0, 8, 128)
+    #     x    dtype   b    b_s  c    cdtype  m  n     k     block fmt ws    ws_bytes stream
+    ok = [A16, L.BF16, A16, A16, A16, L.BF16, 4, 1536, 7168, 128,  0,  A16 * 16, 1 << 30, None]
+
+    def call(i=None, v=None):
+        a = list(ok)
+        if i is not None:
+            a[i] = v
+        return f(*a)
+    assert call(0, None) == 1 and call(2, None) == 1 and call(3, None) == 1 and call(4, None) == 1
+    assert call(1, L.F32) == 5 and call(5, 7) == 5 and call(10, 3) == 5
+    assert call(9, 64) == 3
+    assert call(8, 7000) == 2 and call(6, 64) == 2          # K not a multiple of 128; too many rows for the fused kernel
+    assert call(0, A16 + 2) == 4
+    assert call(11, None) == 6 and call(12, 16) == 6         # the split-K workspace is required and checked
+    assert call(6, 0) == 0

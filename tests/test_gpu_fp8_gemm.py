@@ -198,3 +198,29 @@ def test_asserts_match_reference(K):
         K.fp8_gemm(a.t(), a_s, b, b_s)
     with pytest.raises(AssertionError):
         K.fp8_gemm(a, a_s.t(), b, b_s)
+
+
+@pytest.mark.parametrize("fmt", [None, "ue8m0"])
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+def test_fused_linear_equals_act_quant_then_gemm(K, m, fmt):
+    """dsv3_linear_fp8 (activation quantisation inside the M <= 16 weight-streaming kernel) against the two separate
+    calls, bit for bit, on every decode shape; and the two-step result against the oracle as everywhere else."""
+    from dsv3fp8 import workloads, ops, _lib
+    code_fmt = _lib.SCALE_FMT_UE8M0 if fmt == "ue8m0" else _lib.SCALE_FMT_NONE
+    for name, (k, n) in workloads.DECODE_SHAPES.items():
+        assert ops.linear_fp8_fused(m, n, k) == (m * k <= 131072), name     # beyond that the op issues the two calls
+        x = workloads.activations(m, k, seed=m + n % 7, outliers=True).cuda()
+        w8, ws = workloads.weight(n, k, seed=3)
+        w8, ws = w8.cuda(), ws.cuda()
+        a, a_s = K.act_quant(x, 128, fmt)
+        for code in (_lib.BF16, _lib.F32):
+            two = torch.ops.dsv3fp8.fp8_gemm(a, a_s, w8, ws, code)
+            one = torch.ops.dsv3fp8.linear_fp8(x, w8, ws, code_fmt, code)
+            assert one.dtype == two.dtype and torch.equal(one, two), (name, code)
+    # rows above the fused kernel's range take the two calls inside the op
+    x = workloads.activations(40, 512, seed=1).cuda()
+    w8, ws = workloads.weight(256, 512, seed=2)
+    a, a_s = K.act_quant(x, 128, fmt)
+    assert not ops.linear_fp8_fused(40, 256, 512)
+    assert torch.equal(torch.ops.dsv3fp8.linear_fp8(x, w8.cuda(), ws.cuda(), code_fmt, _lib.F32),
+                       torch.ops.dsv3fp8.fp8_gemm(a, a_s, w8.cuda(), ws.cuda(), _lib.F32))
