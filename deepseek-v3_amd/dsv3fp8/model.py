@@ -193,6 +193,11 @@ class MLA(nn.Module):
     the same bf16 rounding of every dequantised weight.  ``MLA.fused = False`` selects the dequantise-then-einsum
     sequence of the reference instead.  The score / softmax / weighted-sum einsums are bf16 torch operations as
     in the reference: they do not touch FP8 data.
+
+    ``wq_a`` and ``wkv_a`` read the same input.  With FP8 weights (and ``q_lora_rank`` a multiple of the block size,
+    so that both keep their own scale blocks) ``stack_a()`` lays them out as one ``[q_lora_rank + kv_lora_rank +
+    rope, dim]`` weight whose halves the two layers keep as views, and the forward pass runs one linear instead of
+    two (``MLA.stacked_a = False`` keeps them apart).
     """
 
     fused: bool = True
@@ -230,6 +235,26 @@ class MLA(nn.Module):
             self.register_buffer("kv_cache", torch.zeros(b, t, self.kv_lora_rank), persistent=False)
             self.register_buffer("pe_cache", torch.zeros(b, t, self.qk_rope_head_dim), persistent=False)
 
+    stacked_a: bool = True
+
+    def stack_a(self) -> bool:
+        """wq_a over wkv_a in one buffer (scales likewise); returns whether the layers qualify.  Idempotent; the
+        layers' parameters become views, so in-place weight loading keeps working."""
+        if getattr(self, "_wa", None) is not None:
+            return True
+        if self.q_lora_rank == 0 or self.q_lora_rank % block_size or self.wq_a.weight.element_size() != 1 \
+                or self.wkv_a.weight.element_size() != 1 or self.wq_a.scale_fmt != self.wkv_a.scale_fmt:
+            return False
+        qa, ka = self.wq_a, self.wkv_a
+        with torch.no_grad():
+            w = torch.cat([qa.weight.data.view(torch.uint8), ka.weight.data.view(torch.uint8)]).view(qa.weight.dtype)
+            sc = torch.cat([qa.scale.data, ka.scale.data])
+            qa.weight.data, ka.weight.data = w[:qa.out_features], w[qa.out_features:]
+            qa.scale.data, ka.scale.data = sc[:qa.scale.size(0)], sc[qa.scale.size(0):]
+        w.scale = sc
+        self._wa = w
+        return True
+
     def _absorb(self, x: torch.Tensor, side: int, wkv_b: Optional[torch.Tensor]) -> torch.Tensor:
         """One of the two wkv_b products.  ``wkv_b`` is the [h, nope+v, c] bf16 weight for the einsum path, or
         None to read the FP8 weight in place."""
@@ -243,11 +268,17 @@ class MLA(nn.Module):
     def forward(self, x: torch.Tensor, start_pos: int, freqs_cis: torch.Tensor, mask: Optional[torch.Tensor]):
         bsz, seqlen, _ = x.size()
         end_pos = start_pos + seqlen
-        q = self.wq(x) if self.q_lora_rank == 0 else self.wq_b(self.q_norm(self.wq_a(x)))
+        if self.stacked_a and gemm_impl == "fp8" and x.is_cuda and self.stack_a():
+            qa, kva = torch.split(linear(x, self._wa, None, self.wq_a.scale_fmt),
+                                  [self.q_lora_rank, self.kv_lora_rank + self.qk_rope_head_dim], dim=-1)
+            q = self.wq_b(self.q_norm(qa))
+        else:
+            q = self.wq(x) if self.q_lora_rank == 0 else self.wq_b(self.q_norm(self.wq_a(x)))
+            kva = self.wkv_a(x)
         q = q.view(bsz, seqlen, self.n_local_heads, self.qk_head_dim)
         q_nope, q_pe = torch.split(q, [self.qk_nope_head_dim, self.qk_rope_head_dim], dim=-1)
         q_pe = apply_rotary_emb(q_pe, freqs_cis)
-        kv, k_pe = torch.split(self.wkv_a(x), [self.kv_lora_rank, self.qk_rope_head_dim], dim=-1)
+        kv, k_pe = torch.split(kva, [self.kv_lora_rank, self.qk_rope_head_dim], dim=-1)
         k_pe = apply_rotary_emb(k_pe.unsqueeze(2), freqs_cis)
         if attn_impl == "naive":
             q = torch.cat([q_nope, q_pe], dim=-1)

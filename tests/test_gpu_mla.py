@@ -170,6 +170,7 @@ def M():
     model.gemm_impl, model.attn_impl = old[0], old[1]
     model.Linear.dtype = torch.bfloat16
     model.MLA.fused = True
+    model.MLA.stacked_a = True
     torch.set_default_dtype(old[2])
 
 
@@ -219,6 +220,15 @@ def test_mla_prefill_then_decode_vs_oracle(M):
         _close(y0, ref0, 2e-2)
         _close(y1, ref1, 2e-2)
         _close(layer.kv_cache, kv_c, 2e-2)
+        # wq_a and wkv_a ran as one stacked linear; the two layers still see their own weights
+        assert layer._wa is not None and layer.wkv_a.weight.data_ptr() == layer._wa[layer.q_lora_rank:].data_ptr()
+        M.MLA.stacked_a = False
+        layer.kv_cache.zero_(); layer.pe_cache.zero_()
+        u0 = layer(x0.cuda(), 0, freqs[:7].cuda(), mask.cuda())
+        u1 = layer(x1.cuda(), 7, freqs[7:8].cuda(), None)
+        M.MLA.stacked_a = True
+        _close(y0, u0.cpu(), 1e-2)
+        _close(y1, u1.cpu(), 1e-2)
         # the fused products against the reference's dequantise-then-einsum sequence on the same device
         M.MLA.fused = False
         layer.kv_cache.zero_(); layer.pe_cache.zero_()
