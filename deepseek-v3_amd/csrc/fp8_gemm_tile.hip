@@ -294,11 +294,13 @@ int forced_kernel() {
 }
 
 // Which problems go to the large-M kernel (K range cut into slices when the tiles do not fill the chip): every M
-// above 64, and M = 17 .. 64 when the weight is large (>= 96 MiB, e.g. 16384 -> 7168: 32 us against 35 - 42 us of
-// the streaming kernel at M = 32 .. 64; for the smaller decode weights the streaming and tile kernels are faster).
+// above 64, and M = 9 .. 64 when the weight is large (>= 96 MiB).  There it runs at a flat ~30 us per 117-132 MB
+// from 2 to 64 rows, while the M <= 16 streaming kernel grows with M (its K splits multiply with the rows it has
+// to stage: 31 us at 8 rows, 42-50 us at 16) and the M = 32 .. 64 streaming kernel takes 35-42 us; for the
+// smaller decode weights the streaming and tile kernels are faster.
 bool to_large_m_kernel(int64_t m, int64_t n, int64_t k) {
     if (!prefill_supported(m, n, k)) return false;
-    return m > 64 || (m > 16 && n * k >= (96ll << 20));
+    return m > 64 || (m > 8 && n * k >= (96ll << 20));
 }
 
 template <int CD>

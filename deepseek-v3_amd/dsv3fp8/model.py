@@ -320,7 +320,45 @@ class MLP(nn.Module):
         self.w2 = RowParallelLinear(inter_dim, dim)
         self.w3 = ColumnParallelLinear(dim, inter_dim)
 
+    stacked: bool = True
+
+    def stack_13(self) -> bool:
+        """w1 over w3 in one [2*inter, dim] FP8 buffer (scales likewise), the two layers keeping views of it, so
+        that both projections of an input are one GEMM.  Returns whether the layers qualify; re-stacks if the
+        layers' storage was moved since (MoE.stack_experts does that for its shared expert)."""
+        w1, w3 = self.w1, self.w3
+        if w1.weight.element_size() != 1 or w3.weight.element_size() != 1 or w1.out_features % block_size \
+                or w1.in_features % block_size or w1.out_features != w3.out_features:
+            return False
+        w13 = getattr(self, "_w13", None)
+        nbytes = w1.out_features * w1.in_features
+        if w13 is not None and w13.data_ptr() == w1.weight.data_ptr() and w3.weight.data_ptr() == w13.data_ptr() + nbytes:
+            return True
+        with torch.no_grad():
+            if w3.weight.data_ptr() == w1.weight.data_ptr() + nbytes and \
+                    w3.scale.data_ptr() == w1.scale.data_ptr() + w1.scale.numel() * 4:
+                # already adjacent (views of a stacked expert buffer): alias instead of copying
+                w = torch.as_strided(w1.weight.data, (2 * w1.out_features, w1.in_features), (w1.in_features, 1))
+                sc = torch.as_strided(w1.scale.data, (2 * w1.scale.size(0), w1.scale.size(1)), (w1.scale.size(1), 1))
+            else:
+                w = torch.cat([w1.weight.data.view(torch.uint8), w3.weight.data.view(torch.uint8)]).view(w1.weight.dtype)
+                sc = torch.cat([w1.scale.data, w3.scale.data])
+                w1.weight.data, w3.weight.data = w[:w1.out_features], w[w1.out_features:]
+                w1.scale.data, w3.scale.data = sc[:w1.scale.size(0)], sc[w1.scale.size(0):]
+        w.scale = sc
+        self._w13 = w
+        return True
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if (self.stacked and gemm_impl == "fp8" and world_size == 1 and x.is_cuda and x.dtype == torch.bfloat16
+                and x.is_contiguous() and torch.get_default_dtype() == torch.bfloat16 and block_size == 128
+                and self.w2.bias is None and self.w1.bias is None and self.w3.bias is None and self.stack_13()):
+            # one GEMM for both projections, SwiGLU fused with the re-quantisation of w2's input: the same
+            # arithmetic and roundings as the three linears and two tensor ops below
+            h = linear(x, self._w13)
+            gq, gs = torch.ops.dsv3fp8.swiglu_quant(h.view(-1, h.size(-1)), block_size, ops._lib.SCALE_FMT_NONE)
+            y = fp8_gemm(gq, gs, self.w2.weight, self.w2.weight.scale)
+            return y.view(*x.size()[:-1], y.size(-1))
         return self.w2(F.silu(self.w1(x)) * self.w3(x))
 
 

@@ -126,3 +126,26 @@ def test_gate_with_bias_671b_width(M):
     assert all(len(set(r.tolist())) == 8 for r in idx.cpu())
     assert all(len(set((r // 8).tolist())) <= 4 for r in idx.cpu())
     assert torch.allclose(w.float().sum(-1).cpu(), torch.full((32,), 2.5, dtype=torch.float32), atol=0.05)
+
+
+@pytest.mark.parametrize("tokens", [5, 300])
+def test_mlp_stacked_matches_three_linears_and_oracle(M, tokens):
+    """MLP.forward with w1 | w3 as one GEMM and SwiGLU fused with the re-quantisation, against the reference's
+    three linears on the device and against the oracle."""
+    M.gemm_impl = "fp8"
+    with torch.device("cuda"):
+        mlp = M.MLP(256, 384)
+    w1, s1 = _fill(mlp.w1, 1); w2, s2 = _fill(mlp.w2, 2); w3, s3 = _fill(mlp.w3, 3)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(tokens, 256, generator=g).bfloat16()
+    with torch.inference_mode():
+        y = mlp(x.cuda())
+        assert mlp._w13 is not None and mlp.w3.weight.data_ptr() == mlp._w13[384:].data_ptr()
+        M.MLP.stacked = False
+        try:
+            y3 = mlp(x.cuda())
+        finally:
+            M.MLP.stacked = True
+    ref = oracle.mlp(x, w1, s1, w2, s2, w3, s3)
+    _close(y, ref)
+    _close(y, y3.cpu(), tol=1e-2)
