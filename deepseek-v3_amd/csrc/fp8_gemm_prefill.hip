@@ -437,35 +437,56 @@ constexpr int64_t kCUs = 256;
 inline int env_tile_rows() { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }
 }  // namespace
 
-// Few row tiles (M up to a few hundred rows) leave most compute units without a tile: the K range is then cut
-// into slices that run as separate workgroups and write binary32 partial sums, which a second kernel adds in a
-// fixed order.  Worth it while the slices still hold 8 K blocks and the workgroup count stays within one round.
+// Tile height and K slicing.  A K block of a 256-row tile costs about 1.64x one of a 128-row tile (measured,
+// K = 7168), the tiles are dealt over 256 compute units in whole rounds, and when they do not fill a round the K
+// range is cut into up to 8 slices of at least 8 blocks that run as separate workgroups and write binary32 partial
+// sums, which a second kernel adds in a fixed order.  Pick the height (and its slicing) with the lower cost in
+// rounds x K blocks per workgroup x per-block cost.  (M = 4096 x N = 18432: 5 rounds of tall tiles beat 9 of short
+// ones; M = 1024: 3 short rounds beat 2 tall ones; M = 192 ... 256 x N = 18432: 72 tall tiles in 3 slices beat
+// 144 unsliced short ones; M = 128: 72 short tiles in 3 slices.)
+namespace {
+struct PrefillPlan { int tile_rows; int splits; };
+PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
+    const int64_t tn = (n + prefill::BN - 1) / prefill::BN, kb = k / 128;
+    const int forced = env_tile_rows();
+    static const bool nosplit = getenv("DSV3_PREFILL_NOSPLIT") != nullptr;
+    PrefillPlan best{128, 1};
+    int64_t best_cost = -1;
+    for (int h : {128, 256}) {
+        if (forced && forced != h) continue;
+        const int64_t tiles = ((m + h - 1) / h) * tn;
+        int64_t splits = kCUs / tiles;
+        if (splits > kb / 8) splits = kb / 8;
+        if (splits > 8) splits = 8;
+        if (splits < 2 || nosplit) splits = 1;
+        const int64_t per = (kb + splits - 1) / splits, slabs = (kb + per - 1) / per;
+        const int64_t rounds = (tiles * slabs + kCUs - 1) / kCUs;
+        // per-block cost in hundredths of a short tile's (1.14 us); a sliced plan also pays for a second launch
+        // and for writing and re-reading its binary32 slabs (8 bytes per element and slab at ~6 TB/s)
+        int64_t cost = rounds * per * (h == 128 ? 100 : 164);
+        if (slabs > 1) cost += 300 + slabs * m * n * 12 / 100000;
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = PrefillPlan{h, (int)slabs}; }
+    }
+    return best;
+}
+}  // namespace
+
 int prefill_splits(int64_t m, int64_t n, int64_t k) {
     if (m <= 0 || n <= 0 || k < 128) return 1;
-    if (getenv("DSV3_PREFILL_NOSPLIT")) return 1;
-    const int64_t tiles = ((m + 127) / 128) * ((n + prefill::BN - 1) / prefill::BN);
-    int64_t splits = kCUs / tiles;
-    const int64_t kb = k / 128;
-    if (splits > kb / 8) splits = kb / 8;
-    if (splits > 8) splits = 8;
-    return splits < 2 ? 1 : (int)splits;
+    return prefill_plan(m, n, k).splits;
 }
 
+// `splits` must be prefill_splits(m, n, k); with splits > 1, CD is DSV3_F32 and c the slab workspace.
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, int splits, hipStream_t stream) {
-    // Two tile heights.  A round of 256-row tiles over the 256 compute units takes about 1.64x as long as a round
-    // of 128-row tiles (measured, K = 7168), and the last round is rarely full: pick whichever needs less time in
-    // whole rounds.  (M = 4096 x N = 18432: 5 rounds of tall tiles beat 9 of short ones; M = 1024: 3 short rounds
-    // beat 2 tall ones; below ~400 rows the short tile always wins.)
+    const PrefillPlan p = prefill_plan(m, n, k);
+    if (p.splits != splits) return DSV3_ERR_WORKSPACE;
     const int64_t tn = (n + prefill::BN - 1) / prefill::BN;
-    const int64_t tm256 = (m + 255) / 256, tm128 = (m + 127) / 128;
-    auto rounds = [](int64_t tiles) { return (tiles + kCUs - 1) / kCUs; };
-    const int forced = env_tile_rows();
     const prefill::GroupTable none{};
-    if (splits > 1 || forced == 128 || (forced != 256 && 100 * rounds(tm128 * tn) <= 164 * rounds(tm256 * tn)))
-        return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, tm128, 0, tn, none, stream, splits);
-    return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, tm256, 0, tn, none, stream);
+    if (p.tile_rows == 128)
+        return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, (m + 127) / 128, 0, tn, none, stream, splits);
+    return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, (m + 255) / 256, 0, tn, none, stream, splits);
 }
 
 // Rows per tile slot of the grouped kernel: the caller's tile table is built for this height.
