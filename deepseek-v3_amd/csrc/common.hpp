@@ -83,10 +83,10 @@ int launch_skinny(const void* a, const float* a_s, const void* b, const float* b
 int launch_linear_fp8(const void* x, const void* b, const float* b_s, void* c, int c_dtype, int64_t m, int64_t n,
                       int64_t k, int scale_fmt, void* workspace, hipStream_t stream);
 bool linear_fp8_supported(int64_t m, int64_t n, int64_t k);
-int prefill_splits(int64_t m, int64_t n, int64_t k);
+size_t prefill_workspace_bytes(int64_t m, int64_t n, int64_t k);
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
-                   int64_t m, int64_t n, int64_t k, int splits, hipStream_t stream);
+                   int64_t m, int64_t n, int64_t k, void* ws, hipStream_t stream);
 int grouped_tile_rows();
 bool grouped_supported(int64_t a_num_rows, int64_t n, int64_t k);
 template <int CD>

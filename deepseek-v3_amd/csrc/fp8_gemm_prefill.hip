@@ -84,7 +84,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
-        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, GroupTable g) {
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g) {
     using C = Cfg<TM, S>;
     constexpr int WM = C::WM, SM = C::SM, A_LOADS = C::A_LOADS, B_LOADS = C::B_LOADS;
     constexpr int A_STAGE = C::A_STAGE, B_STAGE = C::B_STAGE, LDS_A = C::LDS_A, LDS_B = C::LDS_B, LDS_SC = C::LDS_SC;
@@ -137,7 +137,10 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     const int KBT = K / 128;
     const int kb0 = blockIdx.y * kb_per_split;
     const int KB = min(kb_per_split, KBT - kb0);
-    c += (size_t)blockIdx.y * (size_t)M * (size_t)N;
+    // c has row stride ldc and starts at column tn_first * BN (ldc = N, tn_first = 0 for a plain launch; a slab
+    // of partial sums covers only the launch's column range)
+    c += (size_t)blockIdx.y * (size_t)M * (size_t)ldc;
+    const int n_base = ldc == N ? 0 : tn_first * BN;
     a += (size_t)kb0 * 128u; b += (size_t)kb0 * 128u;
 
     // ---- global -> LDS copy plan: a stage is TM rows of A, then 256 of B, in 1 KiB wavefront-loads of 8 rows;
@@ -369,7 +372,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 #undef DSV3_SGB
 
     // ---- epilogue: lane holds c[m][n .. n+3] for every (i, j)
-    const bool vec_ok = (N % 4) == 0;
+    const bool vec_ok = (N % 4) == 0 && (ldc % 4) == 0;
 #pragma unroll
     for (int j = 0; j < SM; ++j) {
         const int r = sub_row(j) + fr;
@@ -378,7 +381,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 #pragma unroll
         for (int i = 0; i < SN; ++i) {
             const int n = n0 + wn * WN + i * 16 + fq * 4;
-            typename OutT<CD>::type* dst = c + (size_t)m * N + n;
+            typename OutT<CD>::type* dst = c + (size_t)m * ldc + (n - n_base);
             if (vec_ok && n + 3 < N) {
                 if (CD == DSV3_F32) {
                     *(v4f*)dst = acc[i][j];
@@ -410,7 +413,7 @@ namespace {
 template <int CD, bool G, int TM, int S>
 int launch_kernel(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                   int64_t m, int64_t n, int64_t k, int64_t tm, int64_t tn_first, int64_t tn_count,
-                  prefill::GroupTable g, hipStream_t stream, int splits = 1) {
+                  prefill::GroupTable g, hipStream_t stream, int splits = 1, int64_t ldc = 0) {
     using namespace prefill;
     constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
     if ((tm + 8) * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
@@ -429,7 +432,7 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
     hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)((kb + kb_per_split - 1) / kb_per_split)), dim3(THREADS),
                        LDS_BYTES, stream, (const uint8_t*)a, a_s, (const uint8_t*)b, b_s,
                        (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)tm, (int)tn_count, (int)tn_first,
-                       kb_per_split, g);
+                       kb_per_split, (int)(ldc ? ldc : n), g);
     return launch_status();
 }
 constexpr int kGroupedTileRows = 128;
@@ -437,56 +440,128 @@ constexpr int64_t kCUs = 256;
 inline int env_tile_rows() { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }
 }  // namespace
 
-// Tile height and K slicing.  A K block of a 256-row tile costs about 1.64x one of a 128-row tile (measured,
-// K = 7168), the tiles are dealt over 256 compute units in whole rounds, and when they do not fill a round the K
-// range is cut into up to 8 slices of at least 8 blocks that run as separate workgroups and write binary32 partial
-// sums, which a second kernel adds in a fixed order.  Pick the height (and its slicing) with the lower cost in
-// rounds x K blocks per workgroup x per-block cost.  (M = 4096 x N = 18432: 5 rounds of tall tiles beat 9 of short
-// ones; M = 1024: 3 short rounds beat 2 tall ones; M = 192 ... 256 x N = 18432: 72 tall tiles in 3 slices beat
-// 144 unsliced short ones; M = 128: 72 short tiles in 3 slices.)
+// Tile height, K slicing and the last partial round.  A K block of a 256-row tile costs about 1.64x one of a
+// 128-row tile (measured, K = 7168) and the tiles are dealt over 256 compute units in whole rounds.  Three kinds of
+// plan, compared by rounds x K blocks per workgroup x per-block cost:
+//   plain   all tiles in one launch;
+//   sliced  when the tiles do not fill a round: the K range cut into up to 8 slices of at least 8 blocks that run
+//           as separate workgroups and write binary32 partial sums ("slabs"), added in a fixed order by a second
+//           kernel;
+//   hybrid  the column tiles that fill whole rounds as a plain launch, the remaining columns (less than a round
+//           of tiles) as a sliced launch -- instead of a last round that leaves most of the chip idle.
+// (M = 4096 x N = 18432: plain, 5 rounds of tall tiles beat 9 of short ones; M = 1024: hybrid, 256 tall tiles + 32
+// tall tiles in 8 slices; M = 192 ... 256: sliced, 72 tall tiles in 3 slices; M = 128: sliced, 72 short tiles.)
 namespace {
-struct PrefillPlan { int tile_rows; int splits; };
+struct PrefillPlan {
+    int tile_rows;      // 128 or 256
+    int tn_plain;       // column tiles of the plain launch (0: none)
+    int slabs;          // K slices of the remaining column tiles (1 with tn_plain == all: no sliced launch)
+};
+
+// sums `slabs` binary32 slabs [m, w] into columns [n0, n0 + w) of c [m, n]; 4 columns per thread when aligned
+template <int CD>
+__global__ __launch_bounds__(256) void slab_reduce_kernel(
+        const float* __restrict__ ws, typename OutT<CD>::type* __restrict__ c, int64_t m, int w, int64_t n, int n0,
+        int slabs) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;       // element of the [m, w] slab
+    const int64_t mw = m * w;
+    if (i >= mw) return;
+    const int64_t row = i / w;
+    const int col = (int)(i - row * w);
+    typename OutT<CD>::type* dst = c + row * n + n0 + col;
+    if ((w & 3) == 0 && (n & 3) == 0) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < slabs; ++s) v += *(const v4f*)(ws + (int64_t)s * mw + i);
+        if (CD == DSV3_F32) *(v4f*)dst = v;
+        else if (CD == DSV3_BF16) *(v2u*)dst = v2u{ pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]) };
+        else *(v2u*)dst = v2u{ pack_f16(v[0], v[1]), pack_f16(v[2], v[3]) };
+    } else {
+        for (int e = 0; e < 4 && i + e < mw; ++e) {
+            const int64_t r = (i + e) / w;
+            const int cc = (int)(i + e - r * w);
+            float v = 0.f;
+            for (int s = 0; s < slabs; ++s) v += ws[(int64_t)s * mw + i + e];
+            c[r * n + n0 + cc] = cvt_out<CD>(v);
+        }
+    }
+}
+
 PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
     const int64_t tn = (n + prefill::BN - 1) / prefill::BN, kb = k / 128;
     const int forced = env_tile_rows();
     static const bool nosplit = getenv("DSV3_PREFILL_NOSPLIT") != nullptr;
-    PrefillPlan best{128, 1};
+    PrefillPlan best{128, (int)tn, 1};
     int64_t best_cost = -1;
+    auto slices_for = [&](int64_t tiles) {       // K slices that keep `tiles` within one round
+        int64_t s = tiles > 0 ? kCUs / tiles : 1;
+        if (s > kb / 8) s = kb / 8;
+        if (s > 8) s = 8;
+        return (s < 2 || nosplit) ? (int64_t)1 : s;
+    };
+    // a sliced launch also pays for a second launch and for writing and re-reading its binary32 slabs (8 bytes per
+    // element and slab at ~6 TB/s), in hundredths of a short tile's K block (1.14 us)
+    auto slab_cost = [&](int64_t slabs, int64_t cols) { return 300 + slabs * m * cols * 12 / 100000; };
     for (int h : {128, 256}) {
         if (forced && forced != h) continue;
-        const int64_t tiles = ((m + h - 1) / h) * tn;
-        int64_t splits = kCUs / tiles;
-        if (splits > kb / 8) splits = kb / 8;
-        if (splits > 8) splits = 8;
-        if (splits < 2 || nosplit) splits = 1;
-        const int64_t per = (kb + splits - 1) / splits, slabs = (kb + per - 1) / per;
-        const int64_t rounds = (tiles * slabs + kCUs - 1) / kCUs;
-        // per-block cost in hundredths of a short tile's (1.14 us); a sliced plan also pays for a second launch
-        // and for writing and re-reading its binary32 slabs (8 bytes per element and slab at ~6 TB/s)
-        int64_t cost = rounds * per * (h == 128 ? 100 : 164);
-        if (slabs > 1) cost += 300 + slabs * m * n * 12 / 100000;
-        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = PrefillPlan{h, (int)slabs}; }
+        const int64_t unit = h == 128 ? 100 : 164, tm = (m + h - 1) / h, tiles = tm * tn;
+        // plain or sliced over all columns
+        {
+            const int64_t s = slices_for(tiles), per = (kb + s - 1) / s, slabs = (kb + per - 1) / per;
+            int64_t cost = ((tiles * slabs + kCUs - 1) / kCUs) * per * unit;
+            if (slabs > 1) cost += slab_cost(slabs, n);
+            if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = PrefillPlan{h, slabs > 1 ? 0 : (int)tn, (int)slabs}; }
+        }
+        // hybrid: whole rounds plain, the remaining column tiles sliced
+        const int64_t tn_plain = (tiles / kCUs) * kCUs / tm, tn_rest = tn - tn_plain;
+        // (only for launches of up to three rounds: behind more rounds the partial one overlaps the skew of the
+        // full ones, and two serialised launches measured slower -- M = 4096 x N = 18432: 534 against 515 us)
+        if (tn_plain > 0 && tn_rest > 0 && !nosplit && tiles <= 3 * kCUs) {
+            const int64_t s = slices_for(tm * tn_rest), per = (kb + s - 1) / s, slabs = (kb + per - 1) / per;
+            if (slabs > 1) {
+                const int64_t cols = n - tn_plain * prefill::BN;
+                const int64_t cost = ((tm * tn_plain + kCUs - 1) / kCUs) * kb * unit + per * unit + slab_cost(slabs, cols) + 300;
+                if (cost < best_cost) { best_cost = cost; best = PrefillPlan{h, (int)tn_plain, (int)slabs}; }
+            }
+        }
     }
     return best;
 }
 }  // namespace
 
-int prefill_splits(int64_t m, int64_t n, int64_t k) {
-    if (m <= 0 || n <= 0 || k < 128) return 1;
-    return prefill_plan(m, n, k).splits;
+size_t prefill_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+    if (m <= 0 || n <= 0 || k < 128) return 0;
+    const PrefillPlan p = prefill_plan(m, n, k);
+    if (p.slabs <= 1) return 0;
+    const int64_t cols = n - (int64_t)p.tn_plain * prefill::BN;
+    return (size_t)p.slabs * (size_t)m * (size_t)cols * sizeof(float);
 }
 
-// `splits` must be prefill_splits(m, n, k); with splits > 1, CD is DSV3_F32 and c the slab workspace.
+// ws must hold prefill_workspace_bytes(m, n, k) bytes
 template <int CD>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
-                   int64_t m, int64_t n, int64_t k, int splits, hipStream_t stream) {
+                   int64_t m, int64_t n, int64_t k, void* ws, hipStream_t stream) {
     const PrefillPlan p = prefill_plan(m, n, k);
-    if (p.splits != splits) return DSV3_ERR_WORKSPACE;
     const int64_t tn = (n + prefill::BN - 1) / prefill::BN;
+    const int64_t tm = (m + p.tile_rows - 1) / p.tile_rows;
     const prefill::GroupTable none{};
-    if (p.tile_rows == 128)
-        return launch_kernel<CD, false, 128, 3>(a, a_s, b, b_s, c, m, n, k, (m + 127) / 128, 0, tn, none, stream, splits);
-    return launch_kernel<CD, false, 256, 2>(a, a_s, b, b_s, c, m, n, k, (m + 255) / 256, 0, tn, none, stream, splits);
+    auto run = [&](auto cd, void* out, int64_t tn_first, int64_t tn_count, int splits, int64_t ldc) {
+        constexpr int OD = decltype(cd)::value;
+        if (p.tile_rows == 128)
+            return launch_kernel<OD, false, 128, 3>(a, a_s, b, b_s, out, m, n, k, tm, tn_first, tn_count, none, stream, splits, ldc);
+        return launch_kernel<OD, false, 256, 2>(a, a_s, b, b_s, out, m, n, k, tm, tn_first, tn_count, none, stream, splits, ldc);
+    };
+    if (p.tn_plain > 0) {
+        const int rc = run(std::integral_constant<int, CD>{}, c, 0, p.tn_plain, 1, 0);
+        if (rc != DSV3_OK || p.slabs <= 1) return rc;
+    }
+    if (!ws) return DSV3_ERR_WORKSPACE;
+    const int64_t n0 = (int64_t)p.tn_plain * prefill::BN, cols = n - n0;
+    const int rc = run(std::integral_constant<int, DSV3_F32>{}, ws, p.tn_plain, tn - p.tn_plain, p.slabs, cols);
+    if (rc != DSV3_OK) return rc;
+    const int64_t threads = (m * cols + 3) / 4;
+    hipLaunchKernelGGL((slab_reduce_kernel<CD>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                       (const float*)ws, (typename OutT<CD>::type*)c, m, (int)cols, n, (int)n0, p.slabs);
+    return launch_status();
 }
 
 // Rows per tile slot of the grouped kernel: the caller's tile table is built for this height.
@@ -508,7 +583,7 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
 }
 
 #define DSV3_INST(CD) \
-    template int launch_prefill<CD>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, int, hipStream_t); \
+    template int launch_prefill<CD>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, void*, hipStream_t); \
     template int launch_grouped<CD>(const void*, const float*, const int*, const void*, const float*, void*, int64_t, int64_t, int64_t, \
                                     int64_t, const int*, const int*, const int*, int64_t, int64_t, hipStream_t);
 DSV3_INST(DSV3_BF16)

@@ -216,25 +216,6 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(
     c[i] = cvt_out<CD>(v);
 }
 
-// The same for four consecutive elements per thread (mn % 4 == 0): 16-byte loads for the large slabs of the
-// K-split large-M kernel.
-template <int CD>
-__global__ __launch_bounds__(256) void splitk_reduce4_kernel(
-        const v4f* __restrict__ ws, typename OutT<CD>::type* __restrict__ c, int64_t mn4, int splits) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= mn4) return;
-    v4f v = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < splits; ++s) v += ws[(int64_t)s * mn4 + i];
-    if (CD == DSV3_F32) {
-        *(v4f*)(c + 4 * i) = v;
-    } else {
-        v2u o;
-        if (CD == DSV3_BF16) o = v2u{ pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]) };
-        else o = v2u{ pack_f16(v[0], v[1]), pack_f16(v[2], v[3]) };
-        *(v2u*)(c + 4 * i) = o;
-    }
-}
-
 template <int BM, int BN, int WM, int WN, int CD>
 int launch_cfg(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                int64_t m, int64_t n, int64_t k, int splits, int kb_per_split, hipStream_t stream) {
@@ -325,22 +306,7 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
                            (const float*)ws, (typename OutT<CD>::type*)c, mn, splits);
         return launch_status();
     }
-    if (to_prefill) {
-        const int splits = prefill_splits(m, n, k);
-        if (splits == 1) return launch_prefill<CD>(a, a_s, b, b_s, c, m, n, k, 1, st);
-        const int rc = launch_prefill<DSV3_F32>(a, a_s, b, b_s, ws, m, n, k, splits, st);
-        if (rc != DSV3_OK) return rc;
-        const int64_t mn = m * n;
-        const int kb = (int)(k / 128), per = (kb + splits - 1) / splits;
-        const int slabs = (kb + per - 1) / per;
-        if (mn % 4 == 0)
-            hipLaunchKernelGGL((splitk_reduce4_kernel<CD>), dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, st,
-                               (const v4f*)ws, (typename OutT<CD>::type*)c, mn / 4, slabs);
-        else
-            hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
-                               (const float*)ws, (typename OutT<CD>::type*)c, mn, slabs);
-        return launch_status();
-    }
+    if (to_prefill) return launch_prefill<CD>(a, a_s, b, b_s, c, m, n, k, ws, st);
     const Plan p = make_plan(m, n, k);
     if (p.splits == 1) {
         if (p.bm == 32) return launch_cfg<32, 128, 32, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
@@ -390,10 +356,7 @@ size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
     size_t need = tile_ws;
     if (skinny_supported(m, n, k) && skinny_workspace_bytes(m, n, k) > need) need = skinny_workspace_bytes(m, n, k);
     if (stream_supported(m, n, k) && stream_workspace_bytes(m, n, k) > need) need = stream_workspace_bytes(m, n, k);
-    if (to_large_m_kernel(m, n, k) && prefill_splits(m, n, k) > 1) {
-        const size_t pre = (size_t)prefill_splits(m, n, k) * (size_t)m * (size_t)n * sizeof(float);
-        if (pre > need) need = pre;
-    }
+    if (to_large_m_kernel(m, n, k) && prefill_workspace_bytes(m, n, k) > need) need = prefill_workspace_bytes(m, n, k);
     return need;
 }
 

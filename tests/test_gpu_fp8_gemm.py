@@ -224,3 +224,15 @@ def test_fused_linear_equals_act_quant_then_gemm(K, m, fmt):
     assert not ops.linear_fp8_fused(40, 256, 512)
     assert torch.equal(torch.ops.dsv3fp8.linear_fp8(x, w8.cuda(), ws.cuda(), code_fmt, _lib.F32),
                        torch.ops.dsv3fp8.fp8_gemm(a, a_s, w8.cuda(), ws.cuda(), _lib.F32))
+
+
+@pytest.mark.parametrize("m,n,k", [
+    (1024, 18432, 4096),   # 4 x 72 tall tiles: 256 of them as a plain launch, the last 8 column tiles in 4 K slices
+    (1030, 17000, 4096),   # ragged M and N: 5 x 67 tall tiles, the sliced part ends in a 104-column tile
+])
+def test_hybrid_plan_whole_rounds_plus_sliced_rest(K, m, n, k):
+    from dsv3fp8 import workloads, _lib
+    assert _lib.lib.dsv3_fp8_gemm_workspace_bytes(m, n, k) > 0
+    x = workloads.activations(m, k, seed=m)
+    w8, ws = workloads.weight(n, k, seed=n % 89)
+    _check(K, x, w8, ws)
