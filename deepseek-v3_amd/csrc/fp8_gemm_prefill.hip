@@ -363,16 +363,51 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         __builtin_amdgcn_s_waitcnt(0x0f70);             // the clamped refills of the last blocks are still in flight
         }
     };
+    // 16-bit outputs with full-width rows are stored through LDS (see the epilogue)
+    const bool lds_epilogue = CD != DSV3_F32 && (N % 8) == 0 && ldc == N;
     static_assert(SM == 4 || SM == 2, "dispatch below");
     if (!G || ja_live == SM) pipeline(std::integral_constant<int, SM>{});
     else if (SM == 4 && ja_live == 3) pipeline(std::integral_constant<int, (SM == 4 ? 3 : 1)>{});
     else if (SM == 4 && ja_live == 2) pipeline(std::integral_constant<int, (SM == 4 ? 2 : 1)>{});
     else if (ja_live == 1)  pipeline(std::integral_constant<int, 1>{});
-    else { pipeline(std::integral_constant<int, 0>{}); return; }
+    else {
+        pipeline(std::integral_constant<int, 0>{});
+        if (lds_epilogue) wg_barrier();     // the barrier the other wavefronts take before they reuse the LDS stages
+        return;
+    }
 #undef DSV3_SGB
 
     // ---- epilogue: lane holds c[m][n .. n+3] for every (i, j)
     const bool vec_ok = (N % 4) == 0 && (ldc % 4) == 0;
+    if (lds_epilogue) {
+        // 16-bit outputs go through LDS (free now: one barrier, then a private 256-byte-per-row region per
+        // wavefront) so that a store instruction writes 4 rows x 256 contiguous bytes instead of 16 rows x four
+        // 8-byte pieces.  16-byte chunks are xor-ed with the row, which spreads both the 8-byte writes of the 16 rows
+        // of a sub-tile and the 16-byte reads of a row over all banks.
+        wg_barrier();
+        uint8_t* stg = lds + wave * (WM * 256);
+#pragma unroll
+        for (int j = 0; j < SM; ++j)
+#pragma unroll
+            for (int i = 0; i < SN; ++i) {
+                v2u o;
+                if (CD == DSV3_BF16) o = v2u{ pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3]) };
+                else o = v2u{ pack_f16(acc[i][j][0], acc[i][j][1]), pack_f16(acc[i][j][2], acc[i][j][3]) };
+                const int lr = j * 16 + fr, chunk = (i * 2 + (fq >> 1)) ^ fr;
+                *(v2u*)(stg + lr * 256 + chunk * 16 + (fq & 1) * 8) = o;
+            }
+        const int rr = lane >> 4, ch = lane & 15;
+#pragma unroll
+        for (int p = 0; p < WM / 4; ++p) {
+            const int lr = p * 4 + rr;                                   // local row: sub-tile lr / 16, row lr % 16
+            const v4u v = *(const v4u*)(stg + lr * 256 + ((ch ^ (lr & 15)) * 16));
+            const int r = sub_row(lr >> 4) + (lr & 15);
+            const int n = n0 + wn * WN + ch * 8;
+            if (r < rows_here && n < N)                                   // N % 8 == 0: a chunk is inside or outside
+                *(v4u*)(c + (size_t)(m0 + r) * N + n) = v;
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < SM; ++j) {
         const int r = sub_row(j) + fr;
