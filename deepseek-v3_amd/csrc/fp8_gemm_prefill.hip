@@ -365,6 +365,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     };
     // 16-bit outputs with full-width rows are stored through LDS (see the epilogue)
     const bool lds_epilogue = CD != DSV3_F32 && (N % 8) == 0 && ldc == N;
+    const bool f32_lds_epilogue = CD == DSV3_F32 && (N % 4) == 0 && (ldc % 4) == 0 && (SN % 2) == 0;
     static_assert(SM == 4 || SM == 2, "dispatch below");
     if (!G || ja_live == SM) pipeline(std::integral_constant<int, SM>{});
     else if (SM == 4 && ja_live == 3) pipeline(std::integral_constant<int, (SM == 4 ? 3 : 1)>{});
@@ -372,7 +373,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     else if (ja_live == 1)  pipeline(std::integral_constant<int, 1>{});
     else {
         pipeline(std::integral_constant<int, 0>{});
-        if (lds_epilogue) wg_barrier();     // the barrier the other wavefronts take before they reuse the LDS stages
+        if (lds_epilogue || f32_lds_epilogue) wg_barrier();     // the barrier the other wavefronts take before they reuse the LDS stages
         return;
     }
 #undef DSV3_SGB
@@ -405,6 +406,34 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
             const int n = n0 + wn * WN + ch * 8;
             if (r < rows_here && n < N)                                   // N % 8 == 0: a chunk is inside or outside
                 *(v4u*)(c + (size_t)(m0 + r) * N + n) = v;
+        }
+        return;
+    }
+    if (f32_lds_epilogue) {
+        // The same for fp32 results (the slabs of a K slice, mostly), half of the wavefront's columns per pass so that
+        // the region stays at 256 bytes per row: a store instruction then writes 4 rows x 256 contiguous bytes
+        // instead of 16 rows x 64.
+        wg_barrier();
+        uint8_t* stg = lds + wave * (WM * 256);
+        const int rr = lane >> 4, ch = lane & 15;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int j = 0; j < SM; ++j)
+#pragma unroll
+                for (int i = 0; i < SN / 2; ++i) {
+                    const int lr = j * 16 + fr, chunk = (i * 4 + fq) ^ fr;
+                    *(v4f*)(stg + lr * 256 + chunk * 16) = acc[h * (SN / 2) + i][j];
+                }
+#pragma unroll
+            for (int p = 0; p < WM / 4; ++p) {
+                const int lr = p * 4 + rr;
+                const v4f v = *(const v4f*)(stg + lr * 256 + ((ch ^ (lr & 15)) * 16));
+                const int r = sub_row(lr >> 4) + (lr & 15);
+                const int n = n0 + wn * WN + h * (WN / 2) + ch * 4;
+                if (r < rows_here && n < N)                               // N % 4 == 0: a chunk is inside or outside
+                    *(v4f*)(c + (size_t)(m0 + r) * ldc + (n - n_base)) = v;
+            }
         }
         return;
     }
