@@ -151,6 +151,7 @@ def run_extras(K, W):
         del wqs
     out["linear_decode"] = lin
     out["moe_layer_T4096"] = run_moe(K, W)
+    out["moe_layer_T4096_balanced"] = run_moe(K, W, bias_std=0.0, expert_loop=False)
     out["wkv_b_absorb"] = run_absorb(K, W)
     return out
 
@@ -184,12 +185,17 @@ def run_absorb(K, W, token_counts=(1, 16, 64, 128, 4096)):
     return res
 
 
-def run_moe(K, W, tokens: int = 4096):
+def run_moe(K, W, tokens: int = 4096, bias_std: float = 0.1, expert_loop: bool = True):
     """The MoE-layer configuration: one MoE layer (256 routed + 1 shared SwiGLU experts, 7168 -> 2048 -> 7168, fp8
     block-scaled weights generated on the device), T tokens, sigmoid gate with bias over random logits'
     weights, 8 groups / top-4 groups / top-8 experts, route_scale 2.5.  Timed twice: the grouped path
     (device-side token lists, two grouped GEMMs, fused SwiGLU + re-quantisation, ordered combine) and the
-    reference's host-driven pass over the experts' token lists (model.py:679-693) on the same kernels."""
+    reference's host-driven pass over the experts' token lists (model.py:679-693) on the same kernels.
+
+    The logits have a standard deviation of 1.7, so the best sigmoid scores of a token lie within 0.04 of 1 and a
+    bias drawn with bias_std = 0.1 decides most of the selection: the load is skewed (a third of the experts get no
+    token, the busiest about 1100 of the 32768 rows).  bias_std = 0 gives the balanced load a trained router aims
+    for (97 .. 161 rows per expert), in which every expert's weights are streamed.  The result names the load."""
     from dsv3fp8 import model as Mdl
     old = Mdl.gemm_impl, Mdl.Linear.dtype, Mdl.MoE.grouped
     Mdl.gemm_impl, Mdl.Linear.dtype = "fp8", torch.float8_e4m3fn
@@ -200,7 +206,7 @@ def run_moe(K, W, tokens: int = 4096):
         g = torch.Generator(device="cuda").manual_seed(5)
         with torch.no_grad():
             moe.gate.weight.copy_(torch.randn(args.n_routed_experts, args.dim, generator=g, device="cuda") * 0.02)
-            moe.gate.bias.copy_(torch.randn(args.n_routed_experts, generator=g, device="cuda") * 0.1)
+            moe.gate.bias.copy_(torch.randn(args.n_routed_experts, generator=g, device="cuda") * bias_std)
             protos = [W.weight(args.moe_inter_dim, args.dim, 40, "cuda"), W.weight(args.dim, args.moe_inter_dim, 41, "cuda")]
             for ex in list(moe.experts) + [moe.shared_experts]:
                 for lin, (w8, sc) in ((ex.w1, protos[0]), (ex.w3, protos[0]), (ex.w2, protos[1])):
@@ -209,10 +215,14 @@ def run_moe(K, W, tokens: int = 4096):
         moe.stack_experts()
         x = W.activations(tokens, args.dim, 6, "cuda")
         flops = 2.0 * 3 * args.dim * args.moe_inter_dim * (tokens * args.n_activated_experts + tokens)
-        wbytes = 257 * 3 * args.dim * args.moe_inter_dim
         res = {}
         with torch.inference_mode():
-            for key, grouped, steps in (("grouped", True, 10), ("expert_loop", False, 2)):
+            counts = torch.bincount(moe.gate(x)[1].reshape(-1), minlength=args.n_routed_experts)
+            hit = int((counts > 0).sum())
+            res["load"] = {"bias_std": bias_std, "experts_with_tokens": hit,
+                           "rows_per_expert_min_mean_max": [int(counts.min()), float(counts.float().mean()), int(counts.max())]}
+            wbytes = (hit + 1) * 3 * args.dim * args.moe_inter_dim      # weights of the experts that get a token
+            for key, grouped, steps in (("grouped", True, 10), ("expert_loop", False, 2))[:2 if expert_loop else 1]:
                 Mdl.MoE.grouped = grouped
                 ms = time_loop(lambda: moe(x), steps, 2 if grouped else 1)
                 res[key] = {"ms": round(ms, 3), "TFLOPs": round(flops / ms / 1e9, 1),

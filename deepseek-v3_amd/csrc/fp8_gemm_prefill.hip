@@ -79,8 +79,9 @@ struct GroupTable {
     int64_t bs_stride;       // floats between consecutive groups' weight scales
 };
 
+// One workgroup's tile (grouped mode: tile slot) from start to end; the kernels below are thin wrappers.
 template <int CD, bool G, int TM, int S>
-__global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
+__device__ __forceinline__ void prefill_tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
@@ -465,6 +466,33 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     }
 }
 
+template <int CD, bool G, int TM, int S>
+__global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c,
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g) {
+    prefill_tile<CD, G, TM, S>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g);
+}
+
+// Grouped GEMM over a tile table with slots of up to 256 rows.  A slot with more than 128 rows runs the 256-row
+// configuration (the weights pass through LDS once for up to 256 rows); one with fewer runs the 128-row
+// configuration with its deeper prefetch.  The choice is uniform over the workgroup and needs no host knowledge of
+// the group sizes: a layer with a few rows per expert and one with hundreds go through the same launch.
+template <int CD>
+__global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c,
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g) {
+    const int idx = blockIdx.x / 8, tm = (idx / tiles_n) * 8 + blockIdx.x % 8;
+    if (tm >= tiles_m) return;
+    if (g.tile_rows[tm] > 128)
+        prefill_tile<CD, true, 256, 2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g);
+    else
+        prefill_tile<CD, true, 128, 3>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g);
+}
+
 }  // namespace prefill
 
 // Usable when the row offsets fit 32 bits; the caller falls back to the generic tile kernel otherwise.
@@ -499,7 +527,7 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
                        kb_per_split, (int)(ldc ? ldc : n), g);
     return launch_status();
 }
-constexpr int kGroupedTileRows = 128;
+constexpr int kGroupedTileRows = 256;     // slot height of the grouped kernel's tile table
 constexpr int64_t kCUs = 256;
 inline int env_tile_rows() { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }
 }  // namespace
@@ -641,9 +669,26 @@ template <int CD>
 int launch_grouped(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
                    const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream) {
-    prefill::GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
-    return launch_kernel<CD, true, kGroupedTileRows, 3>(a, a_s, b, b_s, c, m, n, k, num_tiles, 0,
-                                                          (n + prefill::BN - 1) / prefill::BN, g, stream);
+    using namespace prefill;
+    GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
+    constexpr int LDS_BYTES = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
+    const int64_t tn = (n + BN - 1) / BN;
+    if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (num_tiles * tn == 0) return DSV3_OK;
+    auto kern = fp8_gemm_grouped_kernel<CD>;
+    static bool granted[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
+    if (!granted[dev]) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
+            return DSV3_ERR_LAUNCH;
+        granted[dev] = true;
+    }
+    const int64_t grid = (num_tiles + 7) / 8 * 8 * tn;                  // row tiles are dealt over the 8 XCDs
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
+                       (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)num_tiles,
+                       (int)tn, 0, (int)(k / 128), (int)n, g);
+    return launch_status();
 }
 
 #define DSV3_INST(CD) \

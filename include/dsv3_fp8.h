@@ -131,7 +131,9 @@ size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
  * summed per token in ascending expert order, rounding to bf16 where the reference's tensor ops round.
  */
 
-/* Height of a row tile of dsv3_fp8_gemm_grouped; dsv3_group_tiles cuts groups into tiles of this many rows. */
+/* Height of a tile slot of dsv3_fp8_gemm_grouped (256 today); dsv3_group_tiles cuts groups into slots of at most
+ * this many rows.  The kernel runs a slot of more than 128 rows as one 256-row tile and a smaller one as a 128-row
+ * tile, so one table serves a few rows per group as well as hundreds. */
 int dsv3_fp8_gemm_grouped_tile_rows(void);
 
 /*

@@ -56,6 +56,7 @@ def _grouped_case(counts, n, k, seed, gather):
     ([5, 0, 300, 256, 1], 384, 512, True),
     ([129, 64], 576, 256, False),            # ragged n: 576 = 2 tiles + 64, 5 scale rows
     ([40] * 6, 256, 1152, True),             # odd number of K blocks
+    ([145, 177, 200, 241, 17], 512, 384, True),   # 256-row slots with 10, 12, 13 and 16 live sub-tiles, then a small one
 ])
 def test_fp8_gemm_grouped_vs_oracle(K, counts, n, k, gather):
     from dsv3fp8 import ops
