@@ -85,7 +85,8 @@ __device__ __forceinline__ void prefill_tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
-        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g) {
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g,
+        int wg) {                           // index of the workgroup among those that run this configuration
     using C = Cfg<TM, S>;
     constexpr int WM = C::WM, SM = C::SM, A_LOADS = C::A_LOADS, B_LOADS = C::B_LOADS;
     constexpr int A_STAGE = C::A_STAGE, B_STAGE = C::B_STAGE, LDS_A = C::LDS_A, LDS_B = C::LDS_B, LDS_SC = C::LDS_SC;
@@ -98,7 +99,7 @@ __device__ __forceinline__ void prefill_tile(
     // tile on one XCD (they share the gathered rows of a).
     int m0, n0, rows_here;              // first row of the tile in c, first column, valid rows
     if (G) {
-        const int x = blockIdx.x % 8, idx = blockIdx.x / 8;
+        const int x = wg % 8, idx = wg / 8;
         const int tm = (idx / tiles_n) * 8 + x, tn = idx - (idx / tiles_n) * tiles_n;
         if (tm >= tiles_m) return;      // uniform over the workgroup, before any barrier
         const int grp = g.tile_group[tm];
@@ -110,7 +111,7 @@ __device__ __forceinline__ void prefill_tile(
         b_s += (size_t)grp * g.bs_stride;
     } else {
         const int T = tiles_m * tiles_n;
-        int pid = blockIdx.x;
+        int pid = wg;
         {
             const int q = T / 8, r = T % 8, x = pid % 8;
             pid = x * q + (x < r ? x : r) + pid / 8;
@@ -472,7 +473,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
         int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g) {
-    prefill_tile<CD, G, TM, S>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g);
+    prefill_tile<CD, G, TM, S>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
 }
 
 // Grouped GEMM over a tile table with slots of up to 256 rows.  A slot with more than 128 rows runs the 256-row
@@ -488,9 +489,28 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
     const int idx = blockIdx.x / 8, tm = (idx / tiles_n) * 8 + blockIdx.x % 8;
     if (tm >= tiles_m) return;
     if (g.tile_rows[tm] > 128)
-        prefill_tile<CD, true, 256, 2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g);
+        prefill_tile<CD, true, 256, 2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
     else
-        prefill_tile<CD, true, 128, 3>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g);
+        prefill_tile<CD, true, 128, 3>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+}
+
+// Dense GEMM whose last column tiles run as 128-row tiles: the first tiles_m * tn_tall workgroups compute 256-row
+// tiles over the column tiles [0, tn_tall), the others 128-row tiles over [tn_tall, tn_tall + tn_short).  Workgroups
+// are handed out in index order, so the short tiles fill the compute units that the last, partly filled round of
+// tall tiles would leave idle.
+template <int CD>
+__global__ __launch_bounds__(THREADS, 1) void fp8_gemm_two_heights_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c, int M, int N, int K, int tn_tall, int tn_short) {
+    const int tm_tall = (M + 255) / 256, n_tall = tm_tall * tn_tall;
+    const int short_first = (n_tall + 7) & ~7;        // keeps workgroup index % 8 = XCD for the short tiles too
+    const GroupTable none{};
+    if ((int)blockIdx.x < n_tall)
+        prefill_tile<CD, false, 256, 2>(a, a_s, b, b_s, c, M, N, K, tm_tall, tn_tall, 0, K / 128, N, none, blockIdx.x);
+    else if ((int)blockIdx.x >= short_first)
+        prefill_tile<CD, false, 128, 3>(a, a_s, b, b_s, c, M, N, K, (M + 127) / 128, tn_short, tn_tall, K / 128, N, none,
+                                        blockIdx.x - short_first);
 }
 
 }  // namespace prefill
@@ -548,6 +568,8 @@ struct PrefillPlan {
     int tile_rows;      // 128 or 256
     int tn_plain;       // column tiles of the plain launch (0: none)
     int slabs;          // K slices of the remaining column tiles (1 with tn_plain == all: no sliced launch)
+    int tn_short;       // two heights: the last tn_short column tiles run as 128-row tiles in the same launch as the
+                        // tn_plain tall ones (tile_rows == 256, slabs == 1); 0 otherwise
 };
 
 // sums `slabs` binary32 slabs [m, w] into columns [n0, n0 + w) of c [m, n]; 4 columns per thread when aligned
@@ -582,7 +604,7 @@ PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
     const int64_t tn = (n + prefill::BN - 1) / prefill::BN, kb = k / 128;
     const int forced = env_tile_rows();
     static const bool nosplit = getenv("DSV3_PREFILL_NOSPLIT") != nullptr;
-    PrefillPlan best{128, (int)tn, 1};
+    PrefillPlan best{128, (int)tn, 1, 0};
     int64_t best_cost = -1;
     auto slices_for = [&](int64_t tiles) {       // K slices that keep `tiles` within one round
         int64_t s = tiles > 0 ? kCUs / tiles : 1;
@@ -601,7 +623,7 @@ PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
             const int64_t s = slices_for(tiles), per = (kb + s - 1) / s, slabs = (kb + per - 1) / per;
             int64_t cost = ((tiles * slabs + kCUs - 1) / kCUs) * per * unit;
             if (slabs > 1) cost += slab_cost(slabs, n);
-            if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = PrefillPlan{h, slabs > 1 ? 0 : (int)tn, (int)slabs}; }
+            if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = PrefillPlan{h, slabs > 1 ? 0 : (int)tn, (int)slabs, 0}; }
         }
         // hybrid: whole rounds plain, the remaining column tiles sliced
         const int64_t tn_plain = (tiles / kCUs) * kCUs / tm, tn_rest = tn - tn_plain;
@@ -612,8 +634,29 @@ PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
             if (slabs > 1) {
                 const int64_t cols = n - tn_plain * prefill::BN;
                 const int64_t cost = ((tm * tn_plain + kCUs - 1) / kCUs) * kb * unit + per * unit + slab_cost(slabs, cols) + 300;
-                if (cost < best_cost) { best_cost = cost; best = PrefillPlan{h, (int)tn_plain, (int)slabs}; }
+                if (cost < best_cost) { best_cost = cost; best = PrefillPlan{h, (int)tn_plain, (int)slabs, 0}; }
             }
+        }
+    }
+    // two heights: the last c column tiles as short tiles behind the tall ones, in one launch.  Workgroups start in
+    // index order on the first free compute unit: the tall tiles leave r units with q + 1 tiles and the others with
+    // q; the short tiles then fill up from the least loaded unit.
+    if (!forced && !nosplit && m > 128) {
+        const int64_t tm_tall = (m + 255) / 256, tm_short = (m + 127) / 128;
+        for (int64_t c = 1; c < tn && c <= 32; ++c) {
+            const int64_t n_tall = tm_tall * (tn - c), n_short = tm_short * c;
+            const int64_t q = n_tall / kCUs, r = n_tall % kCUs;
+            // kCUs - r units carry lo = q * 164, r units hi = lo + 164; the short tiles (100 each) go to whichever
+            // unit is free first, level by level
+            const int64_t lo = q * 164, hi = lo + 164;
+            int64_t t = lo, t_lo = lo + 100, t_hi = hi + 100, done = 0;
+            while (done < n_short) {
+                if (r == 0 || t_lo <= t_hi) { t = t_lo; t_lo += 100; done += kCUs - r; }
+                else                        { t = t_hi; t_hi += 100; done += r; }
+            }
+            const int64_t span = (r > 0 && hi > t) ? hi : t;
+            const int64_t cost = span * kb + 100;                // (a little extra: prefer one height at equal cost)
+            if (cost * 100 < best_cost * 97) { best_cost = cost; best = PrefillPlan{256, (int)(tn - c), 1, (int)c}; }
         }
     }
     return best;
@@ -636,6 +679,25 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
     const int64_t tn = (n + prefill::BN - 1) / prefill::BN;
     const int64_t tm = (m + p.tile_rows - 1) / p.tile_rows;
     const prefill::GroupTable none{};
+    if (p.tn_short > 0) {
+        using namespace prefill;
+        constexpr int LDS_BYTES = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
+        auto kern = fp8_gemm_two_heights_kernel<CD>;
+        static bool granted[64] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
+        if (!granted[dev]) {
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
+                return DSV3_ERR_LAUNCH;
+            granted[dev] = true;
+        }
+        const int64_t n_tall = (m + 255) / 256 * p.tn_plain;
+        const int64_t grid = (n_tall + 7) / 8 * 8 + (m + 127) / 128 * p.tn_short;
+        if (grid > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
+                           (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, p.tn_plain, p.tn_short);
+        return launch_status();
+    }
     auto run = [&](auto cd, void* out, int64_t tn_first, int64_t tn_count, int splits, int64_t ldc) {
         constexpr int OD = decltype(cd)::value;
         if (p.tile_rows == 128)

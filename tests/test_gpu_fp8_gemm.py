@@ -226,13 +226,18 @@ def test_fused_linear_equals_act_quant_then_gemm(K, m, fmt):
                        torch.ops.dsv3fp8.fp8_gemm(a, a_s, w8.cuda(), ws.cuda(), _lib.F32))
 
 
-@pytest.mark.parametrize("m,n,k", [
-    (1024, 18432, 4096),   # 4 x 72 tall tiles: 256 of them as a plain launch, the last 8 column tiles in 4 K slices
-    (1030, 17000, 4096),   # ragged M and N: 5 x 67 tall tiles, the sliced part ends in a 104-column tile
+@pytest.mark.parametrize("m,n,k,sliced", [
+    (1024, 18432, 4096, True),    # 4 x 72 tall tiles: 256 of them as a plain launch, the last 8 column tiles in 4 K slices
+    (1030, 17000, 4096, False),   # ragged M and N, 5 x 67 tall tiles: the last column tiles (one of 104 columns) as
+                                  # 128-row tiles behind the tall ones, in one launch
+    (1280, 18432, 1024, False),   # K too short to slice: 5 x 72 tall tiles, a partly filled second round
+    (2100, 9000, 640, False),     # 9 x 36 tall tiles, ragged both ways, odd number of K blocks
 ])
-def test_hybrid_plan_whole_rounds_plus_sliced_rest(K, m, n, k):
+def test_partly_filled_last_round(K, m, n, k, sliced):
+    """Launches of more than one round of tiles whose last round is partly filled: the planner either cuts the K
+    range of the remaining column tiles into slices or runs them as short tiles behind the tall ones."""
     from dsv3fp8 import workloads, _lib
-    assert _lib.lib.dsv3_fp8_gemm_workspace_bytes(m, n, k) > 0
+    assert (_lib.lib.dsv3_fp8_gemm_workspace_bytes(m, n, k) > 0) == sliced
     x = workloads.activations(m, k, seed=m)
     w8, ws = workloads.weight(n, k, seed=n % 89)
     _check(K, x, w8, ws)
