@@ -122,6 +122,11 @@ def run_extras(K, W):
     out["weight_dequant_18432x7168"] = {"us": round(us, 2), "GBps": round(396.394e6 / us / 1e3, 1),
                                         "hbm_frac": round(396.394e6 / us / 1e3 / HBM_PEAK_GBS, 3)}
     del ws_, w8
+    wb = [(torch.randn(18432, 7168, device="cuda") * 0.02).bfloat16() for _ in range(4)]   # 4 x 264 MB
+    us = time_graph([(lambda t=t: K.weight_quant(t)) for t in wb] * 2)
+    out["weight_quant_18432x7168"] = {"us": round(us, 2), "GBps": round(396.394e6 / us / 1e3, 1),
+                                      "hbm_frac": round(396.394e6 / us / 1e3 / HBM_PEAK_GBS, 3)}
+    del wb
     k, n = W.PREFILL_SHAPES["w2"]
     a, a_s = K.act_quant(W.activations(4096, k, 0, "cuda"))
     wq, wsc = W.weight(n, k, 1, "cuda")

@@ -1,6 +1,6 @@
 """PyTorch-ROCm custom ops over the C ABI.
 
-``torch.ops.dsv3fp8.{act_quant, weight_dequant, fp8_gemm}`` and the grouped
+``torch.ops.dsv3fp8.{act_quant, weight_dequant, weight_quant, fp8_gemm}`` and the grouped
 mixture-of-experts ops ``{gate_route, group_tiles, moe_route, fp8_gemm_grouped, swiglu_quant, moe_combine}`` and the
 attention op ``wkv_b_absorb`` take and return torch tensors; the device implementations hand raw device pointers and the
 current HIP stream of the tensors' device to libdsv3fp8.so.  Only a device
@@ -22,6 +22,7 @@ FP8 = torch.float8_e4m3fn
 _libdef = torch.library.Library("dsv3fp8", "DEF")
 _libdef.define("act_quant(Tensor x, int block_size, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("weight_dequant(Tensor x, Tensor s, int block_size, int out_dtype) -> Tensor")
+_libdef.define("weight_quant(Tensor w, int block_size) -> (Tensor, Tensor)")
 _libdef.define("fp8_gemm(Tensor a, Tensor a_s, Tensor b, Tensor b_s, int out_dtype) -> Tensor")
 _libdef.define("linear_fp8(Tensor x, Tensor b, Tensor b_s, int scale_fmt, int out_dtype) -> Tensor")
 _libdef.define("group_tiles(Tensor counts, int max_tiles) -> (Tensor, Tensor, Tensor)")
@@ -86,6 +87,22 @@ def _weight_dequant_dev(x: torch.Tensor, s: torch.Tensor, block_size: int, out_d
 
 def _weight_dequant_meta(x, s, block_size, out_dtype):
     return torch.empty_like(x, dtype=_CODE_DTYPE[out_dtype])
+
+
+def _weight_quant_dev(w: torch.Tensor, block_size: int):
+    m, n = w.size()
+    y = torch.empty_like(w, dtype=FP8)
+    s = w.new_empty(-(-m // block_size), -(-n // block_size), dtype=torch.float32)
+    with torch.cuda.device(w.device):
+        rc = _lib.lib.dsv3_weight_quant(w.data_ptr(), dtype_code(w.dtype), y.data_ptr(), s.data_ptr(), m, n,
+                                        block_size, _stream(w))
+    _lib.check(rc, "dsv3_weight_quant")
+    return y, s
+
+
+def _weight_quant_meta(w, block_size):
+    m, n = w.size()
+    return torch.empty_like(w, dtype=FP8), w.new_empty(-(-m // block_size), -(-n // block_size), dtype=torch.float32)
 
 
 def _fp8_gemm_dev(a, a_s, b, b_s, out_dtype: int):
@@ -307,7 +324,9 @@ for _name, _dev, _meta in (("wkv_b_absorb", _wkv_b_absorb_dev, _wkv_b_absorb_met
     _libimpl.impl(_name, _meta, "Meta")
 _libimpl.impl("act_quant", _act_quant_dev, "CUDA")
 _libimpl.impl("weight_dequant", _weight_dequant_dev, "CUDA")
+_libimpl.impl("weight_quant", _weight_quant_dev, "CUDA")
 _libimpl.impl("fp8_gemm", _fp8_gemm_dev, "CUDA")
 _libimpl.impl("act_quant", _act_quant_meta, "Meta")
 _libimpl.impl("weight_dequant", _weight_dequant_meta, "Meta")
+_libimpl.impl("weight_quant", _weight_quant_meta, "Meta")
 _libimpl.impl("fp8_gemm", _fp8_gemm_meta, "Meta")

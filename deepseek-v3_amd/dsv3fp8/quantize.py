@@ -1,9 +1,13 @@
-"""Offline weight block-quantiser: bf16/fp32 weight -> (fp8 e4m3fn, fp32 scales).
+"""Weight block-quantiser: bf16/fp16/fp32 weight -> (fp8 e4m3fn, fp32 scales).
 
 Produces the on-disk format that ``weight_dequant`` / ``fp8_gemm`` consume
 (reference: README_WEIGHTS.md:60-92, the ``weight`` + ``weight_scale_inv`` pair;
-scale tensor shape as in inference/model.py:184-187).  Plain torch ops on the
-tensor's own device; this is set-up code, not part of the per-token hot path.
+scale tensor shape as in inference/model.py:184-187).
+
+``weight_quant`` is the device path (the gfx950 kernel behind ``torch.ops.dsv3fp8.weight_quant``);
+``block_quant_weight`` states the same rule in plain torch ops on the tensor's own device and is what
+the synthetic-input generators use (on the host the two agree bit for bit; torch's device division is not
+correctly rounded, so on a GPU its scales can differ from the kernel's in the last place).
 """
 from __future__ import annotations
 
@@ -30,3 +34,12 @@ def block_quant_weight(w: torch.Tensor, block_size: int = 128) -> Tuple[torch.Te
     scale = amax / 448.0
     w8 = (tiles / scale[:, None, :, None]).reshape(mb * block_size, nb * block_size)[:m, :n]
     return w8.contiguous().to(FP8), scale
+
+
+def weight_quant(w: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``block_quant_weight`` on the device: one pass over ``w`` (2-D, contiguous, on the GPU) by the HIP kernel.
+    Returns ``(w8 [m,n] e4m3fn, scale [ceil(m/128), ceil(n/128)] fp32)``."""
+    from . import ops  # noqa: F401  (registers torch.ops.dsv3fp8)
+    assert w.is_contiguous(), 'Input tensor must be contiguous'
+    assert w.dim() == 2, 'Input tensor must have 2 dimensions'
+    return torch.ops.dsv3fp8.weight_quant(w, block_size)

@@ -101,6 +101,19 @@ int dsv3_weight_dequant(const void* x, const float* s, void* y, int y_dtype,
                         int64_t m, int64_t n, int block_size, void* stream);
 
 /*
+ * Weight block-quantiser, the inverse of weight_dequant and the producer of the checkpoint format the reference
+ * loads (README_WEIGHTS.md:60-92: `weight` e4m3 + `weight_scale_inv` binary32 per 128 x 128 block, a block that
+ * is not aligned to 128 is zero-padded before its scale is calculated and the padding removed afterwards; scale
+ * tensor shape inference/model.py:184-187).  The reference ships only the dequantising direction; the rule here is
+ * the one its activation quantiser uses on 1 x 128 blocks (inference/kernel.py:23-35), applied to the square block:
+ *     s[i,j] = max(amax(|w| over block i,j), 1e-4) / 448;   y = e4m3( w / s[i / 128, j / 128] )   (RNE)
+ * w: [m,n] of w_dtype, y: [m,n] fp8 bytes, s: [ceil(m/128), ceil(n/128)] binary32.  block_size must be 128.
+ * Any m, n >= 0; n % 8 == 0 with 16-byte aligned w and 8-byte aligned y takes the vectorised kernel.
+ */
+int dsv3_weight_quant(const void* w, int w_dtype, void* y, float* s,
+                      int64_t m, int64_t n, int block_size, void* stream);
+
+/*
  * fp8_gemm (inference/kernel.py:145-172):
  *     c[i,j] = c_dtype( sum_kb ( sum_{t<128} a[i,128kb+t] * b[j,128kb+t] )
  *                                * a_s[i,kb] * b_s[j/128,kb] )

@@ -60,3 +60,71 @@ def test_convert_synthetic_checkpoint(tmp_path):
     assert index["metadata"] == {}
     assert set(index["weight_map"]) == {"l0.a.weight", "l0.norm.weight", "l0.b.weight", "l1.c.weight", "l1.orphan.weight"}
     assert index["weight_map"]["l1.c.weight"] == "model-00002-of-00002.safetensors"
+
+
+def test_bf16_to_fp8_and_back(tmp_path):
+    """The quantising direction on a synthetic HF-named bf16 checkpoint: FP8 layers become `weight` +
+    `weight_scale_inv` pairs equal to the oracle's quantisation, everything else passes through, and
+    fp8_cast_bf16 on the result gives back the oracle's dequantisation of those pairs."""
+    from dsv3fp8 import bf16_cast_fp8, fp8_cast_bf16
+    g = torch.Generator().manual_seed(1)
+    src, mid, dst = tmp_path / "bf16", tmp_path / "fp8", tmp_path / "back"
+    src.mkdir()
+
+    def w(rows, cols):
+        return (torch.randn(rows, cols, generator=g) * 0.05).bfloat16()
+    L = "model.layers.3."
+    tensors = {
+        "model.embed_tokens.weight": w(300, 256),
+        L + "self_attn.q_a_proj.weight": w(192, 256),
+        L + "self_attn.kv_a_proj_with_mqa.weight": w(72, 256),          # 72 rows: one ragged block row
+        L + "self_attn.q_a_layernorm.weight": torch.randn(192, generator=g).bfloat16(),
+        L + "self_attn.o_proj.weight": w(256, 384),
+        L + "mlp.gate.weight": w(8, 256),                               # the router: a parameter, not a Linear
+        L + "mlp.gate.e_score_correction_bias": torch.randn(8, generator=g),
+        L + "mlp.experts.5.gate_proj.weight": w(130, 256),
+        L + "mlp.experts.5.down_proj.weight": w(256, 130),
+        L + "mlp.shared_experts.up_proj.weight": w(128, 256),
+        "lm_head.weight": w(300, 256),
+    }
+    names = sorted(tensors)
+    shards = {"model-00001-of-00002.safetensors": {k: tensors[k] for k in names[:6]},
+              "model-00002-of-00002.safetensors": {k: tensors[k] for k in names[6:]}}
+    weight_map = {}
+    for fname, ts in shards.items():
+        save_file(ts, str(src / fname))
+        weight_map.update({k: fname for k in ts})
+    (src / "model.safetensors.index.json").write_text(json.dumps({"metadata": {"total_size": 1}, "weight_map": weight_map}))
+
+    bf16_cast_fp8.main(str(src), str(mid))
+    fp8_names = {k for k in tensors if k.split(".")[-2].endswith("_proj") or k.split(".")[-2] == "kv_a_proj_with_mqa"}
+    assert len(fp8_names) == 6
+    index = json.loads((mid / "model.safetensors.index.json").read_text())
+    assert set(index["weight_map"]) == set(tensors) | {k + "_scale_inv" for k in fp8_names}
+    out = {}
+    for fname in shards:
+        got = load_file(str(mid / fname))
+        assert all(index["weight_map"][k] == fname for k in got)
+        out.update(got)
+    for k, t in tensors.items():
+        if k in fp8_names:
+            ref8, refs = oracle.block_quant_weight(t)
+            assert out[k].dtype == FP8 and torch.equal(out[k].view(torch.uint8), ref8.view(torch.uint8)), k
+            assert out[k + "_scale_inv"].dtype == torch.float32 and torch.equal(out[k + "_scale_inv"], refs), k
+        else:
+            assert out[k].dtype == t.dtype and torch.equal(out[k], t), k
+
+    old = torch.get_default_dtype()
+    try:
+        fp8_cast_bf16.main(str(mid), str(dst))
+    finally:
+        torch.set_default_dtype(old)
+    back = {}
+    for fname in shards:
+        back.update(load_file(str(dst / fname)))
+    assert set(back) == set(tensors)
+    for k in fp8_names:
+        want = oracle.weight_dequant(out[k], out[k + "_scale_inv"])
+        assert torch.equal(back[k].view(torch.int16), want.view(torch.int16)), k
+        rel = (back[k].float() - tensors[k].float()).abs().max() / tensors[k].float().abs().max()
+        assert rel < 0.07, (k, rel)                                     # half an e4m3 step of the block maximum

@@ -1,0 +1,116 @@
+"""GPU parity: the weight block-quantiser through the C ABI vs the torch-CPU oracle, bit for bit (bytes and scales).
+Format: README_WEIGHTS.md:60-92 (128 x 128 blocks, ragged blocks zero-padded before the scale is taken); the rule is
+the activation quantiser's (inference/kernel.py:23-35) on a square block."""
+import pytest
+import torch
+
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+FP8 = torch.float8_e4m3fn
+
+
+@pytest.fixture(scope="module")
+def K():
+    import dsv3fp8
+    return dsv3fp8
+
+
+def _check(K, w):
+    ref8, refs = oracle.block_quant_weight(w)
+    q8, qs = K.weight_quant(w.cuda())
+    assert q8.dtype == FP8 and qs.dtype == torch.float32
+    assert q8.shape == ref8.shape and qs.shape == refs.shape
+    assert torch.equal(qs.cpu(), refs)
+    assert torch.equal(q8.cpu().view(torch.uint8), ref8.view(torch.uint8))
+    return q8, qs
+
+
+@pytest.mark.parametrize("shape", [(256, 512), (1536, 7168), (576, 7168), (130, 272), (1, 8), (128, 7168 + 16),
+                                   (300, 520), (127, 129 * 8)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_random_vector_path(K, shape, dtype):
+    g = torch.Generator().manual_seed(shape[0] + shape[1])
+    w = (torch.randn(*shape, generator=g) * 0.02).to(dtype)
+    _check(K, w)
+
+
+@pytest.mark.parametrize("shape", [(200, 301), (5, 7), (129, 1), (64, 1027)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_row_lengths_that_are_not_multiples_of_8(K, shape, dtype):
+    g = torch.Generator().manual_seed(shape[1])
+    w = (torch.randn(*shape, generator=g) * 0.5).to(dtype)
+    _check(K, w)
+
+
+def test_magnitudes_signed_zeros_and_the_clamp(K):
+    g = torch.Generator().manual_seed(5)
+    # blocks whose amax spans 60 decades of binary32-representable bf16 magnitudes, one all-zero block, signed zeros
+    w = torch.randn(256, 1024, generator=g)
+    expo = torch.linspace(-30, 30, 8).repeat_interleave(128)[None, :]
+    w = (w * torch.pow(10.0, expo)).bfloat16()
+    w[:128, 128:256] = 0
+    w[5, 130] = -0.0
+    w[128:, 0] = -0.0
+    w[200, 700] = 3.0e38
+    w[130, 900] = -3.3e38
+    q8, qs = _check(K, w)
+    assert qs[0, 1].item() == pytest.approx(1e-4 / 448, rel=1e-7)
+    assert q8.cpu().view(torch.uint8)[5, 130] == 0x80                      # -0 stays -0
+
+
+def test_every_bf16_value_as_an_element(K):
+    """All finite bf16 bit patterns: block b holds one sign and 16 consecutive exponents (all 128 mantissas each), a
+    range the e4m3 codes of one scale can resolve, so every quotient the correction sequence for bf16 inputs can
+    meet at that block's scale occurs."""
+    blocks = []
+    for sign in (0, 0x8000):
+        for e0 in range(0, 255, 16):
+            exps = torch.arange(e0, min(e0 + 16, 255))
+            pats = (sign | (exps[:, None] << 7) | torch.arange(128)[None, :]).flatten()
+            blocks.append(pats.repeat(-(-16384 // pats.numel()))[:16384].view(128, 128))
+    bits = torch.cat(blocks, 1)
+    w = ((bits + 0x8000) % 0x10000 - 0x8000).to(torch.int16).view(torch.bfloat16).contiguous()
+    assert w.shape == (128, 32 * 128) and bool(w.float().isfinite().all())
+    _check(K, w)
+    _check(K, w.t().contiguous())
+
+
+def test_known_answers_on_device(K):
+    g = torch.Generator().manual_seed(11)
+    m, n = 300, 520
+    b = torch.randint(0, 256, (m, n), generator=g, dtype=torch.int16)
+    b = torch.where((b & 0x7F) == 0x7F, b & 0x80, b).to(torch.uint8)
+    for i in range(3):
+        for j in range(5):
+            b[min(i * 128 + 7 * j + 3, m - 1), min(j * 128 + 5 * i + 2, n - 1)] = 0x7E if (i + j) % 2 else 0xFE
+    s = torch.pow(2.0, torch.randint(-12, 3, (3, 5), generator=g).float())
+    w = oracle.weight_dequant(b.view(FP8), s, out_dtype=torch.float32)
+    for src in (w, w.bfloat16()):
+        q8, qs = K.weight_quant(src.cuda())
+        assert torch.equal(qs.cpu(), s)
+        assert torch.equal(q8.cpu().float(), b.view(FP8).float())
+
+
+def test_full_size_round_trip(K):
+    """[18432, 7168] on the device: every block reaches the largest code, weight_dequant brings the weights back to
+    within half an e4m3 step, and sampled row bands equal the oracle's bytes and scales."""
+    g = torch.Generator(device="cuda").manual_seed(1)
+    w = (torch.randn(18432, 7168, generator=g, device="cuda") * 0.02).bfloat16()
+    q8, qs = K.weight_quant(w)
+    assert q8.shape == (18432, 7168) and qs.shape == (144, 56)
+    assert bool((q8.float().abs().view(144, 128, 56, 128).amax(dim=(1, 3)) == 448).all())
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float32)
+    try:
+        back = K.weight_dequant(q8, qs)
+    finally:
+        torch.set_default_dtype(old)
+    es = qs.repeat_interleave(128, 0).repeat_interleave(128, 1)
+    err = (back - w.float()).abs()
+    assert bool((err <= torch.maximum(w.float().abs() * 2.0 ** -4, es * 2.0 ** -10) * (1 + 1e-6)).all())
+    for r0 in (0, 9088, 18304):                                 # three 128-row bands against the CPU oracle
+        ref8, refs = oracle.block_quant_weight(w[r0:r0 + 128].cpu())
+        assert torch.equal(qs[r0 // 128].cpu(), refs[0])
+        assert torch.equal(q8[r0:r0 + 128].cpu().view(torch.uint8), ref8.view(torch.uint8))

@@ -162,6 +162,39 @@ def test_block_quant_round_trip_and_padding():
     assert torch.equal(w8p.view(torch.uint8), w8.view(torch.uint8)) and torch.equal(sp, s)
 
 
+def test_block_quant_known_answers():
+    """What pins the quantiser without restating it: weights that ARE e4m3 values times a power-of-two scale, with
+    a +-448 in every block, have exactly one quantisation -- those bytes and that scale -- and the reference's
+    dequantisation rule (README_WEIGHTS.md:88-90, oracle.weight_dequant) must give the weights back."""
+    g = torch.Generator().manual_seed(11)
+    m, n = 300, 520                                            # ragged both ways: 3 x 5 blocks
+    b = torch.randint(0, 256, (m, n), generator=g, dtype=torch.int16)
+    b = torch.where((b & 0x7F) == 0x7F, b & 0x80, b).to(torch.uint8)         # no NaN bytes
+    mb, nb = 3, 5
+    for i in range(mb):                                        # a 448 (0x7e) or -448 (0xfe) inside every block's real part
+        for j in range(nb):
+            b[min(i * 128 + 7 * j + 3, m - 1), min(j * 128 + 5 * i + 2, n - 1)] = 0x7E if (i + j) % 2 else 0xFE
+    w8 = b.view(FP8)
+    s = torch.pow(2.0, torch.randint(-12, 3, (mb, nb), generator=g).float())
+    w = oracle.weight_dequant(w8, s, out_dtype=torch.float32)                # exact: 4 significant bits times 2^e
+    assert torch.equal(w.bfloat16().float(), w)                              # ... and exactly representable in bf16
+    for src in (w, w.bfloat16()):
+        q8, qs = oracle.block_quant_weight(src)
+        assert torch.equal(qs, s)
+        assert torch.equal(q8.float(), w8.float())                           # (+0 and -0 bytes compare equal here)
+    # an all-zero block takes the clamp: scale 1e-4 / 448, bytes zero
+    q8, qs = oracle.block_quant_weight(torch.zeros(128, 256))
+    assert qs[0, 0].item() == pytest.approx(1e-4 / 448, rel=1e-7) and int(q8.view(torch.uint8).max()) == 0
+    # every block of a generic weight reaches the largest code, and the quantisation error is within half an e4m3
+    # step (2^-4 relative for normal codes, 2^-10 * scale absolute for the subnormal ones)
+    wg = (torch.randn(256, 384, generator=g) * 0.03).bfloat16()
+    q8, qs = oracle.block_quant_weight(wg)
+    assert bool((q8.float().abs().view(2, 128, 3, 128).amax(dim=(1, 3)) == 448).all())
+    err = (oracle.weight_dequant(q8, qs, out_dtype=torch.float32) - wg.float()).abs()
+    es = oracle.expand_block_scale(qs, 256, 384)
+    assert bool((err <= torch.maximum(wg.float().abs() * 2.0 ** -4, es * 2.0 ** -10) * (1 + 1e-6)).all())
+
+
 # ---------------------------------------------------------------- fp8_gemm
 
 def _rand_problem(m, n, k, seed):
