@@ -248,6 +248,17 @@ def run_moe(K, W, tokens: int = 4096, bias_std: float = 0.1, expert_loop: bool =
                             "weight_stream_GBps": round(wbytes / ms / 1e6, 1),
                             "mfma_frac": round(flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 4),
                             "hbm_frac": round(wbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            if expert_loop:                  # decode sizes on the same layer, one captured forward each
+                Mdl.MoE.grouped = True
+                dec = {}
+                for t in (1, 8, 32):
+                    xd = W.activations(t, args.dim, 60 + t, "cuda")
+                    hit_d = int(moe.gate(xd)[1].unique().numel())
+                    us = time_graph([lambda: moe(xd)], replays=20)
+                    wb = (hit_d + 1) * 3 * args.dim * args.moe_inter_dim
+                    dec[f"T{t}"] = {"us": round(us, 1), "experts_with_tokens": hit_d,
+                                    "weight_stream_GBps": round(wb / us / 1e3, 1)}
+                res["decode_graph"] = dec
         res["note"] = ("grouped: MoE.forward as shipped (no host sync); expert_loop: the reference's per-expert "
                        "loop, 3 act_quant + 3 fp8_gemm per expert")
         return res

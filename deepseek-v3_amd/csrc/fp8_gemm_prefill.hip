@@ -732,6 +732,13 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
                    int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
                    const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream) {
     using namespace prefill;
+    // few rows in all (an MoE layer at up to ~35 tokens): the weight-streaming kernel fills the chip where
+    // groups x 16 tiles would not, and a group of a few rows costs it no 128-row tile (measured on the 256-expert
+    // layer: 116 against 157 us at one token, 695 against 766 us at 32, equal at 48-64, slower beyond)
+    static const int skinny_max = getenv("DSV3_GROUPED_SKINNY_MAX") ? atoi(getenv("DSV3_GROUPED_SKINNY_MAX")) : 320;
+    if (m <= skinny_max)
+        return launch_grouped_skinny(a, a_s, a_rows, b, b_s, c, CD, n, k, num_tiles, tile_group, tile_row0, tile_rows,
+                                     b_stride, bs_stride, stream);
     GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
     constexpr int LDS_BYTES = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
     const int64_t tn = (n + BN - 1) / BN;

@@ -57,6 +57,11 @@ def _grouped_case(counts, n, k, seed, gather):
     ([129, 64], 576, 256, False),            # ragged n: 576 = 2 tiles + 64, 5 scale rows
     ([40] * 6, 256, 1152, True),             # odd number of K blocks
     ([145, 177, 200, 241, 17], 512, 384, True),   # 256-row slots with 10, 12, 13 and 16 live sub-tiles, then a small one
+    ([1] * 9, 4096, 7168, True),             # one token of the MoE layer: the weight-streaming kernel (up to 320 rows in all)
+    ([2, 0, 1, 5, 0, 3], 7168, 2048, False), # ... its second GEMM shape, ragged group sizes, no gather
+    ([20, 3, 13], 200, 640, True),           # ... a slot of more than 16 rows (two passes), n not a multiple of 32
+    ([36], 48, 128, False),                  # ... one K block, three passes
+    ([40] * 8, 96, 256, True),               # ... 320 rows: the largest launch that takes this kernel
 ])
 def test_fp8_gemm_grouped_vs_oracle(K, counts, n, k, gather):
     from dsv3fp8 import ops
@@ -137,7 +142,8 @@ def test_moe_combine_bit_exact(K, with_shared):
     assert torch.equal(got.cpu().view(torch.int16), ref.view(torch.int16))
 
 
-def test_moe_grouped_matches_expert_loop_and_oracle(K):
+@pytest.mark.parametrize("tokens", [300, 1, 3])           # 1 and 3 tokens: the weight-streaming grouped kernel
+def test_moe_grouped_matches_expert_loop_and_oracle(K, tokens):
     from dsv3fp8 import model as M
     old = (M.gemm_impl, torch.get_default_dtype(), M.Linear.dtype)
     torch.set_default_dtype(torch.bfloat16)
@@ -164,7 +170,7 @@ def test_moe_grouped_matches_expert_loop_and_oracle(K):
             experts.append((w1, s1, w2, s2, w3, s3))
         sh = moe.shared_experts
         shared = (*fill(sh.w1, 90), *fill(sh.w2, 91), *fill(sh.w3, 92))
-        x = torch.randn(300, 256, generator=g).bfloat16()
+        x = torch.randn(tokens, 256, generator=g).bfloat16()
         with torch.inference_mode():
             M.MoE.grouped = True
             y_grouped = moe(x.cuda())                   # 300 tokens: the shared expert rides along as group 8
