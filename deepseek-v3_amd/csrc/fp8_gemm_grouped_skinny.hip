@@ -23,9 +23,7 @@
 namespace dsv3 {
 namespace gskinny {
 
-constexpr int kWaves = 4;
 constexpr int S = 2;            // 16-row weight strips per wavefront
-constexpr int NPF = 4;          // K blocks of loads in flight per wavefront
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
     v8i r = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
@@ -44,11 +42,15 @@ __device__ __forceinline__ v8i untangle(v4i a, v4i b) {
     return r;
 }
 
+template <int kWaves>
 __global__ __launch_bounds__(kWaves * kWave) void fp8_gemm_grouped_skinny_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s, const int* __restrict__ a_rows,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s, void* __restrict__ c, int c_dtype,
         int N, int K, const int* __restrict__ tile_group, const int* __restrict__ tile_row0,
         const int* __restrict__ tile_rows, int64_t b_stride, int64_t bs_stride) {
+    // K blocks of loads in flight per wavefront: fewer with more wavefronts per workgroup, so that 16 wavefronts per
+    // compute unit stay resident (128 registers each)
+    constexpr int NPF = kWaves == 4 ? 4 : (kWaves == 8 ? 3 : 2);
     __shared__ v4f red[kWaves * S * 64];
     const int slot = blockIdx.y;
     const int grp = tile_group[slot];
@@ -63,16 +65,17 @@ __global__ __launch_bounds__(kWaves * kWave) void fp8_gemm_grouped_skinny_kernel
     const int nkb = max(0, min(per_wave, KB - kb0));
     const int n0 = blockIdx.x * (16 * S);
     b += (size_t)grp * b_stride;
-    b_s += (size_t)grp * bs_stride + (size_t)min(n0 >> 7, (N - 1) >> 7) * KB;
+    b_s += (size_t)grp * bs_stride + (size_t)min(n0 >> 7, (N - 1) >> 7) * KB + kb0;
 
-    // weight loads: lanes with fr < 8 take the first 64 bytes of row fr & 7 of the strip, the others the last 64
-    const uint8_t* wsrc[S];
-    size_t wrow8[S];
+    // weight loads: lanes with fr < 8 take the first 64 bytes of row fr & 7 of the strip, the others the last 64.
+    // Offsets are 32-bit (the caller checks that a group's weights and the activations stay below 4 GiB) on top of
+    // wavefront-uniform bases.
+    uint32_t woff[S], wrow8[S];
 #pragma unroll
     for (int s = 0; s < S; ++s) {
         const int r_lo = min(n0 + s * 16 + (fr & 7), N - 1), r_hi = min(n0 + s * 16 + (fr & 7) + 8, N - 1);
-        wsrc[s] = b + (size_t)r_lo * K + (size_t)kb0 * 128 + (fr >> 3) * 64 + fq * 16;
-        wrow8[s] = (size_t)(r_hi - r_lo) * K;
+        woff[s] = (uint32_t)r_lo * (uint32_t)K + (uint32_t)kb0 * 128u + (fr >> 3) * 64 + fq * 16;
+        wrow8[s] = (uint32_t)(r_hi - r_lo) * (uint32_t)K;
     }
 
     for (int pass = 0; pass < rows; pass += 16) {
@@ -80,22 +83,22 @@ __global__ __launch_bounds__(kWaves * kWave) void fp8_gemm_grouped_skinny_kernel
         // activation fragment of lane (fr, fq): row fr of this pass (rows past its end repeat the last one; their
         // results are dropped), bytes {16 fq .. +15} and {64 + 16 fq .. +15} of the K block
         const int crow = row0 + pass + min(fr, m_here - 1);
-        const int64_t arow = a_rows ? a_rows[crow] : crow;
-        const uint8_t* asrc = a + arow * K + (int64_t)kb0 * 128 + fq * 16;
-        const float* assrc = a_s + arow * KB + kb0;
+        const uint32_t arow = (uint32_t)(a_rows ? a_rows[crow] : crow);
+        const uint32_t aoff = arow * (uint32_t)K + (uint32_t)kb0 * 128u + fq * 16;
+        const uint32_t asoff = arow * (uint32_t)KB + (uint32_t)kb0;
 
         v4i wlo[NPF][S], whi[NPF][S], alo[NPF], ahi[NPF];
         float sa[NPF], sb[NPF];
         auto fetch = [&](int p, int k) {
 #pragma unroll
             for (int s = 0; s < S; ++s) {
-                wlo[p][s] = __builtin_nontemporal_load((const v4i*)(wsrc[s] + k * 128));
-                whi[p][s] = __builtin_nontemporal_load((const v4i*)(wsrc[s] + wrow8[s] + k * 128));
+                wlo[p][s] = __builtin_nontemporal_load((const v4i*)(b + woff[s] + (uint32_t)k * 128u));
+                whi[p][s] = __builtin_nontemporal_load((const v4i*)(b + woff[s] + wrow8[s] + (uint32_t)k * 128u));
             }
-            alo[p] = *(const v4i*)(asrc + k * 128);
-            ahi[p] = *(const v4i*)(asrc + k * 128 + 64);
-            sa[p] = assrc[k];
-            sb[p] = b_s[kb0 + k];
+            alo[p] = *(const v4i*)(a + aoff + (uint32_t)k * 128u);
+            ahi[p] = *(const v4i*)(a + aoff + (uint32_t)k * 128u + 64u);
+            sa[p] = a_s[asoff + (uint32_t)k];
+            sb[p] = b_s[k];
         };
         v4f acc[S];
 #pragma unroll
@@ -158,14 +161,26 @@ __global__ __launch_bounds__(kWaves * kWave) void fp8_gemm_grouped_skinny_kernel
 int launch_grouped_skinny(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s, void* c,
                           int c_dtype, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group,
                           const int* tile_row0, const int* tile_rows, int64_t b_stride, int64_t bs_stride,
-                          hipStream_t stream) {
+                          int64_t groups_hint, hipStream_t stream) {
     using namespace gskinny;
     const int64_t strips = (n + 16 * S - 1) / (16 * S);
     if (strips > 0x7fffffff || num_tiles > 65535) return DSV3_ERR_BAD_SHAPE;
     if (strips == 0 || num_tiles == 0) return DSV3_OK;
-    hipLaunchKernelGGL(fp8_gemm_grouped_skinny_kernel, dim3((unsigned)strips, (unsigned)num_tiles), dim3(kWaves * kWave),
-                       0, stream, (const uint8_t*)a, a_s, a_rows, (const uint8_t*)b, b_s, c, c_dtype, (int)n, (int)k,
-                       tile_group, tile_row0, tile_rows, b_stride, bs_stride);
+    // wavefronts per workgroup (they split K): at least two K blocks each, and more of them when the strips alone
+    // would leave the chip short of wavefronts.  `groups_hint` is the caller's estimate of the live tile slots.
+    const int64_t kb = k / 128;
+    int waves = 4;
+    static const int forced = getenv("DSV3_GS_WAVES") ? atoi(getenv("DSV3_GS_WAVES")) : 0;
+    while (waves < 16 && strips * groups_hint * waves < 3072 && kb / (waves * 2) >= 2) waves *= 2;
+    if (forced) waves = forced;
+#define DSV3_GS(W)                                                                                                     \
+    hipLaunchKernelGGL(fp8_gemm_grouped_skinny_kernel<W>, dim3((unsigned)strips, (unsigned)num_tiles), dim3(W * kWave), \
+                       0, stream, (const uint8_t*)a, a_s, a_rows, (const uint8_t*)b, b_s, c, c_dtype, (int)n, (int)k,  \
+                       tile_group, tile_row0, tile_rows, b_stride, bs_stride)
+    if (waves >= 16) DSV3_GS(16);
+    else if (waves >= 8) DSV3_GS(8);
+    else DSV3_GS(4);
+#undef DSV3_GS
     return launch_status();
 }
 

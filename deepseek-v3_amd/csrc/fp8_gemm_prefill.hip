@@ -738,7 +738,7 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
     static const int skinny_max = getenv("DSV3_GROUPED_SKINNY_MAX") ? atoi(getenv("DSV3_GROUPED_SKINNY_MAX")) : 320;
     if (m <= skinny_max)
         return launch_grouped_skinny(a, a_s, a_rows, b, b_s, c, CD, n, k, num_tiles, tile_group, tile_row0, tile_rows,
-                                     b_stride, bs_stride, stream);
+                                     b_stride, bs_stride, m < num_tiles ? m : num_tiles, stream);
     GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
     constexpr int LDS_BYTES = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
     const int64_t tn = (n + BN - 1) / BN;
