@@ -35,15 +35,17 @@ constexpr int SC_STAGE = 8 * 256;                        // scales of one K bloc
 // tiles.  <128, 3>: 32 x 128 per wavefront, 3 x 48 KiB -- the loads of a K block then have two blocks of time to
 // land, which is what matters when a tile has little arithmetic per block (the ~128-row groups of an MoE layer:
 // a global -> LDS round trip under load, ~1.4 us, is longer than such a block's MFMA time).
-template <int TM, int S> struct Cfg {
+template <int TM, int S, int SB = S> struct Cfg {                    // S: activation (A) stages, SB: weight (B) stages
     static constexpr int WM = TM / WAVES_M, SM = WM / 16;
     static constexpr int A_LOADS = TM / 64, B_LOADS = BN / 64;        // 1 KiB wavefront-loads per wavefront and stage
     static constexpr int LOADS = A_LOADS + B_LOADS + 1;               // ... plus the scale load
     static constexpr int A_STAGE = TM * 128, B_STAGE = BN * 128;      // bytes per K block
-    static constexpr int LDS_A = 0, LDS_B = S * A_STAGE;              // [A stages | B stages | scale stages]
-    static constexpr int LDS_SC = S * (A_STAGE + B_STAGE);
-    static constexpr int LDS_BYTES = LDS_SC + S * SC_STAGE;
+    static constexpr int SS = SB > S ? SB : S;                        // scale slots
+    static constexpr int LDS_A = 0, LDS_B = S * A_STAGE;              // [A stages | B stages | scale slots]
+    static constexpr int LDS_SC = S * A_STAGE + SB * B_STAGE;
+    static constexpr int LDS_BYTES = LDS_SC + SS * SC_STAGE;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS of a gfx950 compute unit");
+    static_assert(SB >= S, "the weights are the operand that comes from HBM");
 };
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -80,14 +82,15 @@ struct GroupTable {
 };
 
 // One workgroup's tile (grouped mode: tile slot) from start to end; the kernels below are thin wrappers.
-template <int CD, bool G, int TM, int S>
+template <int CD, bool G, int TM, int S, int SB = S>
 __device__ __forceinline__ void prefill_tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
         int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g,
         int wg) {                           // index of the workgroup among those that run this configuration
-    using C = Cfg<TM, S>;
+    using C = Cfg<TM, S, SB>;
+    constexpr int SS = C::SS;
     constexpr int WM = C::WM, SM = C::SM, A_LOADS = C::A_LOADS, B_LOADS = C::B_LOADS;
     constexpr int A_STAGE = C::A_STAGE, B_STAGE = C::B_STAGE, LDS_A = C::LDS_A, LDS_B = C::LDS_B, LDS_SC = C::LDS_SC;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -221,9 +224,18 @@ __device__ __forceinline__ void prefill_tile(
     // stalls instruction issue.  At barrier kb the data of block kb+1 must be there; everything issued later
     // belongs to blocks kb+2 .. kb+S-1, so the wait is vmcnt((S-2) * loads per block).
     constexpr int kSync = SN - 2;
-    constexpr int kWaitSync = 0x0f70 | ((S - 2) * C::LOADS);
-    static_assert((S - 2) * C::LOADS < 16, "vmcnt immediate");
-    auto next_stage = [](int st) { return st + 1 == S ? 0 : st + 1; };
+    // (with more weight stages than activation stages the weight part of a block is requested SB - S blocks
+    // earlier: at barrier kb the loads that may still be in flight are the weight parts of blocks kb+2 .. kb+SB-1
+    // and the activation parts and scales of blocks kb+2 .. kb+S-1, all of them younger than anything of block kb+1)
+    constexpr int kInFlight = (SB - 2) * B_LOADS + (S - 2) * (A_LOADS + 1);
+    constexpr int kWaitSync = 0x0f70 | kInFlight;
+    static_assert(kInFlight < 16, "vmcnt immediate");
+    auto next_a = [](int st) { return st + 1 == S ? 0 : st + 1; };
+    auto next_b = [](int st) { return st + 1 == SB ? 0 : st + 1; };
+    auto next_s = [](int st) { return st + 1 == SS ? 0 : st + 1; };
+    auto prev_b = [](int st) { return st == 0 ? SB - 1 : st - 1; };
+    // scale slot of block kb + S seen from the slot of block kb
+    auto ahead_s = [](int st) { return (st + S) % SS; };
     // sub-tiles of this wavefront that hold at least one valid row (all of them in dense mode; the clamped rows of
     // an edge tile are computed and dropped there).  The pipeline below is instantiated per count, so a wavefront
     // issues MFMAs and FMAs only for live sub-tiles; one without any only feeds LDS and keeps the barriers.
@@ -240,23 +252,28 @@ __device__ __forceinline__ void prefill_tile(
         __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
         wg_barrier();
 #pragma unroll
-        for (int blk = 1; blk < S; ++blk) {
+        for (int blk = 1; blk < SS; ++blk) {
+            if (blk < S) {
 #pragma unroll
-            for (int t = 0; t < (blk < S - 1 ? A_LOADS + B_LOADS : A_LOADS); ++t) issue_load(t, min(blk, KB - 1), blk);
-            issue_scales(min(blk, KB - 1), blk);
+                for (int t = 0; t < A_LOADS; ++t) issue_load(t, min(blk, KB - 1), blk);
+                issue_scales(min(blk, KB - 1), blk);
+            }
+            if (blk < SB - 1) {
+#pragma unroll
+                for (int t = A_LOADS; t < A_LOADS + B_LOADS; ++t) issue_load(t, min(blk, KB - 1), blk);
+            }
         }
         if constexpr (JA == 0) {
-            int st = 0;
+            int st_a = 0, st_b = 0, st_s = 0;
             for (int kb = 0; kb < KB; ++kb) {
-                const int st_prev = st == 0 ? S - 1 : st - 1;
 #pragma unroll
-                for (int t = A_LOADS; t < A_LOADS + B_LOADS; ++t) issue_load(t, min(kb - 1 + S, KB - 1), st_prev);
+                for (int t = A_LOADS; t < A_LOADS + B_LOADS; ++t) issue_load(t, min(kb - 1 + SB, KB - 1), prev_b(st_b));
                 __builtin_amdgcn_s_waitcnt(kWaitSync);
                 wg_barrier();
 #pragma unroll
-                for (int t = 0; t < A_LOADS; ++t) issue_load(t, min(kb + S, KB - 1), st);
-                issue_scales(min(kb + S, KB - 1), st);
-                st = next_stage(st);
+                for (int t = 0; t < A_LOADS; ++t) issue_load(t, min(kb + S, KB - 1), st_a);
+                issue_scales(min(kb + S, KB - 1), ahead_s(st_s));
+                st_a = next_a(st_a); st_b = next_b(st_b); st_s = next_s(st_s);
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);
         } else {
@@ -280,15 +297,15 @@ __device__ __forceinline__ void prefill_tile(
             nf1 = join(*(const v4i*)(bs_base + 2048 + c0), *(const v4i*)(bs_base + 2048 + c1));
         }
 
-        int stage = 0;                        // LDS stage of block kb
+        int st_a = 0, st_b = 0, st_s = 0;     // LDS stages of block kb: activations, weights, scales
         for (int kb = 0; kb < KB; ++kb) {
-            const int st_next = next_stage(stage), st_prev = stage == 0 ? S - 1 : stage - 1;
-            const uint8_t* bs_base = lds + b_rd + stage * B_STAGE;
-            const uint8_t* as_next = lds + a_rd + st_next * A_STAGE;
-            const uint8_t* bs_next = lds + b_rd + st_next * B_STAGE;
+            const int sa_next = next_a(st_a), sb_next = next_b(st_b), ss_next = next_s(st_s);
+            const uint8_t* bs_base = lds + b_rd + st_b * B_STAGE;
+            const uint8_t* as_next = lds + a_rd + sa_next * A_STAGE;
+            const uint8_t* bs_next = lds + b_rd + sb_next * B_STAGE;
 
             // branch-free: past the end the loop re-fetches the last block into stages nobody reads again
-            const int kb_w = min(kb - 1 + S, KB - 1), kb_a = min(kb + S, KB - 1);
+            const int kb_w = min(kb - 1 + SB, KB - 1), kb_a = min(kb + S, KB - 1);
 
             // fold the tile left over from the previous K block with that block's scale, then switch scales
 #pragma unroll
@@ -305,11 +322,11 @@ __device__ __forceinline__ void prefill_tile(
                     __builtin_amdgcn_s_waitcnt(kWaitSync);
                     wg_barrier();
                     {
-                        const float bs = lds_bs(st_next);
+                        const float bs = lds_bs(ss_next);
 #pragma unroll
-                        for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, st_next) * bs;
+                        for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, ss_next) * bs;
                     }
-                    issue_scales(kb_a, stage);
+                    issue_scales(kb_a, ahead_s(st_s));
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // weight rows are streamed two steps ahead; the last two steps fetch steps 0 and 1 of the next block
@@ -335,13 +352,14 @@ __device__ __forceinline__ void prefill_tile(
                 }
                 // refill, see above: activation part of block kb+S after the barrier, weight part of block kb-1+S
                 // at the start of the block
-                if (i >= kSync) {
+                if (i >= kSync) {                           // first half (rounded up) at step kSync, the rest at kSync + 1
+                    constexpr int kHalf = (A_LOADS + 1) / 2;
 #pragma unroll
-                    for (int t = 0; t < A_LOADS / 2; ++t) issue_load((i - kSync) * (A_LOADS / 2) + t, kb_a, stage);
+                    for (int t = (i == kSync ? 0 : kHalf); t < (i == kSync ? kHalf : A_LOADS); ++t) issue_load(t, kb_a, st_a);
                 }
                 if (i < 2) {
 #pragma unroll
-                    for (int t = 0; t < B_LOADS / 2; ++t) issue_load(A_LOADS + i * (B_LOADS / 2) + t, kb_w, st_prev);
+                    for (int t = 0; t < B_LOADS / 2; ++t) issue_load(A_LOADS + i * (B_LOADS / 2) + t, kb_w, prev_b(st_b));
                 }
                 pend = p[JA - 1];
                 nf0 = nf1;
@@ -358,7 +376,7 @@ __device__ __forceinline__ void prefill_tile(
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            stage = st_next;
+            st_a = sa_next; st_b = sb_next; st_s = ss_next;
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[SN - 1][JA - 1][e] = __builtin_fmaf(pend[e], sc[JA - 1], acc[SN - 1][JA - 1][e]);
@@ -368,10 +386,10 @@ __device__ __forceinline__ void prefill_tile(
     // 16-bit outputs with full-width rows are stored through LDS (see the epilogue)
     const bool lds_epilogue = CD != DSV3_F32 && (N % 8) == 0 && ldc == N;
     const bool f32_lds_epilogue = CD == DSV3_F32 && (N % 4) == 0 && (ldc % 4) == 0 && (SN % 2) == 0;
-    static_assert(SM == 4 || SM == 2, "dispatch below");
+    static_assert(SM >= 2 && SM <= 4, "dispatch below");
     if (!G || ja_live == SM) pipeline(std::integral_constant<int, SM>{});
-    else if (SM == 4 && ja_live == 3) pipeline(std::integral_constant<int, (SM == 4 ? 3 : 1)>{});
-    else if (SM == 4 && ja_live == 2) pipeline(std::integral_constant<int, (SM == 4 ? 2 : 1)>{});
+    else if (SM >= 4 && ja_live == 3) pipeline(std::integral_constant<int, (SM >= 4 ? 3 : 1)>{});
+    else if (SM >= 3 && ja_live == 2) pipeline(std::integral_constant<int, (SM >= 3 ? 2 : 1)>{});
     else if (ja_live == 1)  pipeline(std::integral_constant<int, 1>{});
     else {
         pipeline(std::integral_constant<int, 0>{});
@@ -476,9 +494,11 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
     prefill_tile<CD, G, TM, S>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
 }
 
-// Grouped GEMM over a tile table with slots of up to 256 rows.  A slot with more than 128 rows runs the 256-row
-// configuration (the weights pass through LDS once for up to 256 rows); one with fewer runs the 128-row
-// configuration with its deeper prefetch.  The choice is uniform over the workgroup and needs no host knowledge of
+// Grouped GEMM over a tile table with slots of up to 256 rows.  A slot with more than 192 rows runs the 256-row
+// configuration (the weights pass through LDS once for up to 256 rows), one with 129 .. 192 rows a 192-row
+// configuration whose smaller activation stages leave room for a third weight stage (a group's weights come
+// straight from HBM, and a second block of prefetch is what hides that), one with fewer the 128-row
+// configuration with three stages of both.  The choice is uniform over the workgroup and needs no host knowledge of
 // the group sizes: a layer with a few rows per expert and one with hundreds go through the same launch.
 template <int CD>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
@@ -488,8 +508,11 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
         int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g) {
     const int idx = blockIdx.x / 8, tm = (idx / tiles_n) * 8 + blockIdx.x % 8;
     if (tm >= tiles_m) return;
-    if (g.tile_rows[tm] > 128)
+    const int rows = g.tile_rows[tm];
+    if (rows > 192)
         prefill_tile<CD, true, 256, 2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+    else if (rows > 128)
+        prefill_tile<CD, true, 192, 2, 3>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
     else
         prefill_tile<CD, true, 128, 3>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
 }
@@ -740,7 +763,8 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
         return launch_grouped_skinny(a, a_s, a_rows, b, b_s, c, CD, n, k, num_tiles, tile_group, tile_row0, tile_rows,
                                      b_stride, bs_stride, m < num_tiles ? m : num_tiles, stream);
     GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
-    constexpr int LDS_BYTES = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
+    constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES;               // the largest of the three configurations
+    static_assert(LDS_BYTES >= Cfg<256, 2>::LDS_BYTES && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES, "LDS of the grouped kernel");
     const int64_t tn = (n + BN - 1) / BN;
     if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (num_tiles * tn == 0) return DSV3_OK;
