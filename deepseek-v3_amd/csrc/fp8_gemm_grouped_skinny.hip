@@ -48,9 +48,9 @@ __global__ __launch_bounds__(kWaves * kWave) void fp8_gemm_grouped_skinny_kernel
         const uint8_t* __restrict__ b, const float* __restrict__ b_s, void* __restrict__ c, int c_dtype,
         int N, int K, const int* __restrict__ tile_group, const int* __restrict__ tile_row0,
         const int* __restrict__ tile_rows, int64_t b_stride, int64_t bs_stride) {
-    // K blocks of loads in flight per wavefront: fewer with more wavefronts per workgroup, so that 16 wavefronts per
-    // compute unit stay resident (128 registers each)
-    constexpr int NPF = kWaves == 4 ? 4 : (kWaves == 8 ? 3 : 2);
+    // K blocks of loads in flight per wavefront: three keep the kernel at 128 registers or fewer, i.e. 16 resident
+    // wavefronts per compute unit (four blocks in flight and 12 wavefronts measured slower)
+    constexpr int NPF = kWaves <= 8 ? 3 : 2;
     __shared__ v4f red[kWaves * S * 64];
     const int slot = blockIdx.y;
     const int grp = tile_group[slot];
@@ -166,12 +166,15 @@ int launch_grouped_skinny(const void* a, const float* a_s, const int* a_rows, co
     const int64_t strips = (n + 16 * S - 1) / (16 * S);
     if (strips > 0x7fffffff || num_tiles > 65535) return DSV3_ERR_BAD_SHAPE;
     if (strips == 0 || num_tiles == 0) return DSV3_OK;
-    // wavefronts per workgroup (they split K): at least two K blocks each, and more of them when the strips alone
-    // would leave the chip short of wavefronts.  `groups_hint` is the caller's estimate of the live tile slots.
+    // wavefronts per workgroup (they split K), measured on the two GEMMs of the 256-expert layer: about 8 K blocks
+    // per wavefront for a short K (2048: two wavefronts, 24 against 31 us with four at one token); for a long K
+    // (7168) four wavefronts while the launch has few workgroups and eight once it has thousands of them
+    // (one token: 46 against 50 us; eight tokens: 215 against 228 us).  `groups_hint` is the caller's estimate of
+    // the live tile slots.
     const int64_t kb = k / 128;
-    int waves = 4;
+    int waves = kb < 32 ? 2 : 4;
+    if (kb >= 48 && strips * groups_hint >= 4096) waves = 8;
     static const int forced = getenv("DSV3_GS_WAVES") ? atoi(getenv("DSV3_GS_WAVES")) : 0;
-    while (waves < 16 && strips * groups_hint * waves < 3072 && kb / (waves * 2) >= 2) waves *= 2;
     if (forced) waves = forced;
 #define DSV3_GS(W)                                                                                                     \
     hipLaunchKernelGGL(fp8_gemm_grouped_skinny_kernel<W>, dim3((unsigned)strips, (unsigned)num_tiles), dim3(W * kWave), \
@@ -179,7 +182,8 @@ int launch_grouped_skinny(const void* a, const float* a_s, const int* a_rows, co
                        tile_group, tile_row0, tile_rows, b_stride, bs_stride)
     if (waves >= 16) DSV3_GS(16);
     else if (waves >= 8) DSV3_GS(8);
-    else DSV3_GS(4);
+    else if (waves >= 4) DSV3_GS(4);
+    else DSV3_GS(2);
 #undef DSV3_GS
     return launch_status();
 }
