@@ -71,9 +71,9 @@ size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
     return fp8_gemm_workspace_bytes(m, n, k);
 }
 
-int dsv3_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
-                  void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
-                  void* workspace, size_t workspace_bytes, void* stream) {
+static int fp8_gemm_checked(const void* a, const float* a_s, const void* b, const float* b_s,
+                           void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                           void* workspace, size_t workspace_bytes, void* stream, bool pow2_scales) {
     if (!valid_dtype(c_dtype)) return DSV3_ERR_BAD_DTYPE;
     if (m < 0 || n < 0 || k < 0) return DSV3_ERR_BAD_SHAPE;
     if (k % 128 != 0) return DSV3_ERR_BAD_SHAPE;
@@ -86,7 +86,20 @@ int dsv3_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b
         return DSV3_ERR_MISALIGNED;
     const size_t need = dsv3_fp8_gemm_workspace_bytes(m, n, k);
     if (need > 0 && (!workspace || workspace_bytes < need || !aligned(workspace, 256))) return DSV3_ERR_WORKSPACE;
-    return launch_fp8_gemm(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, (hipStream_t)stream);
+    return launch_fp8_gemm(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, (hipStream_t)stream,
+                           pow2_scales);
+}
+
+int dsv3_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
+                  void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                  void* workspace, size_t workspace_bytes, void* stream) {
+    return fp8_gemm_checked(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, stream, false);
+}
+
+int dsv3_fp8_gemm_pow2(const void* a, const float* a_s, const void* b, const float* b_s,
+                       void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+    return fp8_gemm_checked(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, stream, true);
 }
 
 int dsv3_linear_fp8_fused(int64_t m, int64_t n, int64_t k) {

@@ -70,7 +70,7 @@ int launch_weight_dequant(const void* x, const float* s, void* y, int y_dtype,
 int launch_weight_quant(const void* w, int w_dtype, void* y, float* s, int64_t m, int64_t n, hipStream_t stream);
 int launch_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
                     void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
-                    void* workspace, size_t workspace_bytes, hipStream_t stream);
+                    void* workspace, size_t workspace_bytes, hipStream_t stream, bool pow2_scales = false);
 size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 bool prefill_supported(int64_t m, int64_t n, int64_t k);
 bool stream_supported(int64_t m, int64_t n, int64_t k);
@@ -85,7 +85,7 @@ int launch_linear_fp8(const void* x, const void* b, const float* b_s, void* c, i
                       int64_t k, int scale_fmt, void* workspace, hipStream_t stream);
 bool linear_fp8_supported(int64_t m, int64_t n, int64_t k);
 size_t prefill_workspace_bytes(int64_t m, int64_t n, int64_t k);
-template <int CD>
+template <int CD, bool P2 = false>        // P2: every scale is a power of two (they go into the MFMA's scale operands)
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, void* ws, hipStream_t stream);
 int grouped_tile_rows();

@@ -82,7 +82,10 @@ struct GroupTable {
 };
 
 // One workgroup's tile (grouped mode: tile slot) from start to end; the kernels below are thin wrappers.
-template <int CD, bool G, int TM, int S, int SB = S>
+// P2: every scale is a power of two (act_quant's ue8m0 format and checkpoints whose block scales are stored that
+// way).  The block scales then ride in the MFMA's E8M0 scale operands and the products of all K blocks accumulate
+// inside the matrix core: no fold, no vector-ALU work in the K loop.
+template <int CD, bool G, int TM, int S, int SB = S, bool P2 = false>
 __device__ __forceinline__ void prefill_tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -276,6 +279,78 @@ __device__ __forceinline__ void prefill_tile(
                 st_a = next_a(st_a); st_b = next_b(st_b); st_s = next_s(st_s);
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);
+        } else if constexpr (P2) {
+        // biased exponents (E8M0) of the block's scales: the weights' (MFMA A operand, one value per wavefront) and
+        // the activations' (B operand, the lane's row)
+        int eb, ea[JA], eb_nxt, ea_nxt[JA];
+        auto e8m0 = [](float x) { return (int)(f32_as_u32(x) >> 23); };
+        eb_nxt = e8m0(lds_bs(0));
+#pragma unroll
+        for (int j = 0; j < JA; ++j) ea_nxt[j] = e8m0(lds_as(j, 0));
+        v8i nf0, nf1, mf[JA];
+        {
+            const uint8_t* as_base = lds + a_rd;
+            const uint8_t* bs_base = lds + b_rd;
+            nf0 = join(*(const v4i*)(bs_base + c0), *(const v4i*)(bs_base + c1));
+#pragma unroll
+            for (int j = 0; j < JA; ++j)
+                mf[j] = join(*(const v4i*)(as_base + j * A_JSTRIDE + c0), *(const v4i*)(as_base + j * A_JSTRIDE + c1));
+            nf1 = join(*(const v4i*)(bs_base + 2048 + c0), *(const v4i*)(bs_base + 2048 + c1));
+        }
+        int st_a = 0, st_b = 0, st_s = 0;
+        for (int kb = 0; kb < KB; ++kb) {
+            const int sa_next = next_a(st_a), sb_next = next_b(st_b), ss_next = next_s(st_s);
+            const uint8_t* bs_base = lds + b_rd + st_b * B_STAGE;
+            const uint8_t* as_next = lds + a_rd + sa_next * A_STAGE;
+            const uint8_t* bs_next = lds + b_rd + sb_next * B_STAGE;
+            const int kb_w = min(kb - 1 + SB, KB - 1), kb_a = min(kb + S, KB - 1);
+            eb = eb_nxt;
+#pragma unroll
+            for (int j = 0; j < JA; ++j) ea[j] = ea_nxt[j];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < SN; ++i) {
+                if (i == kSync) {
+                    __builtin_amdgcn_s_waitcnt(kWaitSync);
+                    wg_barrier();
+                    eb_nxt = e8m0(lds_bs(ss_next));
+#pragma unroll
+                    for (int j = 0; j < JA; ++j) ea_nxt[j] = e8m0(lds_as(j, ss_next));
+                    issue_scales(kb_a, ahead_s(st_s));
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                v8i nf2;
+                if (i < kSync)
+                    nf2 = join(*(const v4i*)(bs_base + (i + 2) * 2048 + c0), *(const v4i*)(bs_base + (i + 2) * 2048 + c1));
+                else
+                    nf2 = join(*(const v4i*)(bs_next + (i - kSync) * 2048 + c0), *(const v4i*)(bs_next + (i - kSync) * 2048 + c1));
+#pragma unroll
+                for (int j = 0; j < JA; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(nf0, mf[j], acc[i][j], 0, 0, 0, eb, 0, ea[j]);
+                    if (i == SN - 1) mf[j] = join(*(const v4i*)(as_next + j * A_JSTRIDE + c0), *(const v4i*)(as_next + j * A_JSTRIDE + c1));
+                }
+                if (i >= kSync) {
+                    constexpr int kHalf = (A_LOADS + 1) / 2;
+#pragma unroll
+                    for (int t = (i == kSync ? 0 : kHalf); t < (i == kSync ? kHalf : A_LOADS); ++t) issue_load(t, kb_a, st_a);
+                }
+                if (i < 2) {
+#pragma unroll
+                    for (int t = 0; t < B_LOADS / 2; ++t) issue_load(A_LOADS + i * (B_LOADS / 2) + t, kb_w, prev_b(st_b));
+                }
+                nf0 = nf1;
+                nf1 = nf2;
+                DSV3_SGB(0x100, 2);
+#pragma unroll
+                for (int j = 0; j < JA; ++j) {
+                    DSV3_SGB(0x008, 1);
+                    if (i == SN - 1) DSV3_SGB(0x100, 2);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            st_a = sa_next; st_b = sb_next; st_s = ss_next;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
         } else {
         float sc[JA], sc_nxt[JA];
         {
@@ -485,13 +560,13 @@ __device__ __forceinline__ void prefill_tile(
     }
 }
 
-template <int CD, bool G, int TM, int S>
+template <int CD, bool G, int TM, int S, bool P2 = false>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
         int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, GroupTable g) {
-    prefill_tile<CD, G, TM, S>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+    prefill_tile<CD, G, TM, S, S, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
 }
 
 // Grouped GEMM over a tile table with slots of up to 256 rows.  A slot with more than 192 rows runs the 256-row
@@ -521,7 +596,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
 // tiles over the column tiles [0, tn_tall), the others 128-row tiles over [tn_tall, tn_tall + tn_short).  Workgroups
 // are handed out in index order, so the short tiles fill the compute units that the last, partly filled round of
 // tall tiles would leave idle.
-template <int CD>
+template <int CD, bool P2 = false>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_two_heights_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -530,9 +605,9 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_two_heights_kernel(
     const int short_first = (n_tall + 7) & ~7;        // keeps workgroup index % 8 = XCD for the short tiles too
     const GroupTable none{};
     if ((int)blockIdx.x < n_tall)
-        prefill_tile<CD, false, 256, 2>(a, a_s, b, b_s, c, M, N, K, tm_tall, tn_tall, 0, K / 128, N, none, blockIdx.x);
+        prefill_tile<CD, false, 256, 2, 2, P2>(a, a_s, b, b_s, c, M, N, K, tm_tall, tn_tall, 0, K / 128, N, none, blockIdx.x);
     else if ((int)blockIdx.x >= short_first)
-        prefill_tile<CD, false, 128, 3>(a, a_s, b, b_s, c, M, N, K, (M + 127) / 128, tn_short, tn_tall, K / 128, N, none,
+        prefill_tile<CD, false, 128, 3, 3, P2>(a, a_s, b, b_s, c, M, N, K, (M + 127) / 128, tn_short, tn_tall, K / 128, N, none,
                                         blockIdx.x - short_first);
 }
 
@@ -545,7 +620,7 @@ bool prefill_supported(int64_t m, int64_t n, int64_t k) {
 
 namespace {
 // Launches the column tiles [tn_first, tn_first + tn_count) of every row tile.
-template <int CD, bool G, int TM, int S>
+template <int CD, bool G, int TM, int S, bool P2 = false>
 int launch_kernel(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                   int64_t m, int64_t n, int64_t k, int64_t tm, int64_t tn_first, int64_t tn_count,
                   prefill::GroupTable g, hipStream_t stream, int splits = 1, int64_t ldc = 0) {
@@ -553,7 +628,7 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
     constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
     if ((tm + 8) * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (tm * tn_count == 0) return DSV3_OK;
-    auto kern = fp8_gemm_prefill_kernel<CD, G, TM, S>;
+    auto kern = fp8_gemm_prefill_kernel<CD, G, TM, S, P2>;
     static bool granted[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
@@ -695,7 +770,7 @@ size_t prefill_workspace_bytes(int64_t m, int64_t n, int64_t k) {
 }
 
 // ws must hold prefill_workspace_bytes(m, n, k) bytes
-template <int CD>
+template <int CD, bool P2>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, void* ws, hipStream_t stream) {
     const PrefillPlan p = prefill_plan(m, n, k);
@@ -705,7 +780,7 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
     if (p.tn_short > 0) {
         using namespace prefill;
         constexpr int LDS_BYTES = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
-        auto kern = fp8_gemm_two_heights_kernel<CD>;
+        auto kern = fp8_gemm_two_heights_kernel<CD, P2>;
         static bool granted[64] = {};
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
@@ -724,8 +799,8 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
     auto run = [&](auto cd, void* out, int64_t tn_first, int64_t tn_count, int splits, int64_t ldc) {
         constexpr int OD = decltype(cd)::value;
         if (p.tile_rows == 128)
-            return launch_kernel<OD, false, 128, 3>(a, a_s, b, b_s, out, m, n, k, tm, tn_first, tn_count, none, stream, splits, ldc);
-        return launch_kernel<OD, false, 256, 2>(a, a_s, b, b_s, out, m, n, k, tm, tn_first, tn_count, none, stream, splits, ldc);
+            return launch_kernel<OD, false, 128, 3, P2>(a, a_s, b, b_s, out, m, n, k, tm, tn_first, tn_count, none, stream, splits, ldc);
+        return launch_kernel<OD, false, 256, 2, P2>(a, a_s, b, b_s, out, m, n, k, tm, tn_first, tn_count, none, stream, splits, ldc);
     };
     if (p.tn_plain > 0) {
         const int rc = run(std::integral_constant<int, CD>{}, c, 0, p.tn_plain, 1, 0);
@@ -785,7 +860,8 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
 }
 
 #define DSV3_INST(CD) \
-    template int launch_prefill<CD>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, void*, hipStream_t); \
+    template int launch_prefill<CD, false>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, void*, hipStream_t); \
+    template int launch_prefill<CD, true>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, void*, hipStream_t); \
     template int launch_grouped<CD>(const void*, const float*, const int*, const void*, const float*, void*, int64_t, int64_t, int64_t, \
                                     int64_t, const int*, const int*, const int*, int64_t, int64_t, hipStream_t);
 DSV3_INST(DSV3_BF16)

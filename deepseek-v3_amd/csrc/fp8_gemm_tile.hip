@@ -286,7 +286,7 @@ bool to_large_m_kernel(int64_t m, int64_t n, int64_t k) {
 
 template <int CD>
 int launch_typed(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
-                 int64_t m, int64_t n, int64_t k, void* ws, hipStream_t st) {
+                 int64_t m, int64_t n, int64_t k, void* ws, hipStream_t st, bool pow2) {
     if (k == 0) {   // empty sum: c = 0
         const int64_t mn0 = m * n;
         hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn0 + 255) / 256)), dim3(256), 0, st,
@@ -306,7 +306,8 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
                            (const float*)ws, (typename OutT<CD>::type*)c, mn, splits);
         return launch_status();
     }
-    if (to_prefill) return launch_prefill<CD>(a, a_s, b, b_s, c, m, n, k, ws, st);
+    if (to_prefill) return pow2 ? launch_prefill<CD, true>(a, a_s, b, b_s, c, m, n, k, ws, st)
+                                : launch_prefill<CD, false>(a, a_s, b, b_s, c, m, n, k, ws, st);
     const Plan p = make_plan(m, n, k);
     if (p.splits == 1) {
         if (p.bm == 32) return launch_cfg<32, 128, 32, 32, CD>(a, a_s, b, b_s, c, m, n, k, 1, p.kb_per_split, st);
@@ -362,12 +363,12 @@ size_t fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
 
 int launch_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
                     void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
-                    void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                    void* workspace, size_t workspace_bytes, hipStream_t stream, bool pow2_scales) {
     (void)workspace_bytes;
     switch (c_dtype) {
-        case DSV3_BF16: return launch_typed<DSV3_BF16>(a, a_s, b, b_s, c, m, n, k, workspace, stream);
-        case DSV3_F16:  return launch_typed<DSV3_F16>(a, a_s, b, b_s, c, m, n, k, workspace, stream);
-        case DSV3_F32:  return launch_typed<DSV3_F32>(a, a_s, b, b_s, c, m, n, k, workspace, stream);
+        case DSV3_BF16: return launch_typed<DSV3_BF16>(a, a_s, b, b_s, c, m, n, k, workspace, stream, pow2_scales);
+        case DSV3_F16:  return launch_typed<DSV3_F16>(a, a_s, b, b_s, c, m, n, k, workspace, stream, pow2_scales);
+        case DSV3_F32:  return launch_typed<DSV3_F32>(a, a_s, b, b_s, c, m, n, k, workspace, stream, pow2_scales);
         default: return DSV3_ERR_BAD_DTYPE;
     }
 }

@@ -47,6 +47,17 @@ def fp8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Ten
     return torch.ops.dsv3fp8.fp8_gemm(a, a_s, b, b_s, ops.dtype_code(torch.get_default_dtype()))
 
 
+def fp8_gemm_pow2(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Tensor) -> torch.Tensor:
+    """``fp8_gemm`` for scales that are all powers of two -- ``act_quant(..., scale_fmt="ue8m0")`` activations
+    (inference/kernel.py:29-31) on a weight whose block scales are stored that way (the format of
+    inference/configs/config_v3.1.json:22).  Not in the reference, whose ``fp8_gemm`` multiplies by the scales
+    whatever they are; here the caller vouches for the property and the large-M kernel hands the scales to the
+    matrix instruction instead of multiplying per K block."""
+    assert a.is_contiguous() and b.is_contiguous(), 'Input tensors must be contiguous'
+    assert a_s.is_contiguous() and b_s.is_contiguous(), 'Scaling factor tensors must be contiguous'
+    return torch.ops.dsv3fp8.fp8_gemm_pow2(a, a_s, b, b_s, ops.dtype_code(torch.get_default_dtype()))
+
+
 def fp8_gemm_f32(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Tensor) -> torch.Tensor:
     """``fp8_gemm`` with the binary32 accumulators returned unrounded (not in the
     reference; the output-type knob the reference reaches through the default dtype)."""

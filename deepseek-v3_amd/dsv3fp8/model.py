@@ -22,7 +22,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from . import ops
-from .kernel import act_quant, fp8_gemm, weight_dequant
+from .kernel import act_quant, fp8_gemm, fp8_gemm_pow2, weight_dequant
 
 world_size = 1
 rank = 0
@@ -62,6 +62,21 @@ class ModelArgs:
     mscale: float = 1.
 
 
+def _scales_are_powers_of_two(weight: torch.Tensor) -> bool:
+    """Whether every block scale of an fp8 weight is a power of two (checkpoints made for ``scale_fmt = "ue8m0"``,
+    inference/configs/config_v3.1.json:22, store them that way).  Looked at once per version of the scale tensor
+    (one device-to-host read), never while a graph is being captured."""
+    scale = weight.scale
+    cached = getattr(weight, "_dsv3_pow2", None)
+    if cached is not None and cached[0] == scale._version:
+        return cached[1]
+    if torch.cuda.is_current_stream_capturing():
+        return False
+    flag = bool(((scale.detach().view(torch.int32) & 0x7FFFFF) == 0).all().item()) and bool((scale > 0).all().item())
+    weight._dsv3_pow2 = (scale._version, flag)
+    return flag
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            scale_fmt: Optional[str] = None) -> torch.Tensor:
     """y = x @ weight.T + bias with the reference's three-way dispatch (model.py:153-163): wide weights go to
@@ -71,7 +86,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         return F.linear(x, weight, bias)
     if gemm_impl == "bf16":
         return F.linear(x, weight_dequant(weight, weight.scale), bias)
-    if (x.is_cuda and x.is_contiguous() and weight.is_contiguous() and block_size == 128
+    if (scale_fmt == "ue8m0" and x.is_cuda and block_size == 128 and x.numel() > 64 * x.size(-1)
+            and _scales_are_powers_of_two(weight)):
+        # activation and weight scales are all powers of two: they go into the matrix instruction's scale operands
+        xq, xs = act_quant(x, block_size, scale_fmt)
+        y = fp8_gemm_pow2(xq, xs, weight, weight.scale)
+    elif (x.is_cuda and x.is_contiguous() and weight.is_contiguous() and block_size == 128
             and x.size(-1) % block_size == 0):
         # the same two steps behind one op, which runs them as a single launch for few rows (decode)
         fmt = ops._lib.SCALE_FMT_UE8M0 if scale_fmt == "ue8m0" else ops._lib.SCALE_FMT_NONE

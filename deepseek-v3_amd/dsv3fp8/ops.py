@@ -24,6 +24,7 @@ _libdef.define("act_quant(Tensor x, int block_size, int scale_fmt) -> (Tensor, T
 _libdef.define("weight_dequant(Tensor x, Tensor s, int block_size, int out_dtype) -> Tensor")
 _libdef.define("weight_quant(Tensor w, int block_size) -> (Tensor, Tensor)")
 _libdef.define("fp8_gemm(Tensor a, Tensor a_s, Tensor b, Tensor b_s, int out_dtype) -> Tensor")
+_libdef.define("fp8_gemm_pow2(Tensor a, Tensor a_s, Tensor b, Tensor b_s, int out_dtype) -> Tensor")
 _libdef.define("linear_fp8(Tensor x, Tensor b, Tensor b_s, int scale_fmt, int out_dtype) -> Tensor")
 _libdef.define("group_tiles(Tensor counts, int max_tiles) -> (Tensor, Tensor, Tensor)")
 _libdef.define("moe_route(Tensor indices, Tensor weights, int experts, bool shared_group) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)")
@@ -105,7 +106,7 @@ def _weight_quant_meta(w, block_size):
     return torch.empty_like(w, dtype=FP8), w.new_empty(-(-m // block_size), -(-n // block_size), dtype=torch.float32)
 
 
-def _fp8_gemm_dev(a, a_s, b, b_s, out_dtype: int):
+def _fp8_gemm_dev(a, a_s, b, b_s, out_dtype: int, entry: str = "dsv3_fp8_gemm"):
     k = a.size(-1)
     m = a.numel() // k if k else 0
     n = b.size(0)
@@ -114,12 +115,16 @@ def _fp8_gemm_dev(a, a_s, b, b_s, out_dtype: int):
         stream = _stream(a)
         need = _lib.lib.dsv3_fp8_gemm_workspace_bytes(m, n, k)
         ws = _workspace(a, need, stream) if need else None
-        rc = _lib.lib.dsv3_fp8_gemm(a.data_ptr(), a_s.data_ptr(), b.data_ptr(), b_s.data_ptr(),
-                                    c.data_ptr(), out_dtype, m, n, k,
-                                    ws.data_ptr() if ws is not None else None,
-                                    ws.numel() if ws is not None else 0, stream)
-    _lib.check(rc, "dsv3_fp8_gemm")
+        rc = getattr(_lib.lib, entry)(a.data_ptr(), a_s.data_ptr(), b.data_ptr(), b_s.data_ptr(),
+                                      c.data_ptr(), out_dtype, m, n, k,
+                                      ws.data_ptr() if ws is not None else None,
+                                      ws.numel() if ws is not None else 0, stream)
+    _lib.check(rc, entry)
     return c
+
+
+def _fp8_gemm_pow2_dev(a, a_s, b, b_s, out_dtype: int):
+    return _fp8_gemm_dev(a, a_s, b, b_s, out_dtype, "dsv3_fp8_gemm_pow2")
 
 
 def _fp8_gemm_meta(a, a_s, b, b_s, out_dtype):
@@ -326,7 +331,9 @@ _libimpl.impl("act_quant", _act_quant_dev, "CUDA")
 _libimpl.impl("weight_dequant", _weight_dequant_dev, "CUDA")
 _libimpl.impl("weight_quant", _weight_quant_dev, "CUDA")
 _libimpl.impl("fp8_gemm", _fp8_gemm_dev, "CUDA")
+_libimpl.impl("fp8_gemm_pow2", _fp8_gemm_pow2_dev, "CUDA")
 _libimpl.impl("act_quant", _act_quant_meta, "Meta")
 _libimpl.impl("weight_dequant", _weight_dequant_meta, "Meta")
 _libimpl.impl("weight_quant", _weight_quant_meta, "Meta")
 _libimpl.impl("fp8_gemm", _fp8_gemm_meta, "Meta")
+_libimpl.impl("fp8_gemm_pow2", _fp8_gemm_meta, "Meta")

@@ -131,6 +131,19 @@ int dsv3_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b
                   void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
                   void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * dsv3_fp8_gemm for scales that are all powers of two: what act_quant produces with scale_fmt "ue8m0"
+ * (inference/kernel.py:29-31) and what checkpoints made for that format store as block scales
+ * (inference/configs/config_v3.1.json:22).  The caller guarantees it for every element of a_s and b_s; it is not
+ * checked.  For M > 64 the block scales then travel in the E8M0 scale operands of the gfx950 matrix instruction
+ * and all K blocks accumulate inside the matrix core (the binary32 multiply-add per block and output element of
+ * the general kernel disappears; the result differs from dsv3_fp8_gemm's only in the rounding of the sums).
+ * Other shapes run the same kernels as dsv3_fp8_gemm.  Same arguments, workspace and errors.
+ */
+int dsv3_fp8_gemm_pow2(const void* a, const float* a_s, const void* b, const float* b_s,
+                       void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
 /* Bytes of scratch dsv3_fp8_gemm needs for this problem (0 when none). */
 size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 

@@ -75,8 +75,9 @@ def test_weight_quant_validation(L):
     assert f(None, L.BF16, None, None, 0, 128, 128, None) == 0
 
 
-def test_fp8_gemm_validation(L):
-    f = L.lib.dsv3_fp8_gemm
+@pytest.mark.parametrize("entry", ["dsv3_fp8_gemm", "dsv3_fp8_gemm_pow2"])
+def test_fp8_gemm_validation(L, entry):
+    f = getattr(L.lib, entry)
     ws = L.lib.dsv3_fp8_gemm_workspace_bytes
     assert f(None, A16, A16, A16, A16, L.BF16, 4, 128, 128, None, 0, None) == 1
     assert f(A16, A16, A16, A16, None, L.BF16, 4, 128, 128, None, 0, None) == 1

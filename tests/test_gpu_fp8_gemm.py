@@ -241,3 +241,66 @@ def test_partly_filled_last_round(K, m, n, k, sliced):
     x = workloads.activations(m, k, seed=m)
     w8, ws = workloads.weight(n, k, seed=n % 89)
     _check(K, x, w8, ws)
+
+
+def _pow2_problem(m, n, k, seed):
+    """Activations quantised with power-of-two scales (ue8m0) and a weight whose block scales were rounded up to
+    powers of two before quantising -- the format of config_v3.1 checkpoints."""
+    from dsv3fp8 import workloads
+    x = workloads.activations(m, k, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    w = (torch.randn(n, k, generator=g) * 0.02).bfloat16().float()
+    nb, kb = -(-n // 128), k // 128
+    wp = torch.zeros(nb * 128, k)
+    wp[:n] = w
+    amax = wp.view(nb, 128, kb, 128).abs().amax(dim=(1, 3)).clamp_min(1e-4)
+    ws = torch.pow(2.0, torch.ceil(torch.log2(amax / 448.0)))
+    w8 = (wp.view(nb, 128, kb, 128) / ws[:, None, :, None]).reshape(nb * 128, k)[:n].contiguous().to(torch.float8_e4m3fn)
+    a, a_s = oracle.act_quant(x, 128, "ue8m0")
+    assert bool(((a_s.view(torch.int32) & 0x7FFFFF) == 0).all()) and bool(((ws.view(torch.int32) & 0x7FFFFF) == 0).all())
+    return a, a_s, w8, ws
+
+
+@pytest.mark.parametrize("m,n,k", [
+    (300, 640, 1024),      # short tiles
+    (2050, 8192, 384),     # tall tiles, a 2-row edge tile, odd number of K blocks
+    (1030, 17000, 512),    # two tile heights in one launch, ragged N
+    (130, 4096, 2048),     # K range cut into slices (binary32 slabs)
+    (16, 1536, 7168),      # few rows: the same kernels as fp8_gemm
+])
+def test_power_of_two_scales_in_the_matrix_instruction(K, m, n, k):
+    a, a_s, w8, ws = _pow2_problem(m, n, k, seed=m)
+    ref = oracle.fp8_gemm_f32(a, a_s, w8, ws)
+    old = torch.get_default_dtype()
+    try:
+        torch.set_default_dtype(torch.float32)
+        c32 = K.fp8_gemm_pow2(a.cuda(), a_s.cuda(), w8.cuda(), ws.cuda())
+        gen = K.fp8_gemm(a.cuda(), a_s.cuda(), w8.cuda(), ws.cuda())
+        torch.set_default_dtype(torch.bfloat16)
+        c16 = K.fp8_gemm_pow2(a.cuda(), a_s.cuda(), w8.cuda(), ws.cuda())
+    finally:
+        torch.set_default_dtype(old)
+    rms = ref.pow(2).mean().sqrt().item()
+    assert (c32.cpu() - ref).abs().max().item() <= TOL * rms
+    assert (c32 - gen).abs().max().item() <= 1e-4 * rms                  # same products, another order of additions
+    assert torch.equal(c16.cpu().view(torch.int16), c32.cpu().to(torch.bfloat16).view(torch.int16))
+
+
+def test_power_of_two_scales_exact_small_integers(K):
+    """Small-integer fp8 values (block sums below 2^11) and power-of-two scales whose products span seven binades
+    far from 1: every partial sum fits 24 bits, so the result is independent of the summation order and the scale
+    operands must reproduce 2^e exactly."""
+    g = torch.Generator().manual_seed(4)
+    for (m, n, k) in [(200, 384, 512), (600, 1000, 1280)]:
+        a = torch.randint(-4, 5, (m, k), generator=g).float().to(torch.float8_e4m3fn)
+        b = torch.randint(-4, 5, (n, k), generator=g).float().to(torch.float8_e4m3fn)
+        a_s = torch.pow(2.0, torch.randint(-12, -8, (m, k // 128), generator=g).float())
+        b_s = torch.pow(2.0, torch.randint(-10, -6, (-(-n // 128), k // 128), generator=g).float())
+        ref = oracle.fp8_gemm_f32(a, a_s, b, b_s)
+        old = torch.get_default_dtype()
+        torch.set_default_dtype(torch.float32)
+        try:
+            c32 = K.fp8_gemm_pow2(a.cuda(), a_s.cuda(), b.cuda(), b_s.cuda())
+        finally:
+            torch.set_default_dtype(old)
+        assert torch.equal(c32.cpu(), ref)

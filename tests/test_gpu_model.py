@@ -80,6 +80,38 @@ def test_scale_fmt_only_reaches_plain_linear(M):
     _close(yc, oracle.linear(x, w8, scale=s, scale_fmt=None), tol=1e-2)
 
 
+def test_linear_with_power_of_two_scales_takes_the_scaled_matrix_instruction(M, monkeypatch):
+    """scale_fmt = "ue8m0" on a weight whose block scales are powers of two (config_v3.1-style checkpoints) and more
+    than 64 rows: linear() calls fp8_gemm_pow2; any other weight, or few rows, takes the general path."""
+    M.gemm_impl = "fp8"
+    M.Linear.scale_fmt = "ue8m0"
+    with torch.device("cuda"):
+        lin = M.Linear(512, 384)
+    g = torch.Generator().manual_seed(7)
+    w = (torch.randn(384, 512, generator=g) * 0.05).bfloat16().float()
+    amax = w.view(3, 128, 4, 128).abs().amax(dim=(1, 3))
+    s = torch.pow(2.0, torch.ceil(torch.log2(amax / 448.0)))
+    w8 = (w.view(3, 128, 4, 128) / s[:, None, :, None]).reshape(384, 512).to(FP8)
+    with torch.no_grad():
+        lin.weight.copy_(w8.cuda()); lin.scale.copy_(s.cuda())
+    calls = []
+    real = M.fp8_gemm_pow2
+    monkeypatch.setattr(M, "fp8_gemm_pow2", lambda *a: (calls.append(a[0].shape[0]), real(*a))[1])
+    x = torch.randn(300, 512, generator=g).bfloat16()
+    with torch.inference_mode():
+        y = lin(x.cuda())
+        y_few = lin(x[:8].cuda())
+    assert calls == [300]
+    _close(y, oracle.linear(x, w8, scale=s, scale_fmt="ue8m0"), tol=1e-2)
+    _close(y_few, oracle.linear(x[:8], w8, scale=s, scale_fmt="ue8m0"), tol=1e-2)
+    with torch.no_grad():
+        lin.scale.mul_(1.5)                                   # no longer powers of two: noticed through the version
+    with torch.inference_mode():
+        y2 = lin(x.cuda())
+    assert calls == [300]
+    _close(y2, oracle.linear(x, w8, scale=s * 1.5, scale_fmt="ue8m0"), tol=1e-2)
+
+
 def test_moe_layer_small(M):
     M.gemm_impl = "fp8"
     args = M.ModelArgs(dim=256, inter_dim=512, moe_inter_dim=128, n_routed_experts=8, n_shared_experts=1,
