@@ -304,3 +304,26 @@ def test_power_of_two_scales_exact_small_integers(K):
         finally:
             torch.set_default_dtype(old)
         assert torch.equal(c32.cpu(), ref)
+
+
+def test_seeded_shape_sweep(K):
+    """Thirty seeded shapes across the dispatcher's regimes (few rows, mid M with and without K slicing, whole
+    rounds, partly filled last rounds, ragged M and N), each against the oracle."""
+    from dsv3fp8 import workloads
+    g = torch.Generator().manual_seed(2024)
+
+    def pick(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+    shapes = []
+    while len(shapes) < 30:
+        m = pick(1, 64) if len(shapes) % 5 == 0 else pick(65, 2600)
+        n = pick(1, 300) if len(shapes) % 7 == 0 else pick(256, 9000)
+        k = 128 * pick(1, 16)
+        if m * n * k <= 1.2e10:
+            shapes.append((m, n, k))
+    worst = 0.0
+    for i, (m, n, k) in enumerate(shapes):
+        x = workloads.activations(m, k, seed=100 + i)
+        w8, ws = workloads.weight(n, k, seed=200 + i)
+        worst = max(worst, _check(K, x, w8, ws))
+    assert worst <= TOL

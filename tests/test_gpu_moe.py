@@ -87,6 +87,43 @@ def test_fp8_gemm_grouped_vs_oracle(K, counts, n, k, gather):
         row += c
 
 
+def test_fp8_gemm_grouped_seeded_tables(K):
+    """Twelve seeded tables mixing empty, tiny, 129-192-row, 193-256-row and multi-tile groups (every tile
+    configuration of the grouped kernel, and the weight-streaming kernel when the total is small)."""
+    from dsv3fp8 import ops
+    gen = torch.Generator().manual_seed(77)
+    kinds = [(0, 0), (1, 16), (17, 128), (129, 192), (193, 256), (257, 600)]
+    for case in range(12):
+        groups = int(torch.randint(1, 9, (1,), generator=gen))
+        if case % 4 == 3:                                    # a small launch: at most 320 rows in all
+            counts = [int(torch.randint(0, 40, (1,), generator=gen)) for _ in range(groups)]
+        else:
+            counts = []
+            for _ in range(groups):
+                lo, hi = kinds[int(torch.randint(0, len(kinds), (1,), generator=gen))]
+                counts.append(int(torch.randint(lo, hi + 1, (1,), generator=gen)))
+        if sum(counts) == 0:
+            counts[0] = 3
+        n = 8 * int(torch.randint(4, 80, (1,), generator=gen))
+        k = 128 * int(torch.randint(1, 7, (1,), generator=gen))
+        gather = bool(case % 2)
+        xq, xs, w, a_rows = _grouped_case(counts, n, k, 300 + case, gather)
+        rows = sum(counts)
+        R, tg, t0, tr = _tables(counts, rows // ops.grouped_tile_rows() + len(counts))
+        b = torch.stack([wi[0].view(torch.uint8) for wi in w]).view(FP8).cuda()
+        b_s = torch.stack([wi[1] for wi in w]).cuda()
+        out = torch.ops.dsv3fp8.fp8_gemm_grouped(xq.cuda(), xs.cuda(), a_rows.cuda() if gather else None, b, b_s, rows,
+                                                 tg, t0, tr, ops.dtype_code(torch.float32)).cpu()
+        row = 0
+        for gi, c in enumerate(counts):
+            if c:
+                idx = a_rows[row:row + c].long() if gather else torch.arange(row, row + c)
+                ref = oracle.fp8_gemm_f32(xq[idx], xs[idx], w[gi][0], w[gi][1])
+                err = (out[row:row + c] - ref).abs().max().item()
+                assert err <= 1e-2 * ref.pow(2).mean().sqrt().item(), (case, counts, n, k, gi, err)
+            row += c
+
+
 @pytest.mark.parametrize("fmt", [None, "ue8m0"])
 def test_swiglu_quant(K, fmt):
     g = torch.Generator().manual_seed(3)
