@@ -651,16 +651,19 @@ inline int env_tile_rows() { const char* e = getenv("DSV3_PREFILL_TILE"); return
 }  // namespace
 
 // Tile height, K slicing and the last partial round.  A K block of a 256-row tile costs about 1.64x one of a
-// 128-row tile (measured, K = 7168) and the tiles are dealt over 256 compute units in whole rounds.  Three kinds of
+// 128-row tile (measured, K = 7168) and the tiles are dealt over 256 compute units in whole rounds.  Four kinds of
 // plan, compared by rounds x K blocks per workgroup x per-block cost:
 //   plain   all tiles in one launch;
 //   sliced  when the tiles do not fill a round: the K range cut into up to 8 slices of at least 8 blocks that run
 //           as separate workgroups and write binary32 partial sums ("slabs"), added in a fixed order by a second
 //           kernel;
 //   hybrid  the column tiles that fill whole rounds as a plain launch, the remaining columns (less than a round
-//           of tiles) as a sliced launch -- instead of a last round that leaves most of the chip idle.
-// (M = 4096 x N = 18432: plain, 5 rounds of tall tiles beat 9 of short ones; M = 1024: hybrid, 256 tall tiles + 32
-// tall tiles in 8 slices; M = 192 ... 256: sliced, 72 tall tiles in 3 slices; M = 128: sliced, 72 short tiles.)
+//           of tiles) as a sliced launch -- instead of a last round that leaves most of the chip idle;
+//   two heights  tall tiles for the first column tiles and short tiles for the last ones, in ONE launch: the short
+//           tiles start on whichever compute unit is free first and fill the partly filled last round.
+// (M = 4096 x N = 18432: two heights, 4 rounds of tall tiles + 1 of short ones instead of 5 of tall; M = 1024:
+// hybrid, 256 tall tiles + 32 tall tiles in 8 slices; M = 192 ... 256: sliced, 72 tall tiles in 3 slices; M = 128:
+// sliced, 72 short tiles.)
 namespace {
 struct PrefillPlan {
     int tile_rows;      // 128 or 256
