@@ -9,5 +9,6 @@ if __name__ == "__main__":
     parser = ArgumentParser()
     parser.add_argument("--input-bf16-hf-path", type=str, required=True)
     parser.add_argument("--output-fp8-hf-path", type=str, required=True)
+    parser.add_argument("--scale-fmt", type=str, default=None, choices=[None, "ue8m0"])
     args = parser.parse_args()
-    main(args.input_bf16_hf_path, args.output_fp8_hf_path)
+    main(args.input_bf16_hf_path, args.output_fp8_hf_path, scale_fmt=args.scale_fmt)

@@ -56,14 +56,15 @@ int dsv3_weight_dequant(const void* x, const float* s, void* y, int y_dtype,
 }
 
 int dsv3_weight_quant(const void* w, int w_dtype, void* y, float* s,
-                      int64_t m, int64_t n, int block_size, void* stream) {
+                      int64_t m, int64_t n, int block_size, int scale_fmt, void* stream) {
     if (!valid_dtype(w_dtype)) return DSV3_ERR_BAD_DTYPE;
+    if (scale_fmt != DSV3_SCALE_FMT_NONE && scale_fmt != DSV3_SCALE_FMT_UE8M0) return DSV3_ERR_BAD_DTYPE;
     if (block_size != 128) return DSV3_ERR_BAD_BLOCK;
     if (m < 0 || n < 0) return DSV3_ERR_BAD_SHAPE;
     if (m == 0 || n == 0) return DSV3_OK;
     if (!w || !y || !s) return DSV3_ERR_NULL_POINTER;
     if (!aligned(s, 4) || !aligned(w, w_dtype == DSV3_F32 ? 4 : 2)) return DSV3_ERR_MISALIGNED;
-    return launch_weight_quant(w, w_dtype, y, s, m, n, (hipStream_t)stream);
+    return launch_weight_quant(w, w_dtype, y, s, m, n, scale_fmt, (hipStream_t)stream);
 }
 
 size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {

@@ -67,7 +67,8 @@ int launch_act_quant(const void* x, int x_dtype, void* y, float* s, int64_t nume
                      int block_size, int scale_fmt, hipStream_t stream);
 int launch_weight_dequant(const void* x, const float* s, void* y, int y_dtype,
                           int64_t m, int64_t n, int block_size, hipStream_t stream);
-int launch_weight_quant(const void* w, int w_dtype, void* y, float* s, int64_t m, int64_t n, hipStream_t stream);
+int launch_weight_quant(const void* w, int w_dtype, void* y, float* s, int64_t m, int64_t n, int scale_fmt,
+                        hipStream_t stream);
 int launch_fp8_gemm(const void* a, const float* a_s, const void* b, const float* b_s,
                     void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
                     void* workspace, size_t workspace_bytes, hipStream_t stream, bool pow2_scales = false);

@@ -4,6 +4,8 @@
 // its scale is taken and cropped afterwards; scale tensor shape inference/model.py:184-187).
 //
 //     s[i,j] = max(amax(block i,j), 1e-4) / 448        w8 = e4m3( w / s[i,j] )        so that  w ~= w8 * s
+// (scale_fmt ue8m0: s rounded up to a power of two first, the format of checkpoints made for
+// inference/configs/config_v3.1.json:22)
 //
 // the arithmetic of act_quant (inference/kernel.py:23-35) applied to a square block: amax, the clamp that keeps an
 // all-zero block finite, an IEEE division by 448, a correctly rounded quotient, round-to-nearest-even to e4m3.
@@ -63,7 +65,7 @@ template <int CTRL> __device__ __forceinline__ float dpp_max(float v) {
 // inside or outside the matrix; otherwise every element is guarded on its own.
 template <int XD, bool VEC>
 __global__ __launch_bounds__(kThreads) void weight_quant_kernel(
-        const void* __restrict__ w, uint8_t* __restrict__ y, float* __restrict__ s, int m, int n, int nb) {
+        const void* __restrict__ w, uint8_t* __restrict__ y, float* __restrict__ s, int m, int n, int nb, int ue8m0) {
     __shared__ float wave_max[kThreads / kWave];
     const int t = threadIdx.x;
     const int col = blockIdx.x * 128 + (t & 15) * 8;           // first of the thread's 8 columns
@@ -102,7 +104,12 @@ __global__ __launch_bounds__(kThreads) void weight_quant_kernel(
     __syncthreads();
     amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
     amax = fmaxf(amax, 1e-4f);
-    const float sc = amax / 448.f;
+    float sc = amax / 448.f;
+    if (ue8m0) {                                // round the scale up to a power of two, as act_quant does (kernel.py:29-31)
+        uint32_t bits = f32_as_u32(sc);
+        bits = ((bits >> 23) + ((bits & 0x7fffffu) ? 1u : 0u)) << 23;
+        sc = u32_as_f32(bits);
+    }
     if (t == 0) s[(int64_t)blockIdx.y * nb + blockIdx.x] = sc;
 
     const float r = 1.0f / sc;
@@ -133,27 +140,29 @@ __global__ __launch_bounds__(kThreads) void weight_quant_kernel(
 }
 
 template <int XD>
-int launch1(const void* w, void* y, float* s, int64_t m, int64_t n, hipStream_t stream) {
+int launch1(const void* w, void* y, float* s, int64_t m, int64_t n, int ue8m0, hipStream_t stream) {
     const int64_t mb = (m + 127) / 128, nb = (n + 127) / 128;
     if (mb > 65535 || nb > 0x7fffffff || m > 0x7fffffff || n > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     const bool vec = (n % 8) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)y % 8) == 0;
     const dim3 grid((unsigned)nb, (unsigned)mb);
     if (vec)
         hipLaunchKernelGGL((weight_quant_kernel<XD, true>), grid, dim3(kThreads), 0, stream, w, (uint8_t*)y, s,
-                           (int)m, (int)n, (int)nb);
+                           (int)m, (int)n, (int)nb, ue8m0);
     else
         hipLaunchKernelGGL((weight_quant_kernel<XD, false>), grid, dim3(kThreads), 0, stream, w, (uint8_t*)y, s,
-                           (int)m, (int)n, (int)nb);
+                           (int)m, (int)n, (int)nb, ue8m0);
     return launch_status();
 }
 
 }  // namespace
 
-int launch_weight_quant(const void* w, int w_dtype, void* y, float* s, int64_t m, int64_t n, hipStream_t stream) {
+int launch_weight_quant(const void* w, int w_dtype, void* y, float* s, int64_t m, int64_t n, int scale_fmt,
+                        hipStream_t stream) {
+    const int ue8m0 = scale_fmt == DSV3_SCALE_FMT_UE8M0;
     switch (w_dtype) {
-        case DSV3_BF16: return launch1<DSV3_BF16>(w, y, s, m, n, stream);
-        case DSV3_F16:  return launch1<DSV3_F16>(w, y, s, m, n, stream);
-        case DSV3_F32:  return launch1<DSV3_F32>(w, y, s, m, n, stream);
+        case DSV3_BF16: return launch1<DSV3_BF16>(w, y, s, m, n, ue8m0, stream);
+        case DSV3_F16:  return launch1<DSV3_F16>(w, y, s, m, n, ue8m0, stream);
+        case DSV3_F32:  return launch1<DSV3_F32>(w, y, s, m, n, ue8m0, stream);
         default: return DSV3_ERR_BAD_DTYPE;
     }
 }

@@ -23,7 +23,7 @@ EXPORTS = {
     "dsv3_status_string": (c_char_p, [c_int]),
     "dsv3_act_quant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]),
     "dsv3_weight_dequant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p]),
-    "dsv3_weight_quant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
+    "dsv3_weight_quant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]),
     "dsv3_fp8_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                               c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "dsv3_fp8_gemm_pow2": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,

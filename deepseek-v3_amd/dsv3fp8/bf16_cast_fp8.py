@@ -13,6 +13,8 @@ are (model.py:100, 563-566, 769).  Shards keep their file names; the index gains
 A weight sharded afterwards along a dimension (convert.py:67-70) keeps whole scale blocks per shard as long as the
 shard size is a multiple of 128, which holds for every tensor of the released configurations.
 
+``--scale-fmt ue8m0`` rounds every block scale up to a power of two (inference/configs/config_v3.1.json:22).
+
 Streams tensor by tensor (``safe_open``): the device holds one weight, its FP8 image and its scales at a time.
 """
 from __future__ import annotations
@@ -21,7 +23,7 @@ import json
 import os
 from argparse import ArgumentParser
 from glob import glob
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 from safetensors import safe_open
@@ -39,7 +41,7 @@ def is_fp8_weight(name: str, tensor: torch.Tensor) -> bool:
             and tensor.dim() == 2 and tensor.element_size() > 1)
 
 
-def main(bf16_path: str, fp8_path: str, device: str = "cuda") -> None:
+def main(bf16_path: str, fp8_path: str, device: str = "cuda", scale_fmt: Optional[str] = None) -> None:
     os.makedirs(fp8_path, exist_ok=True)
     index_file = os.path.join(bf16_path, "model.safetensors.index.json")
     weight_map: Dict[str, str] = {}
@@ -54,7 +56,7 @@ def main(bf16_path: str, fp8_path: str, device: str = "cuda") -> None:
                 tensor = shard.get_tensor(name)
                 weight_map[name] = file_name
                 if is_fp8_weight(name, tensor):
-                    w8, scale = weight_quant(tensor.contiguous())
+                    w8, scale = weight_quant(tensor.contiguous(), scale_fmt=scale_fmt)
                     new_state_dict[name] = w8.cpu()
                     new_state_dict[f"{name}_scale_inv"] = scale.cpu()
                     weight_map[f"{name}_scale_inv"] = file_name
@@ -69,5 +71,7 @@ if __name__ == "__main__":
     parser = ArgumentParser()
     parser.add_argument("--input-bf16-hf-path", type=str, required=True)
     parser.add_argument("--output-fp8-hf-path", type=str, required=True)
+    parser.add_argument("--scale-fmt", type=str, default=None, choices=[None, "ue8m0"],
+                        help="ue8m0: block scales rounded up to powers of two (the format of config_v3.1.json)")
     a = parser.parse_args()
-    main(a.input_bf16_hf_path, a.output_fp8_hf_path)
+    main(a.input_bf16_hf_path, a.output_fp8_hf_path, scale_fmt=a.scale_fmt)

@@ -22,7 +22,7 @@ FP8 = torch.float8_e4m3fn
 _libdef = torch.library.Library("dsv3fp8", "DEF")
 _libdef.define("act_quant(Tensor x, int block_size, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("weight_dequant(Tensor x, Tensor s, int block_size, int out_dtype) -> Tensor")
-_libdef.define("weight_quant(Tensor w, int block_size) -> (Tensor, Tensor)")
+_libdef.define("weight_quant(Tensor w, int block_size, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("fp8_gemm(Tensor a, Tensor a_s, Tensor b, Tensor b_s, int out_dtype) -> Tensor")
 _libdef.define("fp8_gemm_pow2(Tensor a, Tensor a_s, Tensor b, Tensor b_s, int out_dtype) -> Tensor")
 _libdef.define("linear_fp8(Tensor x, Tensor b, Tensor b_s, int scale_fmt, int out_dtype) -> Tensor")
@@ -90,18 +90,18 @@ def _weight_dequant_meta(x, s, block_size, out_dtype):
     return torch.empty_like(x, dtype=_CODE_DTYPE[out_dtype])
 
 
-def _weight_quant_dev(w: torch.Tensor, block_size: int):
+def _weight_quant_dev(w: torch.Tensor, block_size: int, scale_fmt: int):
     m, n = w.size()
     y = torch.empty_like(w, dtype=FP8)
     s = w.new_empty(-(-m // block_size), -(-n // block_size), dtype=torch.float32)
     with torch.cuda.device(w.device):
         rc = _lib.lib.dsv3_weight_quant(w.data_ptr(), dtype_code(w.dtype), y.data_ptr(), s.data_ptr(), m, n,
-                                        block_size, _stream(w))
+                                        block_size, scale_fmt, _stream(w))
     _lib.check(rc, "dsv3_weight_quant")
     return y, s
 
 
-def _weight_quant_meta(w, block_size):
+def _weight_quant_meta(w, block_size, scale_fmt):
     m, n = w.size()
     return torch.empty_like(w, dtype=FP8), w.new_empty(-(-m // block_size), -(-n // block_size), dtype=torch.float32)
 

@@ -11,14 +11,15 @@ correctly rounded, so on a GPU its scales can differ from the kernel's in the la
 """
 from __future__ import annotations
 
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 
 FP8 = torch.float8_e4m3fn
 
 
-def block_quant_weight(w: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
+def block_quant_weight(w: torch.Tensor, block_size: int = 128,
+                       scale_fmt: Optional[str] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per ``block_size`` x ``block_size`` tile: ``scale = max(amax, 1e-4) / 448`` and
     ``w8 = e4m3(w / scale)``.  Ragged edge tiles are zero-padded before the amax
     (README_WEIGHTS.md:89) and cropped afterwards.  Returns ``(w8 [m,n], scale
@@ -32,14 +33,20 @@ def block_quant_weight(w: torch.Tensor, block_size: int = 128) -> Tuple[torch.Te
     tiles = wf.view(mb, block_size, nb, block_size)
     amax = tiles.abs().amax(dim=(1, 3)).clamp_min(1e-4)
     scale = amax / 448.0
+    if scale_fmt == "ue8m0":                  # round up to a power of two (inference/kernel.py:29-31)
+        bits = scale.view(torch.int32)          # next power of two, on the bits: exponent + (mantissa != 0)
+        scale = (((bits >> 23) + ((bits & 0x7FFFFF) != 0).int()) << 23).view(torch.float32)
     w8 = (tiles / scale[:, None, :, None]).reshape(mb * block_size, nb * block_size)[:m, :n]
     return w8.contiguous().to(FP8), scale
 
 
-def weight_quant(w: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
+def weight_quant(w: torch.Tensor, block_size: int = 128,
+                 scale_fmt: Optional[str] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """``block_quant_weight`` on the device: one pass over ``w`` (2-D, contiguous, on the GPU) by the HIP kernel.
-    Returns ``(w8 [m,n] e4m3fn, scale [ceil(m/128), ceil(n/128)] fp32)``."""
-    from . import ops  # noqa: F401  (registers torch.ops.dsv3fp8)
+    Returns ``(w8 [m,n] e4m3fn, scale [ceil(m/128), ceil(n/128)] fp32)``; ``scale_fmt="ue8m0"`` rounds every
+    scale up to a power of two, as ``act_quant`` does."""
+    from . import _lib, ops  # noqa: F401  (registers torch.ops.dsv3fp8)
     assert w.is_contiguous(), 'Input tensor must be contiguous'
     assert w.dim() == 2, 'Input tensor must have 2 dimensions'
-    return torch.ops.dsv3fp8.weight_quant(w, block_size)
+    fmt = _lib.SCALE_FMT_UE8M0 if scale_fmt == "ue8m0" else _lib.SCALE_FMT_NONE
+    return torch.ops.dsv3fp8.weight_quant(w, block_size, fmt)

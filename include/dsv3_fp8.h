@@ -107,11 +107,14 @@ int dsv3_weight_dequant(const void* x, const float* s, void* y, int y_dtype,
  * tensor shape inference/model.py:184-187).  The reference ships only the dequantising direction; the rule here is
  * the one its activation quantiser uses on 1 x 128 blocks (inference/kernel.py:23-35), applied to the square block:
  *     s[i,j] = max(amax(|w| over block i,j), 1e-4) / 448;   y = e4m3( w / s[i / 128, j / 128] )   (RNE)
+ * With scale_fmt DSV3_SCALE_FMT_UE8M0 the scale is rounded up to a power of two before the division, as act_quant
+ * does for activations (inference/kernel.py:29-31): the block-scale format of checkpoints made for
+ * inference/configs/config_v3.1.json:22, and what dsv3_fp8_gemm_pow2 requires of its weight.
  * w: [m,n] of w_dtype, y: [m,n] fp8 bytes, s: [ceil(m/128), ceil(n/128)] binary32.  block_size must be 128.
  * Any m, n >= 0; n % 8 == 0 with 16-byte aligned w and 8-byte aligned y takes the vectorised kernel.
  */
 int dsv3_weight_quant(const void* w, int w_dtype, void* y, float* s,
-                      int64_t m, int64_t n, int block_size, void* stream);
+                      int64_t m, int64_t n, int block_size, int scale_fmt, void* stream);
 
 /*
  * fp8_gemm (inference/kernel.py:145-172):

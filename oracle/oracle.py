@@ -104,7 +104,8 @@ def fp8_gemm(a, a_s, b, b_s, out_dtype: torch.dtype = torch.bfloat16) -> torch.T
     return fp8_gemm_f32(a, a_s, b, b_s).to(out_dtype)
 
 
-def block_quant_weight(w: torch.Tensor, block_size: int = BLOCK) -> Tuple[torch.Tensor, torch.Tensor]:
+def block_quant_weight(w: torch.Tensor, block_size: int = BLOCK,
+                       scale_fmt: Optional[str] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """README_WEIGHTS.md:83-92: per 128x128 block (ragged edge blocks are
     zero-padded, which leaves their amax unchanged) scale = amax / 448 and
     w8 = e4m3(w / scale); the stored scale is the dequantisation multiplier
@@ -117,6 +118,8 @@ def block_quant_weight(w: torch.Tensor, block_size: int = BLOCK) -> Tuple[torch.
     amax = blocks.abs().amax(dim=(1, 3))
     amax = torch.maximum(amax, torch.tensor(1e-4, dtype=torch.float32))
     s = amax / 448.0
+    if scale_fmt == "ue8m0":                  # kernel.py:29-31 applied to the block scale
+        s = ue8m0_round_up(s)
     w8 = (blocks / s[:, None, :, None]).view(mb * block_size, nb * block_size)[:m, :n].contiguous().to(FP8)
     return w8, s
 

@@ -64,15 +64,16 @@ def test_weight_dequant_validation(L):
 
 def test_weight_quant_validation(L):
     f = L.lib.dsv3_weight_quant
-    assert f(None, L.BF16, A16, A16, 128, 128, 128, None) == 1
-    assert f(A16, L.BF16, None, A16, 128, 128, 128, None) == 1
-    assert f(A16, L.BF16, A16, None, 128, 128, 128, None) == 1
-    assert f(A16, L.BF16, A16, A16, 128, -1, 128, None) == 2
-    assert f(A16, L.BF16, A16, A16, 128, 128, 64, None) == 3            # only 128 x 128 blocks exist on disk
-    assert f(A16, 7, A16, A16, 128, 128, 128, None) == 5
-    assert f(A16 + 1, L.BF16, A16, A16, 128, 128, 128, None) == 4
-    assert f(A16, L.BF16, A16, A16 + 2, 128, 128, 128, None) == 4
-    assert f(None, L.BF16, None, None, 0, 128, 128, None) == 0
+    assert f(None, L.BF16, A16, A16, 128, 128, 128, 0, None) == 1
+    assert f(A16, L.BF16, None, A16, 128, 128, 128, 0, None) == 1
+    assert f(A16, L.BF16, A16, None, 128, 128, 128, 0, None) == 1
+    assert f(A16, L.BF16, A16, A16, 128, -1, 128, 0, None) == 2
+    assert f(A16, L.BF16, A16, A16, 128, 128, 64, 0, None) == 3         # only 128 x 128 blocks exist on disk
+    assert f(A16, L.BF16, A16, A16, 128, 128, 128, 5, None) == 5        # unknown scale format
+    assert f(A16, 7, A16, A16, 128, 128, 128, 0, None) == 5
+    assert f(A16 + 1, L.BF16, A16, A16, 128, 128, 128, 0, None) == 4
+    assert f(A16, L.BF16, A16, A16 + 2, 128, 128, 128, 0, None) == 4
+    assert f(None, L.BF16, None, None, 0, 128, 128, 0, None) == 0
 
 
 @pytest.mark.parametrize("entry", ["dsv3_fp8_gemm", "dsv3_fp8_gemm_pow2"])

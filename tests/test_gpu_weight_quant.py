@@ -17,9 +17,9 @@ def K():
     return dsv3fp8
 
 
-def _check(K, w):
-    ref8, refs = oracle.block_quant_weight(w)
-    q8, qs = K.weight_quant(w.cuda())
+def _check(K, w, fmt=None):
+    ref8, refs = oracle.block_quant_weight(w, scale_fmt=fmt)
+    q8, qs = K.weight_quant(w.cuda(), scale_fmt=fmt)
     assert q8.dtype == FP8 and qs.dtype == torch.float32
     assert q8.shape == ref8.shape and qs.shape == refs.shape
     assert torch.equal(qs.cpu(), refs)
@@ -114,3 +114,41 @@ def test_full_size_round_trip(K):
         ref8, refs = oracle.block_quant_weight(w[r0:r0 + 128].cpu())
         assert torch.equal(qs[r0 // 128].cpu(), refs[0])
         assert torch.equal(q8[r0:r0 + 128].cpu().view(torch.uint8), ref8.view(torch.uint8))
+
+
+@pytest.mark.parametrize("shape,dtype", [((256, 512), torch.bfloat16), ((300, 520), torch.bfloat16),
+                                         ((200, 301), torch.float32), ((130, 272), torch.float16)])
+def test_power_of_two_scales(K, shape, dtype):
+    """scale_fmt "ue8m0": the scales are rounded up to powers of two before the division (kernel.py:29-31 applied to
+    the block scale); bytes and scales equal the oracle's, and the result feeds fp8_gemm_pow2."""
+    g = torch.Generator().manual_seed(shape[1])
+    w = (torch.randn(*shape, generator=g) * 0.04).to(dtype)
+    q8, qs = _check(K, w, "ue8m0")
+    assert bool(((qs.view(torch.int32) & 0x7FFFFF) == 0).all())
+    assert bool((q8.float().abs().amax() <= 448).item())
+    # a power of two is kept: blocks whose amax / 448 is already 2^e
+    w2 = torch.zeros(128, 256)
+    w2[3, 5], w2[100, 200] = 448 * 2.0 ** -9, -448 * 2.0 ** -3
+    w2[0, 0], w2[0, 130] = 2.0 ** -9, 2.0 ** -3
+    p8, ps = _check(K, w2.to(dtype), "ue8m0")
+    assert ps.flatten().tolist() == [2.0 ** -9, 2.0 ** -3]
+    assert p8.cpu().float()[0, 0] == 1 and p8.cpu().float()[100, 200] == -448
+
+
+def test_quantise_then_multiply_with_power_of_two_scales(K):
+    """weight_quant(ue8m0) -> act_quant(ue8m0) -> fp8_gemm_pow2 on the device against the oracle's chain."""
+    g = torch.Generator().manual_seed(9)
+    w = (torch.randn(640, 1024, generator=g) * 0.03).bfloat16()
+    x = torch.randn(300, 1024, generator=g).bfloat16()
+    w8, ws = K.weight_quant(w.cuda(), scale_fmt="ue8m0")
+    a, a_s = K.act_quant(x.cuda(), 128, "ue8m0")
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float32)
+    try:
+        c = K.fp8_gemm_pow2(a, a_s, w8, ws)
+    finally:
+        torch.set_default_dtype(old)
+    r8, rs = oracle.block_quant_weight(w, scale_fmt="ue8m0")
+    ra, ras = oracle.act_quant(x, 128, "ue8m0")
+    ref = oracle.fp8_gemm_f32(ra, ras, r8, rs)
+    assert (c.cpu() - ref).abs().max().item() <= 1e-2 * ref.pow(2).mean().sqrt().item()
