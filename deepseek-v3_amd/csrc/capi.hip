@@ -151,11 +151,11 @@ int dsv3_moe_route(const int64_t* indices, const void* weights, int w_dtype, int
                             tile_group, tile_row0, tile_rows, (hipStream_t)stream);
 }
 
-int dsv3_fp8_gemm_grouped(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
-                          const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
-                          void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
-                          const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
-                          int64_t num_tiles, void* stream) {
+static int fp8_gemm_grouped_checked(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
+                                   const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
+                                   void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                                   const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
+                                   int64_t num_tiles, void* stream, bool pow2) {
     if (!valid_dtype(c_dtype)) return DSV3_ERR_BAD_DTYPE;
     if (m < 0 || n < 0 || k < 0 || a_num_rows < 0 || num_tiles < 0 || b_group_stride < 0 || bs_group_stride < 0)
         return DSV3_ERR_BAD_SHAPE;
@@ -168,11 +168,35 @@ int dsv3_fp8_gemm_grouped(const void* a, const float* a_s, const int32_t* a_rows
         return DSV3_ERR_MISALIGNED;
     if (!grouped_supported(a_num_rows, n, k)) return DSV3_ERR_BAD_SHAPE;
     hipStream_t st = (hipStream_t)stream;
+#define DSV3_GROUPED(CD)                                                                                              \
+    (pow2 ? launch_grouped<CD, true>(a, a_s, a_rows, b, b_s, c, m, n, k, num_tiles, tile_group, tile_row0, tile_rows,  \
+                                     b_group_stride, bs_group_stride, st)                                              \
+          : launch_grouped<CD, false>(a, a_s, a_rows, b, b_s, c, m, n, k, num_tiles, tile_group, tile_row0, tile_rows, \
+                                      b_group_stride, bs_group_stride, st))
     switch (c_dtype) {
-        case DSV3_BF16: return launch_grouped<DSV3_BF16>(a, a_s, a_rows, b, b_s, c, m, n, k, num_tiles, tile_group, tile_row0, tile_rows, b_group_stride, bs_group_stride, st);
-        case DSV3_F16:  return launch_grouped<DSV3_F16>(a, a_s, a_rows, b, b_s, c, m, n, k, num_tiles, tile_group, tile_row0, tile_rows, b_group_stride, bs_group_stride, st);
-        default:        return launch_grouped<DSV3_F32>(a, a_s, a_rows, b, b_s, c, m, n, k, num_tiles, tile_group, tile_row0, tile_rows, b_group_stride, bs_group_stride, st);
+        case DSV3_BF16: return DSV3_GROUPED(DSV3_BF16);
+        case DSV3_F16:  return DSV3_GROUPED(DSV3_F16);
+        default:        return DSV3_GROUPED(DSV3_F32);
     }
+#undef DSV3_GROUPED
+}
+
+int dsv3_fp8_gemm_grouped(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
+                          const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
+                          void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                          const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
+                          int64_t num_tiles, void* stream) {
+    return fp8_gemm_grouped_checked(a, a_s, a_rows, a_num_rows, b, b_s, b_group_stride, bs_group_stride, c, c_dtype,
+                                    m, n, k, tile_group, tile_row0, tile_rows, num_tiles, stream, false);
+}
+
+int dsv3_fp8_gemm_grouped_pow2(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
+                               const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
+                               void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                               const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
+                               int64_t num_tiles, void* stream) {
+    return fp8_gemm_grouped_checked(a, a_s, a_rows, a_num_rows, b, b_s, b_group_stride, bs_group_stride, c, c_dtype,
+                                    m, n, k, tile_group, tile_row0, tile_rows, num_tiles, stream, true);
 }
 
 int dsv3_swiglu_quant(const void* h, int h_dtype, void* y, float* s, int64_t rows, int64_t inter,

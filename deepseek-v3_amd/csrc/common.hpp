@@ -91,7 +91,7 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
                    int64_t m, int64_t n, int64_t k, void* ws, hipStream_t stream);
 int grouped_tile_rows();
 bool grouped_supported(int64_t a_num_rows, int64_t n, int64_t k);
-template <int CD>
+template <int CD, bool P2 = false>
 int launch_grouped(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
                    const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream);

@@ -575,7 +575,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 // straight from HBM, and a second block of prefetch is what hides that), one with fewer the 128-row
 // configuration with three stages of both.  The choice is uniform over the workgroup and needs no host knowledge of
 // the group sizes: a layer with a few rows per expert and one with hundreds go through the same launch.
-template <int CD>
+template <int CD, bool P2 = false>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -585,11 +585,11 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
     if (tm >= tiles_m) return;
     const int rows = g.tile_rows[tm];
     if (rows > 192)
-        prefill_tile<CD, true, 256, 2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+        prefill_tile<CD, true, 256, 2, 2, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
     else if (rows > 128)
-        prefill_tile<CD, true, 192, 2, 3>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+        prefill_tile<CD, true, 192, 2, 3, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
     else
-        prefill_tile<CD, true, 128, 3>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+        prefill_tile<CD, true, 128, 3, 3, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
 }
 
 // Dense GEMM whose last column tiles run as 128-row tiles: the first tiles_m * tn_tall workgroups compute 256-row
@@ -828,7 +828,7 @@ bool grouped_supported(int64_t a_num_rows, int64_t n, int64_t k) {
     return k >= 128 && k % 128 == 0 && n >= 1 && a_num_rows * k < (1ll << 32) && n * k < (1ll << 32);
 }
 
-template <int CD>
+template <int CD, bool P2>
 int launch_grouped(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
                    const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream) {
@@ -846,7 +846,7 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
     const int64_t tn = (n + BN - 1) / BN;
     if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (num_tiles * tn == 0) return DSV3_OK;
-    auto kern = fp8_gemm_grouped_kernel<CD>;
+    auto kern = fp8_gemm_grouped_kernel<CD, P2>;
     static bool granted[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
@@ -865,7 +865,9 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
 #define DSV3_INST(CD) \
     template int launch_prefill<CD, false>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, void*, hipStream_t); \
     template int launch_prefill<CD, true>(const void*, const float*, const void*, const float*, void*, int64_t, int64_t, int64_t, void*, hipStream_t); \
-    template int launch_grouped<CD>(const void*, const float*, const int*, const void*, const float*, void*, int64_t, int64_t, int64_t, \
+    template int launch_grouped<CD, false>(const void*, const float*, const int*, const void*, const float*, void*, int64_t, int64_t, int64_t, \
+                                    int64_t, const int*, const int*, const int*, int64_t, int64_t, hipStream_t);                     \
+    template int launch_grouped<CD, true>(const void*, const float*, const int*, const void*, const float*, void*, int64_t, int64_t, int64_t, \
                                     int64_t, const int*, const int*, const int*, int64_t, int64_t, hipStream_t);
 DSV3_INST(DSV3_BF16)
 DSV3_INST(DSV3_F16)

@@ -62,18 +62,22 @@ class ModelArgs:
     mscale: float = 1.
 
 
-def _scales_are_powers_of_two(weight: torch.Tensor) -> bool:
+def _scales_are_powers_of_two(weight: torch.Tensor, scale: Optional[torch.Tensor] = None) -> bool:
     """Whether every block scale of an fp8 weight is a power of two (checkpoints made for ``scale_fmt = "ue8m0"``,
     inference/configs/config_v3.1.json:22, store them that way).  Looked at once per version of the scale tensor
     (one device-to-host read), never while a graph is being captured."""
-    scale = weight.scale
+    scale = weight.scale if scale is None else scale
+    try:
+        version = scale._version
+    except RuntimeError:            # a tensor made under inference_mode has no version counter: looked at once
+        version = -1
     cached = getattr(weight, "_dsv3_pow2", None)
-    if cached is not None and cached[0] == scale._version:
+    if cached is not None and cached[0] == version:
         return cached[1]
     if torch.cuda.is_current_stream_capturing():
         return False
     flag = bool(((scale.detach().view(torch.int32) & 0x7FFFFF) == 0).all().item()) and bool((scale > 0).all().item())
-    weight._dsv3_pow2 = (scale._version, flag)
+    weight._dsv3_pow2 = (version, flag)
     return flag
 
 
@@ -534,9 +538,14 @@ class MoE(nn.Module):
         fmt = ops._lib.SCALE_FMT_UE8M0 if Linear.scale_fmt == "ue8m0" else ops._lib.SCALE_FMT_NONE
         code = ops.dtype_code(torch.get_default_dtype())
         xq, xs = act_quant(x, block_size, Linear.scale_fmt)           # quantised once: 1x128 blocks are per token
-        h = torch.ops.dsv3fp8.fp8_gemm_grouped(xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, code)
+        # power-of-two activation scales on experts whose block scales are powers of two as well: the scales go
+        # into the matrix instruction (the whole stacked buffers are looked at, once per version of their contents)
+        pow2 = (Linear.scale_fmt == "ue8m0" and _scales_are_powers_of_two(self._stacked[0], self._stacked[1])
+                and _scales_are_powers_of_two(self._stacked[2], self._stacked[3]))
+        gemm = torch.ops.dsv3fp8.fp8_gemm_grouped_pow2 if pow2 else torch.ops.dsv3fp8.fp8_gemm_grouped
+        h = gemm(xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, code)
         gq, gs = torch.ops.dsv3fp8.swiglu_quant(h, block_size, fmt)
-        out = torch.ops.dsv3fp8.fp8_gemm_grouped(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code)
+        out = gemm(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code)
         z = None if fold else self.shared_experts(x).contiguous()
         return torch.ops.dsv3fp8.moe_combine(out, rows, w_sorted, z)
 

@@ -30,6 +30,8 @@ _libdef.define("group_tiles(Tensor counts, int max_tiles) -> (Tensor, Tensor, Te
 _libdef.define("moe_route(Tensor indices, Tensor weights, int experts, bool shared_group) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)")
 _libdef.define("fp8_gemm_grouped(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b, Tensor b_s, int rows, "
                "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int out_dtype) -> Tensor")
+_libdef.define("fp8_gemm_grouped_pow2(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b, Tensor b_s, int rows, "
+               "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int out_dtype) -> Tensor")
 _libdef.define("swiglu_quant(Tensor h, int block_size, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("moe_combine(Tensor expert_out, Tensor rows, Tensor weights, Tensor? shared) -> Tensor")
 _libdef.define("gate_route(Tensor logits, Tensor? bias, int topk, int n_groups, int topk_groups, int score_func, "
@@ -212,7 +214,8 @@ def _moe_route_meta(indices, weights, experts, shared_group):
             i32(max_tiles))
 
 
-def _fp8_gemm_grouped_dev(a, a_s, a_rows, b, b_s, rows: int, tile_group, tile_row0, tile_rows, out_dtype: int):
+def _fp8_gemm_grouped_dev(a, a_s, a_rows, b, b_s, rows: int, tile_group, tile_row0, tile_rows, out_dtype: int,
+                          entry: str = "dsv3_fp8_gemm_grouped"):
     # a: [A, k] fp8; b: [groups, n, k] fp8; b_s: [groups, ceil(n/128), k/128]; result [rows, n]
     assert a.dim() == 2 and b.dim() == 3 and b_s.dim() == 3 and a.is_contiguous() and b.is_contiguous()
     assert a_s.is_contiguous() and b_s.is_contiguous() and b.size(0) == b_s.size(0)
@@ -224,13 +227,18 @@ def _fp8_gemm_grouped_dev(a, a_s, a_rows, b, b_s, rows: int, tile_group, tile_ro
     assert b.size(2) == k
     c = a.new_empty(rows, n, dtype=_CODE_DTYPE[out_dtype])
     with torch.cuda.device(a.device):
-        rc = _lib.lib.dsv3_fp8_gemm_grouped(
+        rc = getattr(_lib.lib, entry)(
             a.data_ptr(), a_s.data_ptr(), a_rows.data_ptr() if a_rows is not None else None, a.size(0),
             b.data_ptr(), b_s.data_ptr(), b.stride(0), b_s.stride(0),
             c.data_ptr(), out_dtype, rows, n, k,
             tile_group.data_ptr(), tile_row0.data_ptr(), tile_rows.data_ptr(), tile_group.numel(), _stream(a))
-    _lib.check(rc, "dsv3_fp8_gemm_grouped")
+    _lib.check(rc, entry)
     return c
+
+
+def _fp8_gemm_grouped_pow2_dev(a, a_s, a_rows, b, b_s, rows: int, tile_group, tile_row0, tile_rows, out_dtype: int):
+    return _fp8_gemm_grouped_dev(a, a_s, a_rows, b, b_s, rows, tile_group, tile_row0, tile_rows, out_dtype,
+                                 "dsv3_fp8_gemm_grouped_pow2")
 
 
 def _fp8_gemm_grouped_meta(a, a_s, a_rows, b, b_s, rows, tile_group, tile_row0, tile_rows, out_dtype):
@@ -323,6 +331,7 @@ for _name, _dev, _meta in (("wkv_b_absorb", _wkv_b_absorb_dev, _wkv_b_absorb_met
                            ("group_tiles", _group_tiles_dev, _group_tiles_meta),
                            ("moe_route", _moe_route_dev, _moe_route_meta),
                            ("fp8_gemm_grouped", _fp8_gemm_grouped_dev, _fp8_gemm_grouped_meta),
+                           ("fp8_gemm_grouped_pow2", _fp8_gemm_grouped_pow2_dev, _fp8_gemm_grouped_meta),
                            ("swiglu_quant", _swiglu_quant_dev, _swiglu_quant_meta),
                            ("moe_combine", _moe_combine_dev, _moe_combine_meta)):
     _libimpl.impl(_name, _dev, "CUDA")

@@ -222,6 +222,15 @@ int dsv3_fp8_gemm_grouped(const void* a, const float* a_s, const int32_t* a_rows
                           const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
                           int64_t num_tiles, void* stream);
 
+/* dsv3_fp8_gemm_grouped for scales that are all powers of two (see dsv3_fp8_gemm_pow2: the caller's guarantee for
+ * every element of a_s and b_s).  The tile kernel then passes the block scales to the matrix instruction; launches
+ * of few rows take the same weight-streaming kernel as dsv3_fp8_gemm_grouped. */
+int dsv3_fp8_gemm_grouped_pow2(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
+                               const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
+                               void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                               const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
+                               int64_t num_tiles, void* stream);
+
 /*
  * silu(h1) * h3 followed by act_quant, in one pass (inference/model.py:633 feeding the act_quant of w2's
  * linear(), inference/model.py:159, inference/kernel.py:23-35):

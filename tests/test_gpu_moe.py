@@ -124,6 +124,34 @@ def test_fp8_gemm_grouped_seeded_tables(K):
             row += c
 
 
+@pytest.mark.parametrize("counts,n,k", [([5, 0, 300, 256, 1], 384, 512), ([145, 177, 200, 241, 17], 512, 384),
+                                        ([3, 2, 9], 256, 256)])
+def test_fp8_gemm_grouped_power_of_two_scales(K, counts, n, k):
+    """Scales that are powers of two on both sides: the grouped tile kernel hands them to the matrix instruction
+    (every tile configuration), a small launch takes the weight-streaming kernel as before."""
+    from dsv3fp8 import ops
+    g = torch.Generator().manual_seed(21)
+    rows = sum(counts)
+    x = torch.randn(rows, k, generator=g).bfloat16()
+    xq, xs = oracle.act_quant(x, 128, "ue8m0")
+    w = [oracle.block_quant_weight((torch.randn(n, k, generator=g) * 0.05).bfloat16(), scale_fmt="ue8m0") for _ in counts]
+    R, tg, t0, tr = _tables(counts, rows // ops.grouped_tile_rows() + len(counts))
+    b = torch.stack([wi[0].view(torch.uint8) for wi in w]).view(FP8).cuda()
+    b_s = torch.stack([wi[1] for wi in w]).cuda()
+    assert bool(((b_s.view(torch.int32) & 0x7FFFFF) == 0).all())
+    args = (xq.cuda(), xs.cuda(), None, b, b_s, rows, tg, t0, tr, ops.dtype_code(torch.float32))
+    out = torch.ops.dsv3fp8.fp8_gemm_grouped_pow2(*args).cpu()
+    gen = torch.ops.dsv3fp8.fp8_gemm_grouped(*args).cpu()
+    row = 0
+    for gi, c in enumerate(counts):
+        if c:
+            ref = oracle.fp8_gemm_f32(xq[row:row + c], xs[row:row + c], w[gi][0], w[gi][1])
+            rms = ref.pow(2).mean().sqrt().item()
+            assert (out[row:row + c] - ref).abs().max().item() <= 1e-2 * rms
+            assert (out[row:row + c] - gen[row:row + c]).abs().max().item() <= 1e-4 * rms
+        row += c
+
+
 @pytest.mark.parametrize("fmt", [None, "ue8m0"])
 def test_swiglu_quant(K, fmt):
     g = torch.Generator().manual_seed(3)
@@ -228,6 +256,56 @@ def test_moe_grouped_matches_expert_loop_and_oracle(K, tokens):
     finally:
         M.MoE.grouped = True
         M.gemm_impl, M.Linear.dtype = old[0], old[2]
+        torch.set_default_dtype(old[1])
+
+
+def test_moe_layer_with_power_of_two_scales(K, monkeypatch):
+    """scale_fmt "ue8m0" on experts whose block scales are powers of two: the grouped GEMMs take the entry point that
+    hands the scales to the matrix instruction, and the layer still agrees with the oracle's expert loop."""
+    from dsv3fp8 import model as M
+    old = (M.gemm_impl, torch.get_default_dtype(), M.Linear.dtype, M.Linear.scale_fmt)
+    torch.set_default_dtype(torch.bfloat16)
+    M.Linear.dtype, M.gemm_impl, M.Linear.scale_fmt = FP8, "fp8", "ue8m0"
+    try:
+        args = M.ModelArgs(dim=256, inter_dim=512, moe_inter_dim=128, n_routed_experts=8, n_shared_experts=1,
+                           n_activated_experts=2, n_expert_groups=2, n_limited_groups=1, route_scale=2.5)
+        with torch.device("cuda"):
+            moe = M.MoE(args)
+        g = torch.Generator().manual_seed(6)
+        with torch.no_grad():
+            moe.gate.weight.copy_((torch.randn(8, 256, generator=g) * 0.05).bfloat16().cuda())
+
+        def fill(lin, seed, fmt):
+            gg = torch.Generator().manual_seed(seed)
+            w8, s = oracle.block_quant_weight((torch.randn(lin.out_features, lin.in_features, generator=gg) * 0.05).bfloat16(),
+                                              scale_fmt=fmt)
+            with torch.no_grad():
+                lin.weight.copy_(w8.cuda()); lin.scale.copy_(s.cuda())
+            return w8, s
+        experts = []
+        for i, ex in enumerate(moe.experts):
+            w1, s1 = fill(ex.w1, 10 + 3 * i, "ue8m0"); w2, s2 = fill(ex.w2, 11 + 3 * i, "ue8m0"); w3, s3 = fill(ex.w3, 12 + 3 * i, "ue8m0")
+            experts.append((w1, s1, w2, s2, w3, s3))
+        sh = moe.shared_experts
+        shared = (*fill(sh.w1, 90, "ue8m0"), *fill(sh.w2, 91, "ue8m0"), *fill(sh.w3, 92, "ue8m0"))
+        calls = []
+        real = torch.ops.dsv3fp8.fp8_gemm_grouped_pow2
+
+        class Spy:
+            def __call__(self, *a):
+                calls.append(a[5])
+                return real(*a)
+        monkeypatch.setattr(M.torch.ops.dsv3fp8, "fp8_gemm_grouped_pow2", Spy(), raising=False)
+        x = torch.randn(600, 256, generator=g).bfloat16()
+        with torch.inference_mode():
+            y = moe(x.cuda())
+            wts, idx = moe.gate(x.cuda())
+        assert calls == [1200, 1200]                      # 600 tokens x 2 experts, both grouped GEMMs
+        ref = oracle.moe(x, wts.cpu(), idx.cpu(), experts, shared, scale_fmt="ue8m0")
+        rms = ref.float().pow(2).mean().sqrt().item()
+        assert (y.float().cpu() - ref.float()).abs().max().item() <= 5e-2 * rms + 2 ** -8 * ref.abs().max().item()
+    finally:
+        M.gemm_impl, M.Linear.dtype, M.Linear.scale_fmt = old[0], old[2], old[3]
         torch.set_default_dtype(old[1])
 
 
