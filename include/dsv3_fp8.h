@@ -10,6 +10,11 @@
  *   dsv3_weight_dequant  <- weight_dequant  (inference/kernel.py:89-110, kernel :60-86)
  *   dsv3_fp8_gemm        <- fp8_gemm        (inference/kernel.py:175-196, kernel :118-172)
  *
+ * Around them, each documented at its declaration: dsv3_linear_fp8 (the two calls of linear() as one launch for
+ * few rows), dsv3_fp8_gemm_pow2 / dsv3_fp8_gemm_grouped_pow2 (power-of-two scales), dsv3_weight_quant (the inverse
+ * of weight_dequant), the mixture-of-experts functions (dsv3_gate_route, dsv3_moe_route, dsv3_group_tiles,
+ * dsv3_fp8_gemm_grouped, dsv3_swiglu_quant, dsv3_moe_combine) and dsv3_wkv_b_absorb (attention).
+ *
  * Conventions
  *   - every pointer is a device pointer into memory the caller owns; the library
  *     never allocates, frees or keeps caller-visible memory;
