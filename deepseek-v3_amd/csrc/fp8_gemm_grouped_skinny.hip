@@ -8,8 +8,8 @@
 // One token activates 8 routed experts (+ the shared one): 9 groups of ONE row each, 44 MB of weights per group.
 // The tile kernel gives such a launch 9 x 16 workgroups -- half the chip -- and each of them is alone with a 1.8 MB
 // weight slab behind a two-block prefetch.  Here a workgroup owns 32 weight rows of one group (two 16-row MFMA
-// strips per wavefront) and its four wavefronts split the K range, so the same launch has 9 x 128 x 4 wavefronts
-// streaming with four K blocks of loads in flight each.
+// strips per wavefront) and its two to eight wavefronts split the K range, so the same launch has 9 x 128 x 4
+// wavefronts streaming with three K blocks of loads in flight each.
 //
 // Weights go straight from global memory into MFMA operand registers exactly as in the dense decode kernel
 // (fp8_gemm_skinny.hip: 8 rows x 128 contiguous bytes per load instruction, halves exchanged by DPP).  The
