@@ -99,6 +99,9 @@ int launch_grouped_skinny(const void* a, const float* a_s, const int* a_rows, co
                           int c_dtype, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group,
                           const int* tile_row0, const int* tile_rows, int64_t b_stride, int64_t bs_stride,
                           int64_t groups_hint, hipStream_t stream);
+bool skinny_single_supported(int64_t m, int64_t n, int64_t k);
+int launch_skinny_single(const void* a, const float* a_s, const void* b, const float* b_s, void* c, int c_dtype,
+                         int64_t m, int64_t n, int64_t k, hipStream_t stream);
 int launch_swiglu_quant(const void* h, void* y, float* s, int64_t rows, int64_t inter, int scale_fmt, hipStream_t st);
 int launch_moe_combine(const void* out, const int* rows, const void* w, const void* shared, void* y,
                        int64_t tokens, int topk, int64_t dim, hipStream_t st);

@@ -47,15 +47,16 @@ __global__ __launch_bounds__(kWaves * kWave) void fp8_gemm_grouped_skinny_kernel
         const uint8_t* __restrict__ a, const float* __restrict__ a_s, const int* __restrict__ a_rows,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s, void* __restrict__ c, int c_dtype,
         int N, int K, const int* __restrict__ tile_group, const int* __restrict__ tile_row0,
-        const int* __restrict__ tile_rows, int64_t b_stride, int64_t bs_stride) {
+        const int* __restrict__ tile_rows, int64_t b_stride, int64_t bs_stride, int single_rows) {
     // K blocks of loads in flight per wavefront: three keep the kernel at 128 registers or fewer, i.e. 16 resident
     // wavefronts per compute unit (four blocks in flight and 12 wavefronts measured slower)
     constexpr int NPF = kWaves <= 8 ? 3 : 2;
     __shared__ v4f red[kWaves * S * 64];
+    // without a tile table the launch is ONE group of single_rows rows: a dense GEMM with few rows
     const int slot = blockIdx.y;
-    const int grp = tile_group[slot];
+    const int grp = tile_group ? tile_group[slot] : 0;
     if (grp < 0) return;                                   // uniform over the workgroup
-    const int row0 = tile_row0[slot], rows = tile_rows[slot];
+    const int row0 = tile_group ? tile_row0[slot] : 0, rows = tile_group ? tile_rows[slot] : single_rows;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int fr = lane & 15, fq = lane >> 4;
@@ -163,6 +164,7 @@ int launch_grouped_skinny(const void* a, const float* a_s, const int* a_rows, co
                           const int* tile_row0, const int* tile_rows, int64_t b_stride, int64_t bs_stride,
                           int64_t groups_hint, hipStream_t stream) {
     using namespace gskinny;
+    const int single_rows = 0;
     const int64_t strips = (n + 16 * S - 1) / (16 * S);
     if (strips > 0x7fffffff || num_tiles > 65535) return DSV3_ERR_BAD_SHAPE;
     if (strips == 0 || num_tiles == 0) return DSV3_OK;
@@ -179,10 +181,36 @@ int launch_grouped_skinny(const void* a, const float* a_s, const int* a_rows, co
 #define DSV3_GS(W)                                                                                                     \
     hipLaunchKernelGGL(fp8_gemm_grouped_skinny_kernel<W>, dim3((unsigned)strips, (unsigned)num_tiles), dim3(W * kWave), \
                        0, stream, (const uint8_t*)a, a_s, a_rows, (const uint8_t*)b, b_s, c, c_dtype, (int)n, (int)k,  \
-                       tile_group, tile_row0, tile_rows, b_stride, bs_stride)
+                       tile_group, tile_row0, tile_rows, b_stride, bs_stride, single_rows)
     if (waves >= 16) DSV3_GS(16);
     else if (waves >= 8) DSV3_GS(8);
     else if (waves >= 4) DSV3_GS(4);
+    else DSV3_GS(2);
+#undef DSV3_GS
+    return launch_status();
+}
+
+// The same kernel as ONE group without a tile table: a dense fp8_gemm with m <= 16 rows on a weight large enough
+// that 32-row strips fill the chip.  No workspace and no second pass (the wavefronts of a workgroup split K).
+bool skinny_single_supported(int64_t m, int64_t n, int64_t k) {
+    return m >= 1 && m <= 16 && k >= 128 && k % 128 == 0 && n >= 1 && n * k < (1ll << 32) && m * k < (1ll << 32);
+}
+
+int launch_skinny_single(const void* a, const float* a_s, const void* b, const float* b_s, void* c, int c_dtype,
+                         int64_t m, int64_t n, int64_t k, hipStream_t stream) {
+    using namespace gskinny;
+    const int64_t strips = (n + 16 * S - 1) / (16 * S), kb = k / 128;
+    if (strips > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    // measured on 16384 -> 7168 (224 strips): 8 wavefronts 25.3 us, 4: 29.9, 16: 26.3
+    const int waves = kb < 32 ? 2 : ((strips * 4 < 2048 && kb >= 64) ? 8 : 4);
+    const int* none = nullptr;
+    const int single_rows = (int)m;
+#define DSV3_GS(W)                                                                                                     \
+    hipLaunchKernelGGL(fp8_gemm_grouped_skinny_kernel<W>, dim3((unsigned)strips, 1u), dim3(W * kWave), 0, stream,      \
+                       (const uint8_t*)a, a_s, none, (const uint8_t*)b, b_s, c, c_dtype, (int)n, (int)k, none, none,   \
+                       none, (int64_t)0, (int64_t)0, single_rows)
+    if (waves == 8) DSV3_GS(8);
+    else if (waves == 4) DSV3_GS(4);
     else DSV3_GS(2);
 #undef DSV3_GS
     return launch_status();

@@ -262,6 +262,14 @@ Plan make_plan(int64_t m, int64_t n, int64_t k) {
     return p;
 }
 
+// 3 to 16 rows on a weight of 96 MiB or more: the dense GEMM runs as one group of the grouped weight-streaming
+// kernel -- 32-row strips of such a weight fill the chip, one launch, no partial sums in memory (16384 -> 7168 at 4
+// rows 25.5 against 30.4 us; 7168 -> 36864 at 8 rows 51 against 70 us).  One and two rows stay with the M <= 16
+// kernel, which quantises bf16 activations itself for linear() there (26.5 us fused against 25.5 + 3.5 us).
+bool single_group_stream(int64_t m, int64_t n, int64_t k) {
+    return m >= 3 && m <= 16 && n * k >= (96ll << 20) && skinny_single_supported(m, n, k);
+}
+
 // DSV3_GEMM_FORCE=tile|prefill pins the large-M kernel choice (tuning / debugging aid).
 int forced_kernel() {
     static const int v = [] {
@@ -294,6 +302,8 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
         return launch_status();
     }
     const int force = forced_kernel();
+    if (force == 0 && single_group_stream(m, n, k))
+        return launch_skinny_single(a, a_s, b, b_s, c, CD, m, n, k, st);
     const bool to_prefill = force != 1 && to_large_m_kernel(m, n, k);
     const bool use_stream = force != 1 && !to_prefill && stream_supported(m, n, k);
     if (use_stream || (force != 1 && !to_prefill && skinny_supported(m, n, k))) {          // decode shapes: weight-streaming kernels
@@ -332,7 +342,7 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
 // small (16 rows x 16384: 51 us fused against 44 us in two launches; 8 rows: equal; fewer: 1 - 3 us saved).
 bool linear_fp8_supported(int64_t m, int64_t n, int64_t k) {
     return forced_kernel() != 1 && k % 128 == 0 && skinny_supported(m, n, k) && !to_large_m_kernel(m, n, k) &&
-           m * k <= 131072;
+           !(forced_kernel() == 0 && single_group_stream(m, n, k)) && m * k <= 131072;
 }
 
 int launch_linear_fp8(const void* x, const void* b, const float* b_s, void* c, int c_dtype, int64_t m, int64_t n,

@@ -208,7 +208,9 @@ def test_fused_linear_equals_act_quant_then_gemm(K, m, fmt):
     from dsv3fp8 import workloads, ops, _lib
     code_fmt = _lib.SCALE_FMT_UE8M0 if fmt == "ue8m0" else _lib.SCALE_FMT_NONE
     for name, (k, n) in workloads.DECODE_SHAPES.items():
-        assert ops.linear_fp8_fused(m, n, k) == (m * k <= 131072), name     # beyond that the op issues the two calls
+        # fused up to 131072 activation elements, except 3+ rows on weights of 96 MiB and more (those take two calls:
+        # the single-launch weight-streaming kernel for large weights has no quantising variant)
+        assert ops.linear_fp8_fused(m, n, k) == (m * k <= 131072 and not (m >= 3 and n * k >= 96 << 20)), name
         x = workloads.activations(m, k, seed=m + n % 7, outliers=True).cuda()
         w8, ws = workloads.weight(n, k, seed=3)
         w8, ws = w8.cuda(), ws.cuda()
