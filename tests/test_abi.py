@@ -229,7 +229,8 @@ def test_gate_route_validation(L):
 
 def test_linear_fp8_validation(L):
     f, fused = L.lib.dsv3_linear_fp8, L.lib.dsv3_linear_fp8_fused
-    assert fused(1, 1536, 7168) and fused(8, 7168, 16384) and not fused(16, 7168, 16384) and not fused(17, 1536, 7168)
+    assert fused(1, 1536, 7168) and fused(2, 7168, 16384) and not fused(16, 7168, 16384) and not fused(17, 1536, 7168)
+    assert fused(8, 24576, 1536) and not fused(8, 7168, 16384)   # 3+ rows on a weight of 96 MiB or more: two calls
     assert not fused(4096, 1536, 7168)
     assert not fused(4, 1536, 7000) and not fused(0, 8, 128)
     #     x    dtype   b    b_s  c    cdtype  m  n     k     block fmt ws    ws_bytes stream
