@@ -14,8 +14,9 @@
 namespace dsv3 {
 namespace {
 
-// Wavefront-wide reductions that leave the result in every lane: four DPP steps inside each row of 16 lanes
-// (no LDS traffic), then two cross-row exchanges.
+// Wavefront-wide reductions that leave the result in every lane: four DPP steps inside each row of 16 lanes, then
+// the four row results are read into scalar registers and combined -- no LDS traffic (a cross-row shuffle is an LDS
+// permute of ~100 cycles, and the selection below is a chain of two dozen such reductions).
 template <int CTRL> __device__ __forceinline__ int dpp_mov(int v) {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
 }
@@ -23,10 +24,10 @@ template <class Op> __device__ __forceinline__ int wave_reduce(int v, Op op) {
     v = op(v, dpp_mov<0xB1>(v));      // quad_perm [1,0,3,2]
     v = op(v, dpp_mov<0x4E>(v));      // quad_perm [2,3,0,1]
     v = op(v, dpp_mov<0x141>(v));     // row_half_mirror
-    v = op(v, dpp_mov<0x140>(v));     // row_mirror
-    v = op(v, __shfl_xor(v, 16, 64));
-    v = op(v, __shfl_xor(v, 32, 64));
-    return v;
+    v = op(v, dpp_mov<0x140>(v));     // row_mirror: every lane of a row holds the row's result
+    const int r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
+    const int r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
+    return op(op(r0, r1), op(r2, r3));
 }
 __device__ __forceinline__ float wave_max(float x) {
     return __builtin_bit_cast(float, wave_reduce(__builtin_bit_cast(int, x), [](int a, int b) {
