@@ -1,0 +1,206 @@
+"""HF-named checkpoint -> local names and model-parallel shards (counterpart of inference/convert.py): the name
+table (:11-30), the text rules (:56-60), the split of routed experts and of column / row parallel weights
+(:64-75), and what the reference leaves unchecked -- that a sliced FP8 weight keeps the scales of its own blocks."""
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from dsv3fp8 import convert
+from oracle import oracle
+
+
+def test_names_follow_the_module_tree_of_model_py():
+    cases = {
+        "model.embed_tokens.weight": ("embed.weight", 0),
+        "model.norm.weight": ("norm.weight", None),
+        "lm_head.weight": ("head.weight", 0),
+        "model.layers.3.input_layernorm.weight": ("layers.3.attn_norm.weight", None),
+        "model.layers.3.post_attention_layernorm.weight": ("layers.3.ffn_norm.weight", None),
+        "model.layers.3.self_attn.q_proj.weight": ("layers.3.attn.wq.weight", 0),
+        "model.layers.3.self_attn.q_a_proj.weight": ("layers.3.attn.wq_a.weight", None),
+        "model.layers.3.self_attn.q_a_proj.weight_scale_inv": ("layers.3.attn.wq_a.scale", None),
+        "model.layers.3.self_attn.q_a_layernorm.weight": ("layers.3.attn.q_norm.weight", None),
+        "model.layers.3.self_attn.q_b_proj.weight": ("layers.3.attn.wq_b.weight", 0),
+        "model.layers.3.self_attn.kv_a_proj_with_mqa.weight": ("layers.3.attn.wkv_a.weight", None),
+        "model.layers.3.self_attn.kv_a_layernorm.weight": ("layers.3.attn.kv_norm.weight", None),
+        "model.layers.3.self_attn.kv_b_proj.weight_scale_inv": ("layers.3.attn.wkv_b.scale", 0),
+        "model.layers.3.self_attn.o_proj.weight": ("layers.3.attn.wo.weight", 1),
+        "model.layers.3.self_attn.o_proj.weight_scale_inv": ("layers.3.attn.wo.scale", 1),
+        "model.layers.0.mlp.gate_proj.weight": ("layers.0.ffn.w1.weight", 0),
+        "model.layers.0.mlp.up_proj.weight": ("layers.0.ffn.w3.weight", 0),
+        "model.layers.0.mlp.down_proj.weight": ("layers.0.ffn.w2.weight", 1),
+        "model.layers.5.mlp.gate.weight": ("layers.5.ffn.gate.weight", None),
+        "model.layers.5.mlp.gate.e_score_correction_bias": ("layers.5.ffn.gate.bias", None),
+        "model.layers.5.mlp.experts.17.gate_proj.weight": ("layers.5.ffn.experts.17.w1.weight", 0),
+        "model.layers.5.mlp.experts.17.down_proj.weight_scale_inv": ("layers.5.ffn.experts.17.w2.scale", 1),
+        "model.layers.5.mlp.shared_experts.up_proj.weight": ("layers.5.ffn.shared_experts.w3.weight", 0),
+    }
+    for hf, want in cases.items():
+        assert convert.local_name(hf) == want, hf
+    with pytest.raises(KeyError, match="not found in mapping"):
+        convert.local_name("model.layers.0.self_attn.rotary_emb.inv_freq")
+
+
+def test_local_names_are_the_parameter_names_of_the_modules():
+    """A converted checkpoint must load with ``load_state_dict``: compare against the modules' own parameter names."""
+    from dsv3fp8 import model as M
+    args = M.ModelArgs(dim=256, inter_dim=512, moe_inter_dim=128, n_routed_experts=4, n_activated_experts=2,
+                       n_expert_groups=1, n_limited_groups=1, n_heads=2, q_lora_rank=128, kv_lora_rank=128,
+                       max_batch_size=1, max_seq_len=16)
+    old = M.Linear.dtype
+    M.Linear.dtype = torch.float8_e4m3fn
+    try:
+        with torch.device("meta"):
+            attn, mlp, moe = M.MLA(args), M.MLP(args.dim, args.inter_dim), M.MoE(args)
+    finally:
+        M.Linear.dtype = old
+    hf_attn = [f"model.layers.0.self_attn.{m}.{t}" for m in ("q_a_proj", "q_b_proj", "kv_a_proj_with_mqa", "kv_b_proj", "o_proj")
+               for t in ("weight", "weight_scale_inv")]
+    hf_attn += ["model.layers.0.self_attn.q_a_layernorm.weight", "model.layers.0.self_attn.kv_a_layernorm.weight"]
+    got = {convert.local_name(n)[0][len("layers.0.attn."):] for n in hf_attn}
+    assert got == {n for n, _ in attn.named_parameters()}
+    hf_mlp = [f"model.layers.0.mlp.{m}.{t}" for m in ("gate_proj", "up_proj", "down_proj") for t in ("weight", "weight_scale_inv")]
+    assert {convert.local_name(n)[0][len("layers.0.ffn."):] for n in hf_mlp} == {n for n, _ in mlp.named_parameters()}
+    hf_moe = ["model.layers.1.mlp.gate.weight"]
+    for owner in [f"experts.{e}" for e in range(4)] + ["shared_experts"]:
+        hf_moe += [f"model.layers.1.mlp.{owner}.{m}.{t}" for m in ("gate_proj", "up_proj", "down_proj")
+                   for t in ("weight", "weight_scale_inv")]
+    assert {convert.local_name(n)[0][len("layers.1.ffn."):] for n in hf_moe} == {n for n, _ in moe.named_parameters()}
+
+
+def test_shard_plan():
+    P = convert.shard_plan
+    # replicated, column parallel (rows), row parallel (columns)
+    assert P("layers.0.attn.wq_a.weight", (1536, 7168), None, 3, 8, 256) == (None, 0, 0)
+    assert P("layers.0.attn.wq_b.weight", (24576, 1536), 0, 3, 8, 256) == (0, 3 * 3072, 3072)
+    assert P("layers.0.attn.wo.weight", (7168, 16384), 1, 7, 8, 256) == (1, 7 * 2048, 2048)
+    assert P("layers.0.attn.wo.weight", (7168, 16384), 1, 0, 1, 256) == (None, 0, 0)
+    # routed experts go whole to their owner, shared experts are split like any other projection
+    assert P("layers.5.ffn.experts.17.w1.weight", (2048, 7168), 0, 0, 8, 256) == (None, 0, 0)        # experts 0..31
+    assert P("layers.5.ffn.experts.32.w1.weight", (2048, 7168), 0, 0, 8, 256) is None
+    assert P("layers.5.ffn.experts.32.w1.weight", (2048, 7168), 0, 1, 8, 256) == (None, 0, 0)
+    assert P("layers.5.ffn.shared_experts.w2.weight", (7168, 2048), 1, 2, 8, 256) == (1, 512, 256)
+    with pytest.raises(AssertionError, match="must be divisible"):
+        P("head.weight", (129280 + 1, 7168), 0, 0, 8, 256)
+    # scales: split like the weight, and only where the weight's slices are whole blocks
+    assert P("layers.0.attn.wo.scale", (56, 128), 1, 7, 8, 256, is_scale_of=(7168, 16384)) == (1, 112, 16)
+    with pytest.raises(ValueError, match="block boundary"):
+        P("layers.0.ffn.w2.scale", (4, 3), 1, 0, 2, 256, is_scale_of=(512, 320))      # 160 columns per rank
+    with pytest.raises(ValueError, match="block boundary"):
+        P("layers.0.ffn.w1.scale", (3, 4), 0, 0, 3, 256, is_scale_of=(384 - 3, 512))  # weight rows not divisible
+
+
+def test_every_671b_projection_splits_on_block_boundaries_up_to_16_ranks():
+    dim, inter, moe_inter, heads = 7168, 18432, 2048, 128
+    col = {"wq_b": (heads * 192, 1536), "wkv_b": (heads * 256, 512), "w1": (inter, dim), "w3": (inter, dim),
+           "shared.w1": (moe_inter, dim)}
+    row = {"wo": (dim, heads * 128), "w2": (dim, inter), "shared.w2": (dim, moe_inter)}
+    for mp in (1, 2, 4, 8, 16):
+        for name, shape in col.items():
+            scale = ((shape[0] + 127) // 128, (shape[1] + 127) // 128)
+            convert.shard_plan(f"layers.0.x.{name}.scale", scale, 0, mp - 1, mp, 256, is_scale_of=shape)
+        for name, shape in row.items():
+            scale = ((shape[0] + 127) // 128, (shape[1] + 127) // 128)
+            convert.shard_plan(f"layers.0.x.{name}.scale", scale, 1, mp - 1, mp, 256, is_scale_of=shape)
+
+
+def _synthetic_hf_checkpoint(path, g):
+    """Two layers with HF names in the FP8 on-disk format, spread over two files: layer 0 dense, layer 1 routed (4
+    experts + shared), plus layer 61 (dropped by the converter), embeddings, head and a tokenizer file."""
+    def q(rows, cols):
+        return oracle.block_quant_weight((torch.randn(rows, cols, generator=g) * 0.05).bfloat16())
+    def vec(n):
+        return torch.randn(n, generator=g).bfloat16()
+    dim, inter, moe_inter = 256, 512, 256
+    tensors, bf16 = {}, {}
+    def lin(name, rows, cols):
+        w, s = q(rows, cols)
+        tensors[f"{name}.weight"], tensors[f"{name}.weight_scale_inv"] = w, s
+    for l in (0, 1, 61):
+        p = f"model.layers.{l}"
+        tensors[f"{p}.input_layernorm.weight"] = vec(dim)
+        tensors[f"{p}.post_attention_layernorm.weight"] = vec(dim)
+        lin(f"{p}.self_attn.q_a_proj", 128, dim)
+        tensors[f"{p}.self_attn.q_a_layernorm.weight"] = vec(128)
+        lin(f"{p}.self_attn.q_b_proj", 512, 128)
+        lin(f"{p}.self_attn.kv_a_proj_with_mqa", 192, dim)
+        tensors[f"{p}.self_attn.kv_a_layernorm.weight"] = vec(128)
+        lin(f"{p}.self_attn.kv_b_proj", 512, 128)
+        lin(f"{p}.self_attn.o_proj", dim, 256)
+    for m, (r, c) in {"gate_proj": (inter, dim), "up_proj": (inter, dim), "down_proj": (dim, inter)}.items():
+        lin(f"model.layers.0.mlp.{m}", r, c)
+    tensors["model.layers.1.mlp.gate.weight"] = torch.randn(4, dim, generator=g).bfloat16()
+    tensors["model.layers.1.mlp.gate.e_score_correction_bias"] = torch.randn(4, generator=g)
+    for owner in [f"experts.{e}" for e in range(4)] + ["shared_experts"]:
+        for m, (r, c) in {"gate_proj": (moe_inter, dim), "up_proj": (moe_inter, dim), "down_proj": (dim, moe_inter)}.items():
+            lin(f"model.layers.1.mlp.{owner}.{m}", r, c)
+    tensors["model.embed_tokens.weight"] = torch.randn(64, dim, generator=g).bfloat16()
+    tensors["model.norm.weight"] = vec(dim)
+    tensors["lm_head.weight"] = torch.randn(64, dim, generator=g).bfloat16()
+    names = sorted(tensors)
+    half = len(names) // 2
+    # a weight and its scales may sit in different files (the released checkpoint does that too)
+    save_file({n: tensors[n] for n in names[:half]}, str(path / "model-00001-of-00002.safetensors"))
+    save_file({n: tensors[n] for n in names[half:]}, str(path / "model-00002-of-00002.safetensors"))
+    (path / "tokenizer.json").write_text("{}")
+    (path / "tokenizer_config.json").write_text("{}")
+    return tensors
+
+
+@pytest.mark.parametrize("mp", [1, 2])
+def test_convert_synthetic_checkpoint(tmp_path, mp):
+    src, dst = tmp_path / "hf", tmp_path / "local"
+    src.mkdir()
+    tensors = _synthetic_hf_checkpoint(src, torch.Generator().manual_seed(3))
+    convert.main(str(src), str(dst), n_experts=4, mp=mp)
+    assert (dst / "tokenizer.json").exists() and (dst / "tokenizer_config.json").exists()
+    ranks = [load_file(str(dst / f"model{r}-mp{mp}.safetensors")) for r in range(mp)]
+
+    def same(a, b):
+        assert a.dtype == b.dtype and a.shape == b.shape
+        nbytes = a.element_size()
+        view = {1: torch.uint8, 2: torch.int16, 4: torch.int32}[nbytes]
+        assert torch.equal(a.contiguous().view(view), b.contiguous().view(view))
+
+    expected_names = set()
+    for hf, t in tensors.items():
+        if "model.layers.61." in hf:
+            continue
+        name, dim = convert.local_name(hf)
+        expected_names.add(name)
+        e = convert.routed_expert(name)
+        for r in range(mp):
+            if e is not None:
+                owner = e // (4 // mp)
+                assert (name in ranks[r]) == (r == owner), (name, r)
+                if r == owner:
+                    same(ranks[r][name], t)
+            elif dim is None:
+                same(ranks[r][name], t)
+            else:
+                part = t.shape[dim] // mp
+                same(ranks[r][name], t.narrow(dim, r * part, part))
+    assert set().union(*[set(r) for r in ranks]) == expected_names
+    assert not any("layers.61" in n for r in ranks for n in r)
+
+    # a rank's (weight slice, scale slice) pair decodes to the same values as the slice of the decoded whole weight
+    for hf in ("model.layers.0.self_attn.q_b_proj", "model.layers.0.self_attn.o_proj", "model.layers.0.mlp.down_proj",
+               "model.layers.1.mlp.shared_experts.gate_proj"):
+        name, dim = convert.local_name(hf + ".weight")
+        whole = oracle.weight_dequant(tensors[hf + ".weight"], tensors[hf + ".weight_scale_inv"])
+        part = whole.shape[dim] // mp
+        for r in range(mp):
+            got = oracle.weight_dequant(ranks[r][name], ranks[r][name[: -len("weight")] + "scale"])
+            same(got, whole.narrow(dim, r * part, part))
+
+
+def test_convert_refuses_a_split_inside_a_scale_block(tmp_path):
+    src = tmp_path / "hf"
+    src.mkdir()
+    g = torch.Generator().manual_seed(4)
+    w, s = oracle.block_quant_weight((torch.randn(256, 320, generator=g) * 0.05).bfloat16())    # 160 columns per rank
+    save_file({"model.layers.0.mlp.down_proj.weight": w, "model.layers.0.mlp.down_proj.weight_scale_inv": s},
+              str(src / "model.safetensors"))
+    with pytest.raises((ValueError, AssertionError)):
+        convert.main(str(src), str(tmp_path / "out"), n_experts=4, mp=2)
+    convert.main(str(src), str(tmp_path / "out1"), n_experts=4, mp=1)        # unsplit: fine

@@ -128,3 +128,68 @@ def test_bf16_to_fp8_and_back(tmp_path):
         assert torch.equal(back[k].view(torch.int16), want.view(torch.int16)), k
         rel = (back[k].float() - tensors[k].float()).abs().max() / tensors[k].float().abs().max()
         assert rel < 0.07, (k, rel)                                     # half an e4m3 step of the block maximum
+
+
+def test_hf_checkpoint_to_loaded_modules(tmp_path):
+    """The whole way a real checkpoint takes: HF-named bf16 tensors -> bf16_cast_fp8 (weight + weight_scale_inv) ->
+    convert (local names, one rank) -> load_state_dict(strict) into FP8 modules -> forward.  The loaded MLP and MoE
+    give the oracle's result for the oracle's quantisation of the same bf16 weights."""
+    from dsv3fp8 import bf16_cast_fp8, convert, model as M
+    g = torch.Generator().manual_seed(5)
+    src, mid, dst = tmp_path / "bf16", tmp_path / "fp8", tmp_path / "local"
+    src.mkdir()
+    dim, inter, moe_inter, E = 256, 512, 256, 4
+
+    def w(rows, cols):
+        return (torch.randn(rows, cols, generator=g) * 0.05).bfloat16()
+    tensors = {}
+    for m, (r, c) in {"gate_proj": (inter, dim), "up_proj": (inter, dim), "down_proj": (dim, inter)}.items():
+        tensors[f"model.layers.0.mlp.{m}.weight"] = w(r, c)
+    tensors["model.layers.1.mlp.gate.weight"] = torch.randn(E, dim, generator=g).bfloat16()
+    for owner in [f"experts.{e}" for e in range(E)] + ["shared_experts"]:
+        for m, (r, c) in {"gate_proj": (moe_inter, dim), "up_proj": (moe_inter, dim), "down_proj": (dim, moe_inter)}.items():
+            tensors[f"model.layers.1.mlp.{owner}.{m}.weight"] = w(r, c)
+    save_file(tensors, str(src / "model-00001-of-00001.safetensors"))
+    bf16_cast_fp8.main(str(src), str(mid))
+    convert.main(str(mid), str(dst), n_experts=E, mp=1)
+    state = load_file(str(dst / "model0-mp1.safetensors"))
+
+    args = M.ModelArgs(dim=dim, inter_dim=inter, moe_inter_dim=moe_inter, n_routed_experts=E, n_activated_experts=2,
+                       n_expert_groups=1, n_limited_groups=1, score_func="softmax", route_scale=1.0)
+    old_impl, old_dtype, old_default = M.gemm_impl, M.Linear.dtype, torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    M.Linear.dtype, M.gemm_impl = FP8, "fp8"
+    try:
+        with torch.device("cuda"):
+            mlp, moe = M.MLP(dim, inter), M.MoE(args)
+        mlp.load_state_dict({k[len("layers.0.ffn."):]: v for k, v in state.items() if k.startswith("layers.0.ffn.")}, strict=True)
+        moe.load_state_dict({k[len("layers.1.ffn."):]: v for k, v in state.items() if k.startswith("layers.1.ffn.")}, strict=True)
+        assert mlp.w1.weight.dtype == FP8 and mlp.w1.weight.scale is mlp.w1.scale          # the attribute survives loading
+        x = torch.randn(24, dim, generator=g).bfloat16()
+        with torch.inference_mode():
+            y_mlp, y_moe = mlp(x.cuda()), moe(x.cuda())
+            weights, indices = (t.cpu() for t in moe.gate(x.cuda()))       # the routing itself is test_gpu_gate's subject
+    finally:
+        M.gemm_impl, M.Linear.dtype = old_impl, old_dtype
+        torch.set_default_dtype(old_default)
+
+    def expert(prefix):          # (w1, s1, w2, s2, w3, s3) as the oracle's quantiser makes them from the bf16 weights
+        out = []
+        for m in ("gate_proj", "down_proj", "up_proj"):
+            out += list(oracle.block_quant_weight(tensors[f"{prefix}.{m}.weight"]))
+        return tuple(out)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        ref_mlp = oracle.mlp(x, *expert("model.layers.0.mlp"))
+        ref_moe = oracle.moe(x, weights, indices, [expert(f"model.layers.1.mlp.experts.{e}") for e in range(E)],
+                             expert("model.layers.1.mlp.shared_experts"))
+    finally:
+        torch.set_default_dtype(old)
+
+    def close(got, ref, tol=2e-2):
+        got, ref = got.float().cpu(), ref.float()
+        rms = ref.pow(2).mean().sqrt().item()
+        assert (got - ref).abs().max().item() <= tol * rms + 2 ** -7 * ref.abs().max().item()
+    close(y_mlp, ref_mlp)
+    close(y_moe, ref_moe)
