@@ -131,24 +131,31 @@ __device__ __forceinline__ void tiles_from_counts(
         const int* counts, int groups, int tile_rows, int max_tiles,
         int* __restrict__ tile_group, int* __restrict__ tile_row0, int* __restrict__ tile_nrows,
         int* offsets) {                        // optional: first row of every group
-    __shared__ int tile_base[kThreads + 1], row_base[kThreads + 1];
+    // Exclusive scans of (tiles, rows) over the groups, kThreads groups per batch: lane shuffles inside a
+    // wavefront, the wavefronts' totals through LDS -- two barriers per batch.
+    constexpr int kWaves = kThreads / kWave;
+    __shared__ int wave_tiles[2][kWaves], wave_rows[2][kWaves];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     int done_tiles = 0, done_rows = 0;
-    for (int g0 = 0; g0 < groups; g0 += kThreads) {
+    for (int g0 = 0, batch = 0; g0 < groups; g0 += kThreads, ++batch) {
         const int g = g0 + threadIdx.x;
         const int cnt = g < groups ? counts[g] : 0;
         const int nt = (cnt + tile_rows - 1) / tile_rows;
-        // exclusive scans over this batch of groups (Hillis-Steele in LDS)
-        tile_base[threadIdx.x + 1] = nt; row_base[threadIdx.x + 1] = cnt;
-        if (threadIdx.x == 0) { tile_base[0] = 0; row_base[0] = 0; }
-        __syncthreads();
-        for (int d = 1; d < kThreads; d <<= 1) {
-            const int a = threadIdx.x + 1 >= d + 1 ? tile_base[threadIdx.x + 1 - d] : 0;
-            const int b = threadIdx.x + 1 >= d + 1 ? row_base[threadIdx.x + 1 - d] : 0;
-            __syncthreads();
-            tile_base[threadIdx.x + 1] += a; row_base[threadIdx.x + 1] += b;
-            __syncthreads();
+        int st = nt, sr = cnt;                 // inclusive scans over the wavefront
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            const int a = __shfl_up(st, d), b = __shfl_up(sr, d);
+            if (lane >= d) { st += a; sr += b; }
         }
-        const int t0 = done_tiles + tile_base[threadIdx.x], r0 = done_rows + row_base[threadIdx.x];
+        int* wt = wave_tiles[batch & 1]; int* wr = wave_rows[batch & 1];      // (alternating: one barrier per batch)
+        if (lane == kWave - 1) { wt[wave] = st; wr[wave] = sr; }
+        __syncthreads();
+        int t0 = done_tiles + st - nt, r0 = done_rows + sr - cnt, all_t = 0, all_r = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            if (w < wave) { t0 += wt[w]; r0 += wr[w]; }
+            all_t += wt[w]; all_r += wr[w];
+        }
         if (offsets && g < groups) offsets[g] = r0;
         for (int i = 0; i < nt; ++i) {
             if (t0 + i < max_tiles) {
@@ -157,8 +164,7 @@ __device__ __forceinline__ void tiles_from_counts(
                 tile_nrows[t0 + i] = min(tile_rows, cnt - i * tile_rows);
             }
         }
-        done_tiles += tile_base[kThreads]; done_rows += row_base[kThreads];
-        __syncthreads();
+        done_tiles += all_t; done_rows += all_r;
     }
     for (int t = done_tiles + threadIdx.x; t < max_tiles; t += kThreads) {
         tile_group[t] = -1; tile_row0[t] = 0; tile_nrows[t] = 0;
@@ -193,64 +199,18 @@ __global__ __launch_bounds__(kThreads) void route_count_kernel(
         if (bins[e]) atomicAdd(&counts[e], bins[e]);
 }
 
-// One thread per token: its experts in ascending order get the next free row of their group.  The order of rows
-// inside a group depends on the order in which threads arrive, which is harmless: a row of the grouped GEMM does
-// not depend on its position, and `rows` records where each pair went.  With `shared_one` != 0 every token also
-// takes row t of one more group (index `experts`, rows in token order) as its last entry, with that 16-bit
-// pattern (1.0 in the weights' type) as its weight: the outputs then have topk + 1 columns.
-template <int MAXK>
-__device__ __forceinline__ void scatter_token(
-        int t, const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int topk, int experts,
+// One thread per (token, slot) pair: the pair takes the next free row of its expert's group.  `rows` lists a
+// token's pairs in ascending expert order -- the order in which the reference's loop adds them -- so a pair finds
+// its place by counting the token's other entries that sort before it (smaller expert, or the same expert in an
+// earlier slot: the order a stable sort gives).  The order of rows inside a group depends on the order in which
+// threads arrive, which is harmless: a row of the grouped GEMM does not depend on its position, and `rows`
+// records where each pair went.  With `shared_one` != 0 every token also takes row t of one more group (index
+// `experts`, rows in token order) as its last entry, with that 16-bit pattern (1.0 in the weights' type) as its
+// weight: the outputs then have topk + 1 columns.
+__device__ __forceinline__ void scatter_pair(
+        int64_t p, const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int topk, int experts,
         const int* offsets, int* cursor, int* __restrict__ a_rows, int* __restrict__ rows,
         uint16_t* __restrict__ w_sorted, int shared_one) {
-    const int cols = topk + (shared_one ? 1 : 0);
-    int e[MAXK], slot[MAXK];
-#pragma unroll
-    for (int j = 0; j < MAXK; ++j) {
-        e[j] = j < topk ? (int)indices[(int64_t)t * topk + j] : 0x7fffffff;
-        slot[j] = j;
-    }
-    // insertion sort by expert index (stable; the reference's top-k never repeats an expert for a token)
-#pragma unroll
-    for (int i = 1; i < MAXK; ++i) {
-#pragma unroll
-        for (int j = i; j > 0; --j) {
-            if (e[j] < e[j - 1]) {
-                const int te = e[j]; e[j] = e[j - 1]; e[j - 1] = te;
-                const int ts = slot[j]; slot[j] = slot[j - 1]; slot[j - 1] = ts;
-            }
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < MAXK; ++j) {
-        if (j < topk) {
-            int pos = 0;
-            if (e[j] >= 0 && e[j] < experts) {
-                pos = offsets[e[j]] + atomicAdd(&cursor[e[j]], 1);
-                a_rows[pos] = t;
-            }
-            rows[(int64_t)t * cols + j] = pos;
-            w_sorted[(int64_t)t * cols + j] = weights[(int64_t)t * topk + slot[j]];
-        }
-    }
-    if (shared_one) {
-        const int pos = offsets[experts] + t;
-        a_rows[pos] = t;
-        rows[(int64_t)t * cols + topk] = pos;
-        w_sorted[(int64_t)t * cols + topk] = (uint16_t)shared_one;
-    }
-}
-
-// The same scatter with one thread per (token, slot) pair, for many tokens: a pair finds its place in the token's
-// ascending-expert order by counting the token's other entries that sort before it (smaller expert, or the same
-// expert in an earlier slot: the order a stable sort gives), so no thread sorts and 8x as many threads share the
-// atomics' latency.
-__global__ __launch_bounds__(kThreads) void route_scatter_pairs_kernel(
-        const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int64_t pairs, int topk, int experts,
-        const int* __restrict__ offsets, int* __restrict__ cursor,
-        int* __restrict__ a_rows, int* __restrict__ rows, uint16_t* __restrict__ w_sorted, int shared_one) {
-    const int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (p >= pairs) return;
     const int t = (int)(p / topk), j0 = (int)(p - (int64_t)t * topk);
     const int cols = topk + (shared_one ? 1 : 0);
     const int64_t e = indices[p];
@@ -274,9 +234,16 @@ __global__ __launch_bounds__(kThreads) void route_scatter_pairs_kernel(
     }
 }
 
+__global__ __launch_bounds__(kThreads) void route_scatter_pairs_kernel(
+        const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int64_t pairs, int topk, int experts,
+        const int* __restrict__ offsets, int* __restrict__ cursor,
+        int* __restrict__ a_rows, int* __restrict__ rows, uint16_t* __restrict__ w_sorted, int shared_one) {
+    const int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (p < pairs) scatter_pair(p, indices, weights, topk, experts, offsets, cursor, a_rows, rows, w_sorted, shared_one);
+}
+
 // The whole bookkeeping in one workgroup, for token counts up to kThreads (decode steps): counts, offsets and
 // cursors stay in LDS; only the counts are also written out.
-template <int MAXK>
 __global__ __launch_bounds__(kThreads) void route_small_kernel(
         const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int tokens, int topk, int experts,
         int groups, int tile_rows, int max_tiles, int* __restrict__ counts_out, int* __restrict__ offsets_out,
@@ -299,8 +266,8 @@ __global__ __launch_bounds__(kThreads) void route_small_kernel(
     tiles_from_counts(bins, groups, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows, offs);
     __syncthreads();
     for (int g = threadIdx.x; g < groups; g += kThreads) offsets_out[g] = offs[g];
-    if (t < tokens)
-        scatter_token<MAXK>(t, indices, weights, topk, experts, offs, cur, a_rows, rows, w_sorted, shared_one);
+    for (int p = threadIdx.x; p < tokens * topk; p += kThreads)
+        scatter_pair(p, indices, weights, topk, experts, offs, cur, a_rows, rows, w_sorted, shared_one);
 }
 
 }  // namespace
@@ -311,7 +278,7 @@ int launch_moe_route(const int64_t* indices, const void* weights, int64_t tokens
     const int64_t pairs = tokens * topk;
     const int groups = experts + (shared_one ? 1 : 0);
     if (tokens <= kThreads && groups <= 4096) {
-        hipLaunchKernelGGL(route_small_kernel<16>, dim3(1), dim3(kThreads), (size_t)3 * groups * sizeof(int), st,
+        hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(kThreads), (size_t)3 * groups * sizeof(int), st,
                            indices, (const uint16_t*)weights, (int)tokens, topk, experts, groups, tile_rows, max_tiles,
                            counts, offsets, a_rows, rows, (uint16_t*)w_sorted, tile_group, tile_row0, tile_nrows, shared_one);
         return launch_status();
