@@ -234,12 +234,45 @@ __device__ __forceinline__ void scatter_pair(
     }
 }
 
+// Many tokens: a workgroup first ranks its kThreads pairs per expert in LDS and then takes one range of rows per
+// expert it holds with a single global atomic -- a popular expert otherwise serialises one atomic per row.
 __global__ __launch_bounds__(kThreads) void route_scatter_pairs_kernel(
         const int64_t* __restrict__ indices, const uint16_t* __restrict__ weights, int64_t pairs, int topk, int experts,
         const int* __restrict__ offsets, int* __restrict__ cursor,
         int* __restrict__ a_rows, int* __restrict__ rows, uint16_t* __restrict__ w_sorted, int shared_one) {
+    extern __shared__ int lds_i[];
+    int* held = lds_i;                      // pairs of this workgroup per expert, then the first row of its range
+    for (int e = threadIdx.x; e < experts; e += kThreads) held[e] = 0;
+    __syncthreads();
     const int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (p < pairs) scatter_pair(p, indices, weights, topk, experts, offsets, cursor, a_rows, rows, w_sorted, shared_one);
+    const int64_t e = p < pairs ? indices[p] : -1;
+    const bool routed = e >= 0 && e < experts;
+    const int local = routed ? atomicAdd(&held[e], 1) : 0;
+    __syncthreads();
+    for (int x = threadIdx.x; x < experts; x += kThreads)
+        if (held[x]) held[x] = offsets[x] + atomicAdd(&cursor[x], held[x]);
+    __syncthreads();
+    if (p >= pairs) return;
+    const int t = (int)(p / topk), j0 = (int)(p - (int64_t)t * topk);
+    const int cols = topk + (shared_one ? 1 : 0);
+    int rank = 0;
+    for (int j = 0; j < topk; ++j) {
+        const int64_t o = indices[(int64_t)t * topk + j];
+        rank += (o < e || (o == e && j < j0)) ? 1 : 0;
+    }
+    int pos = 0;
+    if (routed) {
+        pos = held[e] + local;
+        a_rows[pos] = t;
+    }
+    rows[(int64_t)t * cols + rank] = pos;
+    w_sorted[(int64_t)t * cols + rank] = weights[p];
+    if (shared_one && j0 == 0) {
+        const int spos = offsets[experts] + t;
+        a_rows[spos] = t;
+        rows[(int64_t)t * cols + topk] = spos;
+        w_sorted[(int64_t)t * cols + topk] = (uint16_t)shared_one;
+    }
 }
 
 // The whole bookkeeping in one workgroup, for token counts up to kThreads (decode steps): counts, offsets and
@@ -291,7 +324,8 @@ int launch_moe_route(const int64_t* indices, const void* weights, int64_t tokens
                        indices, pairs, experts, counts, shared_one ? (int)tokens : 0);
     hipLaunchKernelGGL(group_tiles_kernel, dim3(1), dim3(kThreads), 0, st,
                        (const int*)counts, groups, tile_rows, max_tiles, tile_group, tile_row0, tile_nrows, offsets);
-    hipLaunchKernelGGL(route_scatter_pairs_kernel, dim3((unsigned)((pairs + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
+    hipLaunchKernelGGL(route_scatter_pairs_kernel, dim3((unsigned)((pairs + kThreads - 1) / kThreads)), dim3(kThreads),
+                       (size_t)experts * sizeof(int), st,
                        indices, (const uint16_t*)weights, pairs, topk, experts, (const int*)offsets, cursor,
                        a_rows, rows, (uint16_t*)w_sorted, shared_one);
     return launch_status();
