@@ -26,7 +26,7 @@
 namespace dsv3 {
 namespace skinny {
 
-constexpr int kMaxWaves = 8;
+constexpr int kMaxWaves = 16;
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
     v8i r = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
@@ -305,7 +305,10 @@ inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
         p.mt = 1;
         p.s = s_;
         const int64_t groups = (n + 16 * s_ - 1) / (16 * s_);
-        int waves = kMaxWaves;                  // (8 against 4: fewer K splits; wo 16384 -> 7168 at one row 27.0 -> 25.7 us)
+        // more wavefronts per workgroup = fewer K splits, down to a single pass: at one row 16 against 4 gives
+        // wq_a 7168 -> 1536 8.05 -> 6.8 us, wo 16384 -> 7168 27.0 -> 25.6 us; from a few rows up the activation slab a
+        // workgroup stages first grows with its K range, and 8 is the better limit (wkv_a at 8 rows: 7.2 against 7.8 us)
+        int waves = m <= 2 ? kMaxWaves : 8;
         while (waves > 1 && (kb / waves < 2 || groups * waves > capacity)) waves >>= 1;
         int64_t splits = capacity / (groups * waves);
         const int64_t max_splits = kb / (2 * waves) > 0 ? kb / (2 * waves) : 1;
