@@ -177,6 +177,22 @@ def test_swiglu_quant(K, fmt):
     assert torch.equal(s, sd) and torch.equal(y.view(torch.uint8), yd.view(torch.uint8))
 
 
+def test_swiglu_quant_every_bf16_value(K):
+    """silu over all 65536 bf16 bit patterns (times 1, and times a second factor) against F.silu on the device
+    followed by the bf16 product and act_quant: the kernel's exp and division must round to the same bf16."""
+    from dsv3fp8 import _lib
+    x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).view(512, 128)
+    x = torch.where(torch.isnan(x), torch.zeros_like(x), x)            # NaN payloads are not compared
+    h3 = torch.cat([torch.ones(256, 128), torch.full((256, 128), -0.3359375)]).bfloat16()
+    h = torch.cat([x, h3], dim=1).cuda().contiguous()
+    y, s = torch.ops.dsv3fp8.swiglu_quant(h, 128, _lib.SCALE_FMT_NONE)
+    gd = F.silu(h[:, :128]) * h[:, 128:]
+    finite = torch.isfinite(gd).all(dim=1)                              # rows with +-inf quantise to NaN scales
+    yd, sd = K.act_quant(gd.contiguous(), 128, None)
+    assert finite.sum().item() >= 500
+    assert torch.equal(s[finite], sd[finite]) and torch.equal(y.view(torch.uint8)[finite], yd.view(torch.uint8)[finite])
+
+
 @pytest.mark.parametrize("with_shared", [True, False])
 def test_moe_combine_bit_exact(K, with_shared):
     g = torch.Generator().manual_seed(4)
