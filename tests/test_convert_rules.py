@@ -204,3 +204,17 @@ def test_convert_refuses_a_split_inside_a_scale_block(tmp_path):
     with pytest.raises((ValueError, AssertionError)):
         convert.main(str(src), str(tmp_path / "out"), n_experts=4, mp=2)
     convert.main(str(src), str(tmp_path / "out1"), n_experts=4, mp=1)        # unsplit: fine
+
+
+@pytest.mark.parametrize("script,flag", [("convert.py", "--hf-ckpt-path"), ("fp8_cast_bf16.py", "--input-fp8-hf-path"),
+                                         ("bf16_cast_fp8.py", "--input-bf16-hf-path")])
+def test_command_line_aliases_keep_the_reference_flags(script, flag):
+    """The three scripts beside kernel.py start from that directory, as the reference's do from inference/, and
+    take the reference's flags (convert.py:88-96, fp8_cast_bf16.py:106-111)."""
+    import os
+    import subprocess
+    import sys
+    here = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "deepseek-v3_amd")
+    r = subprocess.run([sys.executable, script, "--help"], cwd=here, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert flag in r.stdout
