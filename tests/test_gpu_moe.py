@@ -327,7 +327,7 @@ def test_moe_layer_with_power_of_two_scales(K, monkeypatch):
 
 @pytest.mark.parametrize("shared", [False, True])
 @pytest.mark.parametrize("tokens,topk,experts", [(300, 2, 8), (4096, 8, 256), (1, 4, 16), (33, 1, 5), (256, 8, 256),
-                                                 (257, 8, 256)])
+                                                 (257, 8, 256), (50, 4, 700), (1000, 3, 700)])   # 700: three scan batches
 def test_moe_route(K, tokens, topk, experts, shared):
     """Both routes of the bookkeeping (one workgroup up to 256 tokens, four kernels above), with and without the
     extra group that every token selects last with weight 1."""
