@@ -94,18 +94,47 @@ __global__ __launch_bounds__(64 * kTokensPerWg) void gate_route_kernel(
 
     if (n_groups > 1) {
         float* mine = sh[wave];
-#pragma unroll
-        for (int s = 0; s < EPL; ++s) mine[s * 64 + lane] = sel[s];
         const int gsz = experts / n_groups;
         Best gs = { ninf, lane };
-        if (lane < n_groups) {
-            float top1 = ninf, top2 = ninf;
-            for (int j = 0; j < gsz; ++j) {
-                const float v = mine[lane * gsz + j];
-                if (v > top1) { top2 = top1; top1 = v; }
-                else if (v > top2) top2 = v;
+        if (gsz == 32) {
+            // a group is one half of a wavefront in one slot (the 671B router: 256 experts in 8 groups): its two
+            // largest values by merging (top1, top2) pairs of disjoint lane sets -- four DPP steps inside each row
+            // of 16 lanes, then the two rows of a half through scalar lane reads; every lane stays busy
+#pragma unroll
+            for (int s = 0; s < EPL; ++s) {
+                float t1 = sel[s], t2 = ninf;
+                auto merge = [&](float o1, float o2) {
+                    const float lo = fminf(t1, o1);
+                    t1 = fmaxf(t1, o1);
+                    t2 = fmaxf(lo, fmaxf(t2, o2));
+                };
+                auto f = [](float x) { return __builtin_bit_cast(int, x); };
+                auto g = [](int x) { return __builtin_bit_cast(float, x); };
+                { const float o1 = g(dpp_mov<0xB1>(f(t1))), o2 = g(dpp_mov<0xB1>(f(t2))); merge(o1, o2); }
+                { const float o1 = g(dpp_mov<0x4E>(f(t1))), o2 = g(dpp_mov<0x4E>(f(t2))); merge(o1, o2); }
+                { const float o1 = g(dpp_mov<0x141>(f(t1))), o2 = g(dpp_mov<0x141>(f(t2))); merge(o1, o2); }
+                { const float o1 = g(dpp_mov<0x140>(f(t1))), o2 = g(dpp_mov<0x140>(f(t2))); merge(o1, o2); }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {                      // group 2 s + h: rows 2 h and 2 h + 1
+                    const float a1 = g(__builtin_amdgcn_readlane(f(t1), 32 * h)), a2 = g(__builtin_amdgcn_readlane(f(t2), 32 * h));
+                    const float b1 = g(__builtin_amdgcn_readlane(f(t1), 32 * h + 16)), b2 = g(__builtin_amdgcn_readlane(f(t2), 32 * h + 16));
+                    const float top1 = fmaxf(a1, b1), top2 = fmaxf(fminf(a1, b1), fmaxf(a2, b2));
+                    if (lane == 2 * s + h && 2 * s + h < n_groups) gs.v = bias ? top1 + top2 : top1;
+                }
             }
-            gs.v = bias ? top1 + top2 : top1;
+        } else {
+            // any other group size: through LDS, lane g walks group g
+#pragma unroll
+            for (int s = 0; s < EPL; ++s) mine[s * 64 + lane] = sel[s];
+            if (lane < n_groups) {
+                float top1 = ninf, top2 = ninf;
+                for (int j = 0; j < gsz; ++j) {
+                    const float v = mine[lane * gsz + j];
+                    if (v > top1) { top2 = top1; top1 = v; }
+                    else if (v > top2) top2 = v;
+                }
+                gs.v = bias ? top1 + top2 : top1;
+            }
         }
         uint64_t keep = 0;
         for (int t = 0; t < topk_groups; ++t) {
