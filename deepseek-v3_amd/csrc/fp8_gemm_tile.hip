@@ -25,7 +25,6 @@
 namespace dsv3 {
 namespace {
 
-constexpr int kRowBytes = 128;           // one K block of fp8 per tile row
 constexpr int kRowStride = 128 + 16;     // padded: consecutive rows land in different banks
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
