@@ -99,30 +99,31 @@ __global__ __launch_bounds__(kThreads) void swiglu_quant_kernel(
 
 // One thread per 16-byte chunk of a token's output row (grid: tokens x chunk blocks).  rows[t, k] is the row of
 // `out` holding the token's k-th expert output in ascending expert order, w[t, k] the matching routing weight
-// (bf16).  The additions are a dependent chain of bf16 roundings, the loads are not: four experts' chunks are
+// (bf16).  The additions are a dependent chain of bf16 roundings, the loads are not: eight experts' chunks are
 // fetched before they are added.
 __global__ __launch_bounds__(kThreads) void moe_combine_kernel(
         const v4u* __restrict__ out, const int* __restrict__ rows, const uint16_t* __restrict__ w,
         const v4u* __restrict__ shared, v4u* __restrict__ y, int topk, int chunks_per_row) {
     const int t = blockIdx.x;
-    const int c = blockIdx.y * kThreads + threadIdx.x;
+    const int c = blockIdx.y * (int)blockDim.x + threadIdx.x;
     if (c >= chunks_per_row) return;
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
     v4u z = {0u, 0u, 0u, 0u};
     if (shared) z = shared[(int64_t)t * chunks_per_row + c];
-    for (int k0 = 0; k0 < topk; k0 += 4) {
-        v4u v[4];
-        float wk[4];
+    constexpr int U = 8;                      // expert rows fetched before they are added
+    for (int k0 = 0; k0 < topk; k0 += U) {
+        v4u v[U];
+        float wk[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int k = min(k0 + u, topk - 1);
             wk[u] = bf16lo_to_f32(w[(int64_t)t * topk + k]);
-            v[u] = out[(int64_t)rows[(int64_t)t * topk + k] * chunks_per_row + c];
+            v[u] = __builtin_nontemporal_load(out + (int64_t)rows[(int64_t)t * topk + k] * chunks_per_row + c);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             if (k0 + u < topk) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
@@ -367,8 +368,11 @@ int launch_swiglu_quant(const void* h, void* y, float* s, int64_t rows, int64_t 
 
 int launch_moe_combine(const void* out, const int* rows, const void* w, const void* shared, void* y,
                        int64_t tokens, int topk, int64_t dim, hipStream_t st) {
-    const unsigned chunk_blocks = (unsigned)((dim / 8 + kThreads - 1) / kThreads);
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)tokens, chunk_blocks), dim3(kThreads), 0, st,
+    // 128 threads where that leaves no partly filled workgroup (7168 columns = 896 chunks = 7 x 128)
+    const int64_t chunks = dim / 8;
+    const int threads = (chunks % kThreads != 0 && chunks % 128 == 0) ? 128 : kThreads;
+    const unsigned chunk_blocks = (unsigned)((chunks + threads - 1) / threads);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)tokens, chunk_blocks), dim3(threads), 0, st,
                        (const v4u*)out, rows, (const uint16_t*)w, (const v4u*)shared, (v4u*)y, topk, (int)(dim / 8));
     return launch_status();
 }
