@@ -1,7 +1,8 @@
 // fp8_gemm for decode shapes with a wide enough N: producer / consumer weight-streaming kernel
 // (reference arithmetic: inference/kernel.py:145-172).
 //
-// A workgroup is five wavefronts.  Four CONSUMERS each own a 16-row strip of b (64 rows per workgroup) and walk
+// A workgroup is five or nine wavefronts.  Four or eight CONSUMERS each own a 16-row strip of b (64 or 128 rows per
+// workgroup, inside one 128-row block of weight scales) and walk
 // the workgroup's K range; their weights go straight from global memory into the MFMA register layout through a
 // ring of NPF K blocks whose loads and waits are written out explicitly (inline asm), so that exactly NPF-1
 // blocks stay in flight behind the one being multiplied.  The fifth wavefront is the PRODUCER: it copies the
@@ -19,8 +20,8 @@ namespace stream {
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-constexpr int kConsumers = 4;
-constexpr int kThreads = (kConsumers + 1) * kWave;
+constexpr int kMaxConsumers = 8;          // consumer wavefronts per workgroup: 4 or 8, chosen per launch (blockDim.x / 64 - 1)
+constexpr int kThreads = (kMaxConsumers + 1) * kWave;
 
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
@@ -78,9 +79,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
     const int kb0 = blockIdx.y * nkb;
     const int nchunks = nkb / KC;
 
-    if (wave == kConsumers) {
+    const int consumers = (int)(blockDim.x >> 6) - 1, group_rows = consumers * 16;
+    if (wave == consumers) {
         // ------------------------------------------------------------------ producer
-        const float* bs_src = b_s + (size_t)min((int)(blockIdx.x * 64) >> 7, (N - 1) >> 7) * KB + kb0;
+        const float* bs_src = b_s + (size_t)min((int)(blockIdx.x * group_rows) >> 7, (N - 1) >> 7) * KB + kb0;
         for (int c = 0; c < nchunks; ++c) {
             const int buf = c & 1;
 #pragma unroll
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
 
     // ---------------------------------------------------------------------- consumers
     const int fr = lane & 15, fq = lane >> 4;
-    const int n0 = blockIdx.x * 64 + wave * 16;
+    const int n0 = blockIdx.x * group_rows + wave * 16;
     // lane offsets of its two rows (strip rows fr&7 and (fr&7)+8, clamped to the last row of b) from b, < 2^32
     const uint32_t off_lo = (uint32_t)min(n0 + (fr & 7), N - 1) * (uint32_t)K + (fr >> 3) * 64 + fq * 16;
     const uint32_t off_hi = (uint32_t)min(n0 + (fr & 7) + 8, N - 1) * (uint32_t)K + (fr >> 3) * 64 + fq * 16;
@@ -179,9 +181,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
     }
 }
 
-struct Plan { bool ok; int mt, npf, splits, nkb; };
+struct Plan { bool ok; int mt, npf, splits, nkb, consumers; };
 
-// Usable when N gives enough 64-row groups and the K range splits evenly into ring-sized pieces.
+// Usable when N gives enough groups of 64 (128) rows and the K range splits evenly into ring-sized pieces.
 inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
     Plan p{};
     p.ok = false;
@@ -189,9 +191,13 @@ inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
     if (m <= 16 || m > 64 || k < 1024 || k % 128 || n * k >= (1ll << 32)) return p;
     p.mt = (int)((m + 15) / 16);
     if (p.mt == 3) p.mt = 4;                                    // 3 sub-tiles run as 4 (chunk size stays a power of two)
-    const int64_t kb = k / 128, groups = (n + 63) / 64;
+    // eight consumer wavefronts share an activation chunk where N gives enough groups of 128 rows (half the
+    // activation traffic per weight byte: wq_b 1536 -> 24576 at 64 rows 18.0 -> 16.9 us, wq_a 15.1 -> 14.3), four
+    // otherwise (wkv_a 7168 -> 576: 11.0 against 12.5 us)
+    p.consumers = n >= 1024 ? 8 : 4;
+    const int64_t kb = k / 128, groups = (n + 16 * p.consumers - 1) / (16 * p.consumers);
     if (groups < 4) return p;                                   // a handful of rows: not worth a streaming plan
-    const int64_t capacity = 256 * 3;                           // resident workgroups (3 per CU)
+    const int64_t capacity = 256 * (p.consumers == 4 ? 3 : 1);     // resident workgroups (3 per CU with five wavefronts, 1 with nine)
     // K blocks per workgroup: a divisor of kb that is a multiple of the ring depth; take the split count that
     // fills one round best
     int best_nkb = 0, best_npf = 0;
@@ -219,8 +225,9 @@ void launch_cfg(const Plan& p, const void* a, const float* a_s, const void* b, c
                 void* out, int od, int m, int n, int k, hipStream_t st) {
     constexpr int KC = MT == 1 ? (NPF < 8 ? NPF : 8) : (MT == 2 ? 4 : 2);
     const size_t lds = 2 * (size_t)KC * 16 * MT * (128 + 4);
-    const dim3 grid((unsigned)((n + 63) / 64), (unsigned)p.splits);
-    hipLaunchKernelGGL((fp8_gemm_stream_kernel<MT, NPF, KC>), grid, dim3(kThreads), lds, st,
+    const int group_rows = 16 * p.consumers;
+    const dim3 grid((unsigned)((n + group_rows - 1) / group_rows), (unsigned)p.splits);
+    hipLaunchKernelGGL((fp8_gemm_stream_kernel<MT, NPF, KC>), grid, dim3((p.consumers + 1) * kWave), lds, st,
                        (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, od, m, n, k, p.nkb);
 }
 
