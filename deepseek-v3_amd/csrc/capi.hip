@@ -1,13 +1,38 @@
 // C ABI of libdsv3fp8.so: host-side argument validation and dispatch.
 // Everything is checked before the first HIP call so that the error paths are
 // usable (and tested) on a machine without a GPU.
+#include <mutex>
 #include "common.hpp"
 
 using namespace dsv3;
 
+// Split-K scratch of dsv3_fp8_gemm_static: part of the loaded code object, so every GPU the library runs on holds
+// its own copy at its own address until the process ends.  Host code never passes this name to a kernel (on the
+// host it is only a stand-in for the symbol): static_scratch() resolves the device address once per device.
+static __device__ __align__(256) unsigned char scratch[DSV3_STATIC_SCRATCH_BYTES];
+
 namespace {
 inline bool aligned(const void* p, uintptr_t a) { return ((uintptr_t)p % a) == 0; }
 inline bool valid_dtype(int d) { return d == DSV3_BF16 || d == DSV3_F16 || d == DSV3_F32; }
+
+// Device address of `scratch` on the current device (nullptr on failure); resolved on the first call per device.
+void* static_scratch() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* ptr[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        ptr[dev] = p;
+    }
+    return ptr[dev];
+}
 }
 
 extern "C" {
@@ -24,6 +49,7 @@ const char* dsv3_status_string(int status) {
         case DSV3_ERR_BAD_DTYPE: return "unsupported dtype code";
         case DSV3_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case DSV3_ERR_LAUNCH: return "HIP launch failed";
+        case DSV3_ERR_TOO_LARGE: return "problem needs more scratch than the library's fixed array holds (use the entry point that takes a workspace)";
         default: return "unknown status";
     }
 }
@@ -72,9 +98,10 @@ size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
     return fp8_gemm_workspace_bytes(m, n, k);
 }
 
-static int fp8_gemm_checked(const void* a, const float* a_s, const void* b, const float* b_s,
-                           void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
-                           void* workspace, size_t workspace_bytes, void* stream, bool pow2_scales) {
+// Host-side checks of the fp8_gemm entry points (no GPU call).  DSV3_OK with m == 0 or n == 0 means "nothing to do".
+static int fp8_gemm_validate(const void* a, const float* a_s, const void* b, const float* b_s,
+                             void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                             void* workspace, size_t workspace_bytes) {
     if (!valid_dtype(c_dtype)) return DSV3_ERR_BAD_DTYPE;
     if (m < 0 || n < 0 || k < 0) return DSV3_ERR_BAD_SHAPE;
     if (k % 128 != 0) return DSV3_ERR_BAD_SHAPE;
@@ -87,6 +114,14 @@ static int fp8_gemm_checked(const void* a, const float* a_s, const void* b, cons
         return DSV3_ERR_MISALIGNED;
     const size_t need = dsv3_fp8_gemm_workspace_bytes(m, n, k);
     if (need > 0 && (!workspace || workspace_bytes < need || !aligned(workspace, 256))) return DSV3_ERR_WORKSPACE;
+    return DSV3_OK;
+}
+
+static int fp8_gemm_checked(const void* a, const float* a_s, const void* b, const float* b_s,
+                           void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
+                           void* workspace, size_t workspace_bytes, void* stream, bool pow2_scales) {
+    const int rc = fp8_gemm_validate(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes);
+    if (rc != DSV3_OK || m == 0 || n == 0) return rc;
     return launch_fp8_gemm(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, (hipStream_t)stream,
                            pow2_scales);
 }
@@ -101,6 +136,24 @@ int dsv3_fp8_gemm_pow2(const void* a, const float* a_s, const void* b, const flo
                        void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
                        void* workspace, size_t workspace_bytes, void* stream) {
     return fp8_gemm_checked(a, a_s, b, b_s, c, c_dtype, m, n, k, workspace, workspace_bytes, stream, true);
+}
+
+size_t dsv3_fp8_gemm_static_max_bytes(void) { return DSV3_STATIC_SCRATCH_BYTES; }
+
+int dsv3_fp8_gemm_static(const void* a, const float* a_s, const void* b, const float* b_s,
+                         void* c, int c_dtype, int64_t m, int64_t n, int64_t k, void* stream) {
+    const size_t need = dsv3_fp8_gemm_workspace_bytes(m, n, k);          // 0 for shapes the checks below refuse
+    if (need > DSV3_STATIC_SCRATCH_BYTES) return DSV3_ERR_TOO_LARGE;     // refused before anything is launched
+    // the argument checks of dsv3_fp8_gemm, with a stand-in for the workspace: no GPU call on an error path
+    alignas(256) static unsigned char stand_in;
+    const int rc = fp8_gemm_validate(a, a_s, b, b_s, c, c_dtype, m, n, k, need ? &stand_in : nullptr, need);
+    if (rc != DSV3_OK || m == 0 || n == 0) return rc;
+    void* ws = nullptr;
+    if (need) {
+        ws = static_scratch();
+        if (!ws) return DSV3_ERR_LAUNCH;
+    }
+    return launch_fp8_gemm(a, a_s, b, b_s, c, c_dtype, m, n, k, ws, DSV3_STATIC_SCRATCH_BYTES, (hipStream_t)stream, false);
 }
 
 int dsv3_linear_fp8_fused(int64_t m, int64_t n, int64_t k) {

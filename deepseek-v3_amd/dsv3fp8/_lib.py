@@ -28,6 +28,9 @@ EXPORTS = {
                               c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "dsv3_fp8_gemm_pow2": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                    c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "dsv3_fp8_gemm_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                     c_int64, c_int64, c_int64, c_void_p]),
+    "dsv3_fp8_gemm_static_max_bytes": (c_size_t, []),
     "dsv3_linear_fp8_fused": (c_int, [c_int64, c_int64, c_int64]),
     "dsv3_linear_fp8": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64,
                                 c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -44,7 +44,8 @@ typedef enum dsv3_status {
     DSV3_ERR_MISALIGNED = 4,    /* pointer not aligned as documented                       */
     DSV3_ERR_BAD_DTYPE = 5,     /* dtype code not in dsv3_dtype / not valid here           */
     DSV3_ERR_WORKSPACE = 6,     /* workspace missing or smaller than the size query says   */
-    DSV3_ERR_LAUNCH = 7         /* HIP reported an error at launch                         */
+    DSV3_ERR_LAUNCH = 7,        /* HIP reported an error at launch                         */
+    DSV3_ERR_TOO_LARGE = 8      /* dsv3_fp8_gemm_static: scratch need exceeds the fixed array */
 } dsv3_status;
 
 typedef enum dsv3_dtype {
@@ -154,6 +155,24 @@ int dsv3_fp8_gemm_pow2(const void* a, const float* a_s, const void* b, const flo
 
 /* Bytes of scratch dsv3_fp8_gemm needs for this problem (0 when none). */
 size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
+
+/*
+ * dsv3_fp8_gemm without a workspace argument and without any allocation.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  Same arithmetic, kernels, argument checks and results as dsv3_fp8_gemm
+ * (bit for bit); the partial sums of K-sliced plans go to a fixed array of DSV3_STATIC_SCRATCH_BYTES inside the
+ * library's device image (each GPU the library runs on holds its own copy until the process ends) instead of a
+ * caller's buffer.  A problem whose dsv3_fp8_gemm_workspace_bytes(m,n,k) exceeds that size is refused with
+ * DSV3_ERR_TOO_LARGE before anything is launched (every DeepSeek-V3 projection up to 4096 rows fits).
+ * The first call on a device looks the array's address up (hipGetSymbolAddress; no allocation) -- make that call
+ * outside a graph capture.  The array keeps the previous call's contents; the kernels overwrite what they read, so
+ * nothing has to be cleared.  All calls on one GPU share the array: calls that overlap in time on one GPU (two
+ * streams, two threads) race; order them on one stream.
+ */
+#define DSV3_STATIC_SCRATCH_BYTES (64u << 20)
+size_t dsv3_fp8_gemm_static_max_bytes(void);
+int dsv3_fp8_gemm_static(const void* a, const float* a_s, const void* b, const float* b_s,
+                         void* c, int c_dtype, int64_t m, int64_t n, int64_t k, void* stream);
 
 /*
  * ---- Mixture-of-experts layer on the same GEMM (inference/model.py:601-633 Expert, :669-693 MoE.forward) ----
