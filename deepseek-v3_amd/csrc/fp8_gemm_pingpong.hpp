@@ -1,0 +1,415 @@
+// fp8_gemm, 256 x 256 tile with the two wavefronts of every SIMD in opposite phases (included by
+// fp8_gemm_prefill.hip; reference arithmetic: inference/kernel.py:157-166).
+//
+// Eight wavefronts, 4 along m x 2 along n, each owning 64 (m) x 128 (n) of the tile as 4 x 8 MFMA tiles of 16 x 16
+// (one v_mfma 16x16x128 = one 128-wide scale block of K, folded into binary32 accumulators by one FMA per element
+// with a_s[m, kb] * b_s[n / 128, kb]).  Wavefront w runs on SIMD w % 4, so the two wavefronts of a SIMD are the two
+// column halves ("groups") of one row quarter.  A K block is four phases per wavefront, separated by workgroup
+// barriers:
+//     M1  read the block's activation fragments (64 rows) and the weight fragments of its first 64 columns from LDS
+//         into registers, read the block's scales, request global -> LDS copies
+//     C1  16 MFMAs on those registers, each followed by the four FMAs of the MFMA issued two earlier
+//     M2  read the weight fragments of the other 64 columns, request copies
+//     C2  16 MFMAs
+// Group 1 takes one barrier more before its first block and therefore always runs one phase behind group 0: while
+// one wavefront of a SIMD issues nothing but MFMAs and their FMAs, the other does all of its LDS and global memory
+// work, and the matrix pipe sees an uninterrupted instruction stream from one wavefront at a time.
+//
+// LDS: two stages of [256 rows of A | 256 rows of B] x 128 bytes (the chunk permutation of fp8_gemm_prefill.hip)
+// and four slots of scales.  With block kb in stage kb % 2 and phases numbered from group 0's M1 of block 0:
+//     region                      last read in phase    refilled (block kb + 2) in phase    first read again
+//     A, B columns 0-63 of both   4 kb + 1              4 kb + 2 .. 4 kb + 4                4 kb + 8
+//     B columns 64-127 of both    4 kb + 3              4 kb + 5                            4 kb + 10
+// so every copy has at least one whole K block of time to land.  Group 0 requests, per block kb, the second half of
+// A of block kb + 1 in M1 and the first-columns part of B of block kb + 2 in M2; group 1 the last-columns part of B
+// of block kb + 1 in M1 and the first half of A of block kb + 2 in M2.  Copies retire in program order, so "the
+// copies the next readers need have landed" is a vmcnt(n) with n = the number of younger copies: 9 for group 1 at
+// the end of both M phases, 4 for group 0 at the end of C2.
+#pragma once
+
+namespace pingpong {
+
+// Development aid (never defined in the library build): per-phase time stamps of every wavefront.
+#ifndef DSV3_PP_ABL
+#define DSV3_PP_ABL 0
+#endif
+#ifdef DSV3_PP_PROF
+__device__ unsigned long long pp_prof[8 * 8];
+#ifdef PP_NO_STAMPS
+#define PP_PROF_DECL
+#define PP_PROF_MARK(slot)
+#define PP_PROF_FLUSH
+#else
+#define PP_PROF_DECL unsigned long long prof_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, prof_t; \
+    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(prof_t) :: "memory");
+#define PP_PROF_MARK(slot) { unsigned long long t_; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_) :: "memory"); \
+    prof_acc[slot] += t_ - prof_t; prof_t = t_; }
+#define PP_PROF_FLUSH if (lane == 0) { for (int i_ = 0; i_ < 8; ++i_) atomicAdd(&pp_prof[wave * 8 + i_], prof_acc[i_]); }
+#endif
+__device__ unsigned long long pp_clk[4];
+#define PP_CLK(i) if (wg == 0 && threadIdx.x == 0) { unsigned long long c_, r_; \
+    asm volatile("s_memtime %0\n\ts_memrealtime %1\n\ts_waitcnt lgkmcnt(0)" : "=s"(c_), "=s"(r_) :: "memory"); pp_clk[i] = c_; pp_clk[i + 1] = r_; }
+#else
+#define PP_PROF_DECL
+#define PP_PROF_MARK(slot)
+#define PP_PROF_FLUSH
+#define PP_CLK(i)
+#endif
+
+// One global -> LDS copy of 16 (or 4) bytes per lane: uniform 64-bit base in scalar registers, 32-bit lane offset,
+// uniform LDS address through M0 (lane l lands at lds_addr + 16 l).  Written out because the compiler otherwise
+// forms a 64-bit address per lane with vector ALU instructions in front of every copy.
+__device__ __forceinline__ uint32_t lds_addr_of(const void* p) { return (uint32_t)(uintptr_t)(lptr_t)p; }
+__device__ __forceinline__ void copy16(const void* base, uint32_t lane_off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+__device__ __forceinline__ void copy4(const void* base, uint32_t lane_off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                 :: "v"(lane_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+
+constexpr int TM = 256;
+constexpr int SM = 4;                                   // 16-row sub-tiles per wavefront
+constexpr int STAGE = 256 * 128;                        // bytes of A (or of B) per K block
+constexpr int LDS_A = 0, LDS_B = 2 * STAGE, LDS_SC = 4 * STAGE;
+constexpr int SC_SLOT = 2048, SC_SLOTS = 2;
+constexpr int LDS_BYTES = LDS_SC + SC_SLOTS * SC_SLOT;  // 136 KiB
+
+template <int CD, bool P2>
+__device__ __forceinline__ void tile(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c,
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, int wg) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    // ---- workgroup -> tile: a contiguous run of tiles per XCD, walked in bands of GROUP_M tile rows
+    int m0, n0, rows_here;
+    {
+        const int T = tiles_m * tiles_n;
+        int pid = wg;
+        {
+            const int q = T / 8, r = T % 8, x = pid % 8;
+            pid = x * q + (x < r ? x : r) + pid / 8;
+        }
+        constexpr int GROUP_M = 4;
+        const int band = pid / (GROUP_M * tiles_n);
+        const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+        const int in_band = pid - band * GROUP_M * tiles_n;
+        const int tm = band * GROUP_M + in_band % band_rows;
+        const int tn = in_band / band_rows;
+        m0 = tm * TM; n0 = (tn_first + tn) * BN;
+        rows_here = min(TM, M - m0);
+    }
+    auto a_row = [&](int r) -> uint32_t { return (uint32_t)(((DSV3_PP_ABL & 16) ? 0 : m0) + min(r, rows_here - 1)); };
+    const int n0_ld = (DSV3_PP_ABL & 16) ? 0 : n0;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 3, grp = wave >> 2;
+    const int KBT = K / 128;
+    const int kb0 = blockIdx.y * kb_per_split;
+    const int KB = min(kb_per_split, KBT - kb0);
+    c += (size_t)blockIdx.y * (size_t)M * (size_t)ldc;
+    const int n_base = ldc == N ? 0 : tn_first * BN;
+    a += (size_t)kb0 * 128u; b += (size_t)kb0 * 128u;
+
+    // ---- copy plan.  A K block is 32 + 32 wavefront-copies of 8 rows (1 KiB); copy q covers rows 8q .. 8q + 7.
+    // The copies are requested in the M phases, interleaved with the LDS reads (the copy path takes one 1 KiB copy
+    // per ~16 cycles and compute unit and holds the issuing wavefront meanwhile; a wavefront in a C phase that
+    // issued them would leave gaps in its MFMA stream).  Per block kb a wavefront issues
+    //   in M1  two copies of block kb + 1:  B rows 64-127 (group 0) / 192-255 (group 1), the last-columns part
+    //   in M2  six copies of block kb + 2:  group 0  B rows 0-63 and 128-191 (4) and A rows 0-63 (2)
+    //                                       group 1  A rows 64-255 (6)
+    uint32_t m1_src[2], m2_src[6];
+    int m1_dst[2], m2_dst[6];
+    const uint8_t* m2_base[6];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int q = (grp == 0 ? 8 : 24) + wm * 2 + t;
+        const int r = q * 8 + (lane >> 3), ch = (lane & 7) ^ swz(r);
+        m1_src[t] = (uint32_t)min(n0_ld + r, N - 1) * (uint32_t)K + ch * 16;
+        m1_dst[t] = LDS_B + q * 1024;
+    }
+#pragma unroll
+    for (int t = 0; t < 6; ++t) {
+        const bool from_b = grp == 0 && t < 4;
+        int q;
+        if (grp == 0) { const int idx = wm * 4 + t; q = t < 4 ? (idx < 8 ? idx : idx + 8) : wm * 2 + (t - 4); }
+        else q = 8 + wm * 6 + t;
+        const int r = q * 8 + (lane >> 3), ch = (lane & 7) ^ swz(r);
+        m2_src[t] = (from_b ? (uint32_t)min(n0_ld + r, N - 1) : a_row(r)) * (uint32_t)K + ch * 16;
+        m2_dst[t] = (from_b ? LDS_B : LDS_A) + q * 1024;
+        m2_base[t] = from_b ? b : a;
+    }
+    auto issue_m1 = [&](int t, int kb, int stage) {
+        copy16(b + (uint32_t)kb * 128u, m1_src[t], lds_addr_of(lds + m1_dst[t] + stage * STAGE));
+    };
+    auto issue_m2 = [&](int t, int kb, int stage) {
+        copy16(m2_base[t] + (uint32_t)kb * 128u, m2_src[t], lds_addr_of(lds + m2_dst[t] + stage * STAGE));
+    };
+    // scales of a K block: wavefronts 0-3 copy a_s[row, kb] of 64 tile rows each, wavefront 4 the b_s rows of the two
+    // column halves (wavefronts 5-7 repeat that into slots nobody reads: no branch in the loop)
+    const int nb_last = (N - 1) / 128;
+    const float* sc_base = wave < 4 ? a_s : b_s;
+    const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT
+                                      : (uint32_t)min(n0 / 128 + lane, nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
+    auto issue_scales = [&](int kb, int slot) {
+        copy4(sc_base + (uint32_t)kb, sc_off * 4u, lds_addr_of(lds + LDS_SC + slot * SC_SLOT + wave * 256));
+    };
+
+    // ---- fragment addresses: lane reads row (lane & 15) of a 16-row sub-tile, K bytes 32 (lane >> 4) .. + 31
+    const int fr = lane & 15, fq = lane >> 4;
+    const int fx = swz(fr);
+    const int c0 = ((2 * fq) ^ fx) * 16, c1 = ((2 * fq + 1) ^ fx) * 16;
+    const uint8_t* a_rd = lds + LDS_A + (wm * 64 + fr) * 128;           // + j * 2048 + stage * STAGE
+    const uint8_t* b_rd = lds + LDS_B + (grp * 128 + fr) * 128;         // + i * 2048 + stage * STAGE
+    const uint8_t* sa_rd = lds + LDS_SC + (wm * 64 + fr) * 4;           // + j * 64 + slot * SC_SLOT
+    const uint8_t* sb_rd = lds + LDS_SC + (256 + grp) * 4;
+
+    v4f acc[8][SM];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < SM; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+#define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+    auto run = [&](auto gtag) {
+        constexpr int GRP = decltype(gtag)::value;
+        constexpr bool LD = !(DSV3_PP_ABL & 2), RD = !(DSV3_PP_ABL & 4);
+        // prologue: blocks 0 and 1 as far as the steady state expects them to have been requested
+#pragma unroll
+        for (int t = 0; t < 6; ++t) issue_m2(t, 0, 0);
+        issue_scales(0, 0);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) issue_m1(t, 0, 0);
+#pragma unroll
+        for (int t = 0; t < 6; ++t) issue_m2(t, min(1, KB - 1), 1);
+        issue_scales(min(1, KB - 1), 1);
+        __builtin_amdgcn_s_waitcnt(0x0f70);                         // vmcnt(0)
+        wg_barrier();
+        if (GRP == 1) wg_barrier();                                 // one phase behind group 0 from here on
+
+        v8i af[SM], bf[4];
+        v4f p14 = {0.f, 0.f, 0.f, 0.f}, p15 = {0.f, 0.f, 0.f, 0.f}; // raw products of the last two MFMAs of a C phase
+        float sc[2][SM];                                            // fold factors of even / odd blocks
+        int ea[SM], eb = 0;                                         // P2: biased exponents of the block's scales
+#pragma unroll
+        for (int j = 0; j < SM; ++j) { sc[0][j] = sc[1][j] = 0.f; ea[j] = 0; }
+
+        // 16 MFMAs over column sub-tiles I0 .. I0 + 3 with the fold factors s; every MFMA is followed by the four
+        // FMAs of the MFMA issued two earlier -- the first two by those of the previous C phase's last two MFMAs
+        // (column sub-tile IT, fold factors st), so that the M phases hold no vector ALU work: while the other
+        // wavefront of the SIMD is in a C phase, the vector ALU issues this wavefront's instructions only in the gaps.
+        auto compute = [&](auto i0_tag, auto it_tag, const float (&s)[SM], const float (&st)[SM]) {
+            constexpr int I0 = decltype(i0_tag)::value, IT = decltype(it_tag)::value;
+            __builtin_amdgcn_sched_barrier(0);
+            if (DSV3_PP_ABL & 1) __builtin_amdgcn_s_setprio(1);
+            if constexpr (P2) {
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+                    for (int j = 0; j < SM; ++j)
+                        acc[I0 + ii][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                            bf[ii], af[j], acc[I0 + ii][j], 0, 0, 0, eb, 0, ea[j]);
+            } else {
+                const v4f z = {0.f, 0.f, 0.f, 0.f};
+                v4f p[16];
+#pragma unroll
+                for (int t = 0; t < 16; ++t) {
+                    p[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[t / 4], af[t % 4], z, 0, 0, 0, 0, 0, 0);
+                    if (!(DSV3_PP_ABL & 8)) {
+                        if (t < 2) {
+                            const v4f q = t == 0 ? p14 : p15;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[IT][2 + t][e] = __builtin_fmaf(q[e], st[2 + t], acc[IT][2 + t][e]);
+                        } else {
+                            const int u = t - 2;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                acc[I0 + u / 4][u % 4][e] = __builtin_fmaf(p[u][e], s[u % 4], acc[I0 + u / 4][u % 4][e]);
+                        }
+                    }
+                    DSV3_SGB(0x008, 1);
+                    if (!(DSV3_PP_ABL & 8)) DSV3_SGB(0x002, 4);
+                }
+                p14 = p[14]; p15 = p[15];
+            }
+            if (DSV3_PP_ABL & 1) __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+
+        // one K block whose LDS stage (and scale slot) ST is a compile-time constant: every LDS address of the loop is
+        // a register plus an immediate
+        auto block = [&](int kb, auto st_tag) {
+            constexpr int ST = decltype(st_tag)::value;
+            const int kb1 = min(kb + 1, KB - 1), kb2 = min(kb + 2, KB - 1);
+            // ---- M1
+            if (RD || kb == 0) {
+                const uint8_t* as_base = a_rd + ST * STAGE;
+                const uint8_t* bs_base = b_rd + ST * STAGE;
+#pragma unroll
+                for (int j = 0; j < SM; ++j) {
+                    if (LD && j % 2 == 0) issue_m1(j / 2, kb1, ST ^ 1);
+                    af[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
+                }
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii)
+                    bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
+            }
+            {
+                const float bs = *(const float*)(sb_rd + ST * SC_SLOT);
+#pragma unroll
+                for (int j = 0; j < SM; ++j) {
+                    const float as = *(const float*)(sa_rd + j * 64 + ST * SC_SLOT);
+                    if (P2) ea[j] = (int)(f32_as_u32(as) >> 23);
+                    else sc[ST][j] = as * bs;
+                }
+                if (P2) eb = (int)(f32_as_u32(bs) >> 23);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            PP_PROF_MARK(0)
+            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | 9);
+            wg_barrier();
+            PP_PROF_MARK(1)
+            // ---- C1 (its first two FMA groups belong to C2 of the previous block: zeros at kb = 0)
+            compute(std::integral_constant<int, 0>{}, std::integral_constant<int, 7>{}, sc[ST], sc[ST ^ 1]);
+            PP_PROF_MARK(2)
+            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | 9);
+            wg_barrier();
+            PP_PROF_MARK(3)
+            // ---- M2
+            {
+                const uint8_t* bs_base = b_rd + ST * STAGE + 4 * 2048;
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii) {
+                    if (LD) issue_m2(ii, kb2, ST);
+                    if (RD) bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
+                }
+                if (LD) { issue_m2(4, kb2, ST); issue_m2(5, kb2, ST); issue_scales(kb2, ST); }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            PP_PROF_MARK(4)
+            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | 9);
+            wg_barrier();
+            PP_PROF_MARK(5)
+            // ---- C2
+            compute(std::integral_constant<int, 4>{}, std::integral_constant<int, 3>{}, sc[ST], sc[ST]);
+            PP_PROF_MARK(6)
+            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | 9);
+            wg_barrier();
+            PP_PROF_MARK(7)
+        };
+
+        PP_PROF_DECL
+        int kb = 0;
+        for (; kb + 1 < KB; kb += 2) {
+            block(kb, std::integral_constant<int, 0>{});
+            block(kb + 1, std::integral_constant<int, 1>{});
+        }
+        if (kb < KB) block(kb, std::integral_constant<int, 0>{});
+        PP_PROF_FLUSH
+        // the FMAs of the last two MFMAs
+        if (!P2) {
+            const int last = (KB - 1) & 1;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[7][2][e] = __builtin_fmaf(p14[e], last ? sc[1][2] : sc[0][2], acc[7][2][e]);
+                acc[7][3][e] = __builtin_fmaf(p15[e], last ? sc[1][3] : sc[0][3], acc[7][3][e]);
+            }
+        }
+        if (GRP == 0) wg_barrier();                                 // group 1's last phase
+        __builtin_amdgcn_s_waitcnt(0x0f70);                         // the clamped refills of the last blocks
+    };
+    PP_CLK(0)
+    if (grp == 0) run(std::integral_constant<int, 0>{});
+    else          run(std::integral_constant<int, 1>{});
+    PP_CLK(2)
+#undef DSV3_SGB
+
+    // ---- epilogue: lane holds c[m][n .. n + 3] for every (i, j); see fp8_gemm_prefill.hip for the LDS route
+    constexpr int WM = 64, WN = 128, SN = 8;
+    auto sub_row = [&](int j) { return wm * WM + j * 16; };
+    const bool lds_epilogue = CD != DSV3_F32 && (N % 8) == 0 && ldc == N;
+    const bool f32_lds_epilogue = CD == DSV3_F32 && (N % 4) == 0 && (ldc % 4) == 0;
+    const bool vec_ok = (N % 4) == 0 && (ldc % 4) == 0;
+    if (lds_epilogue) {
+        wg_barrier();
+        uint8_t* stg = lds + wave * (WM * 256);
+#pragma unroll
+        for (int j = 0; j < SM; ++j)
+#pragma unroll
+            for (int i = 0; i < SN; ++i) {
+                v2u o;
+                if (CD == DSV3_BF16) o = v2u{ pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3]) };
+                else o = v2u{ pack_f16(acc[i][j][0], acc[i][j][1]), pack_f16(acc[i][j][2], acc[i][j][3]) };
+                const int lr = j * 16 + fr, chunk = (i * 2 + (fq >> 1)) ^ fr;
+                *(v2u*)(stg + lr * 256 + chunk * 16 + (fq & 1) * 8) = o;
+            }
+        const int rr = lane >> 4, ch = lane & 15;
+#pragma unroll
+        for (int p = 0; p < WM / 4; ++p) {
+            const int lr = p * 4 + rr;
+            const v4u v = *(const v4u*)(stg + lr * 256 + ((ch ^ (lr & 15)) * 16));
+            const int r = sub_row(lr >> 4) + (lr & 15);
+            const int n = n0 + grp * WN + ch * 8;
+            if (r < rows_here && n < N)
+                *(v4u*)(c + (size_t)(m0 + r) * N + n) = v;
+        }
+        return;
+    }
+    if (f32_lds_epilogue) {
+        wg_barrier();
+        uint8_t* stg = lds + wave * (WM * 256);
+        const int rr = lane >> 4, ch = lane & 15;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int j = 0; j < SM; ++j)
+#pragma unroll
+                for (int i = 0; i < SN / 2; ++i) {
+                    const int lr = j * 16 + fr, chunk = (i * 4 + fq) ^ fr;
+                    *(v4f*)(stg + lr * 256 + chunk * 16) = acc[h * (SN / 2) + i][j];
+                }
+#pragma unroll
+            for (int p = 0; p < WM / 4; ++p) {
+                const int lr = p * 4 + rr;
+                const v4f v = *(const v4f*)(stg + lr * 256 + ((ch ^ (lr & 15)) * 16));
+                const int r = sub_row(lr >> 4) + (lr & 15);
+                const int n = n0 + grp * WN + h * (WN / 2) + ch * 4;
+                if (r < rows_here && n < N)
+                    *(v4f*)(c + (size_t)(m0 + r) * ldc + (n - n_base)) = v;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        const int r = sub_row(j) + fr;
+        if (r >= rows_here) continue;
+        const int m = m0 + r;
+#pragma unroll
+        for (int i = 0; i < SN; ++i) {
+            const int n = n0 + grp * WN + i * 16 + fq * 4;
+            typename OutT<CD>::type* dst = c + (size_t)m * ldc + (n - n_base);
+            if (vec_ok && n + 3 < N) {
+                if (CD == DSV3_F32) {
+                    *(v4f*)dst = acc[i][j];
+                } else if (CD == DSV3_BF16) {
+                    v2u o = { pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3]) };
+                    *(v2u*)dst = o;
+                } else {
+                    v2u o = { pack_f16(acc[i][j][0], acc[i][j][1]), pack_f16(acc[i][j][2], acc[i][j][3]) };
+                    *(v2u*)dst = o;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) dst[e] = cvt_out<CD>(acc[i][j][e]);
+            }
+        }
+    }
+}
+
+}  // namespace pingpong

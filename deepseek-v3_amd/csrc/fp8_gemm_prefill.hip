@@ -560,6 +560,19 @@ __device__ __forceinline__ void prefill_tile(
     }
 }
 
+#include "fp8_gemm_pingpong.hpp"
+
+inline bool use_pingpong() { static const bool v = getenv("DSV3_PREFILL_NOPP") == nullptr; return v; }
+
+template <int CD, bool P2 = false>
+__global__ __launch_bounds__(THREADS, 1) void fp8_gemm_pingpong_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c,
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc) {
+    pingpong::tile<CD, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x);
+}
+
 template <int CD, bool G, int TM, int S, bool P2 = false>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
@@ -596,7 +609,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
 // tiles over the column tiles [0, tn_tall), the others 128-row tiles over [tn_tall, tn_tall + tn_short).  Workgroups
 // are handed out in index order, so the short tiles fill the compute units that the last, partly filled round of
 // tall tiles would leave idle.
-template <int CD, bool P2 = false>
+template <int CD, bool P2 = false, bool PP = true>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_two_heights_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -604,9 +617,10 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_two_heights_kernel(
     const int tm_tall = (M + 255) / 256, n_tall = tm_tall * tn_tall;
     const int short_first = (n_tall + 7) & ~7;        // keeps workgroup index % 8 = XCD for the short tiles too
     const GroupTable none{};
-    if ((int)blockIdx.x < n_tall)
-        prefill_tile<CD, false, 256, 2, 2, P2>(a, a_s, b, b_s, c, M, N, K, tm_tall, tn_tall, 0, K / 128, N, none, blockIdx.x);
-    else if ((int)blockIdx.x >= short_first)
+    if ((int)blockIdx.x < n_tall) {
+        if constexpr (PP) pingpong::tile<CD, P2>(a, a_s, b, b_s, c, M, N, K, tm_tall, tn_tall, 0, K / 128, N, blockIdx.x);
+        else prefill_tile<CD, false, 256, 2, 2, P2>(a, a_s, b, b_s, c, M, N, K, tm_tall, tn_tall, 0, K / 128, N, none, blockIdx.x);
+    } else if ((int)blockIdx.x >= short_first)
         prefill_tile<CD, false, 128, 3, 3, P2>(a, a_s, b, b_s, c, M, N, K, (M + 127) / 128, tn_short, tn_tall, K / 128, N, none,
                                         blockIdx.x - short_first);
 }
@@ -628,10 +642,27 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
     constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
     if ((tm + 8) * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (tm * tn_count == 0) return DSV3_OK;
-    auto kern = fp8_gemm_prefill_kernel<CD, G, TM, S, P2>;
-    static bool granted[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
+    if constexpr (!G && TM == 256) {
+        if (use_pingpong()) {
+            auto pp = fp8_gemm_pingpong_kernel<CD, P2>;
+            static bool pp_granted[64] = {};
+            if (!pp_granted[dev]) {
+                if (hipFuncSetAttribute((const void*)pp, hipFuncAttributeMaxDynamicSharedMemorySize, pingpong::LDS_BYTES) != hipSuccess)
+                    return DSV3_ERR_LAUNCH;
+                pp_granted[dev] = true;
+            }
+            const int kbt = (int)(k / 128), per = (kbt + splits - 1) / splits;
+            hipLaunchKernelGGL(pp, dim3((unsigned)(tm * tn_count), (unsigned)((kbt + per - 1) / per)), dim3(THREADS),
+                               pingpong::LDS_BYTES, stream, (const uint8_t*)a, a_s, (const uint8_t*)b, b_s,
+                               (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)tm, (int)tn_count, (int)tn_first,
+                               per, (int)(ldc ? ldc : n));
+            return launch_status();
+        }
+    }
+    auto kern = fp8_gemm_prefill_kernel<CD, G, TM, S, P2>;
+    static bool granted[64] = {};
     if (!granted[dev]) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
             return DSV3_ERR_LAUNCH;
@@ -782,15 +813,17 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
     const prefill::GroupTable none{};
     if (p.tn_short > 0) {
         using namespace prefill;
-        constexpr int LDS_BYTES = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
-        auto kern = fp8_gemm_two_heights_kernel<CD, P2>;
-        static bool granted[64] = {};
+        constexpr int LDS_OLD = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
+        constexpr int LDS_BYTES = LDS_OLD > pingpong::LDS_BYTES ? LDS_OLD : pingpong::LDS_BYTES;
+        const bool pp = use_pingpong();
+        auto kern = pp ? fp8_gemm_two_heights_kernel<CD, P2, true> : fp8_gemm_two_heights_kernel<CD, P2, false>;
+        static bool granted[2][64] = {};
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
-        if (!granted[dev]) {
+        if (!granted[pp][dev]) {
             if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
                 return DSV3_ERR_LAUNCH;
-            granted[dev] = true;
+            granted[pp][dev] = true;
         }
         const int64_t n_tall = (m + 255) / 256 * p.tn_plain;
         const int64_t grid = (n_tall + 7) / 8 * 8 + (m + 127) / 128 * p.tn_short;
