@@ -39,6 +39,59 @@ SETTLE_S = 0.15                # untimed run of the step before the warm-up step
 METRIC = "fp8_gemm TFLOP/s & %fp8 MFMA peak @M=4096; decode-GEMM HBM GB/s @M=1-64"
 
 
+class Probes:
+    """libdsv3probe.so: kernels of known traffic / arithmetic (read stream, copy, fp8 MFMA loop, empty launch) that
+    give the ceilings this GPU sustains.  Measurement infrastructure only."""
+
+    def __init__(self):
+        import ctypes as C
+        path = ROOT / "deepseek-v3_amd" / "lib" / "libdsv3probe.so"
+        if not path.exists():
+            sys.exit(f"bench.py: {path} is missing; run `python deepseek-v3_amd/build.py`.")
+        L = self.lib = C.CDLL(str(path))
+        L.dsv3_probe_read_stream.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
+        L.dsv3_probe_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+        L.dsv3_probe_mfma.argtypes = [C.c_int, C.c_void_p, C.c_void_p]
+        L.dsv3_probe_mfma_flops.restype = C.c_double
+        L.dsv3_probe_mfma_flops.argtypes = [C.c_int]
+        L.dsv3_probe_null.argtypes = [C.c_void_p]
+        self.sink = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
+        self.pool = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device="cuda")      # 1 GiB of random bytes
+
+    @staticmethod
+    def _st():
+        return torch.cuda.current_stream().cuda_stream
+
+    def read(self, offset: int, nbytes: int):
+        rc = self.lib.dsv3_probe_read_stream(self.pool.data_ptr() + offset, nbytes, self.sink.data_ptr(), 0, self._st())
+        assert rc == 0
+
+    def read_stream_us(self, nbytes: int) -> float:
+        """Microseconds per launch of a plain read stream over `nbytes` contiguous bytes, rotating through the pool
+        like the decode sweep rotates its weights (HIP graph, back-to-back launches)."""
+        nbytes = nbytes // 4096 * 4096
+        copies = max(2, min(160, (1 << 30) // nbytes, -(-640_000_000 // nbytes)))
+        launches = [(lambda i=i: self.read(i * nbytes, nbytes)) for i in range(copies)]
+        if len(launches) < 40:
+            launches = launches * (-(-40 // len(launches)))
+        return time_graph(launches)
+
+    def ceilings(self) -> dict:
+        n = self.pool.numel()
+        dst = torch.empty_like(self.pool)
+        rd = time_graph([lambda: self.read(0, n)] * 4)
+        cp = time_graph([lambda: self.lib.dsv3_probe_copy(self.pool.data_ptr(), dst.data_ptr(), n, 0, self._st())] * 4)
+        del dst
+        iters = 2000
+        mf = time_graph([lambda: self.lib.dsv3_probe_mfma(iters, self.sink.data_ptr(), self._st())] * 10)
+        nl = time_graph([lambda: self.lib.dsv3_probe_null(self._st())] * 100)
+        return {"hbm_read_stream_GBps": round(n / rd / 1e3, 1), "hbm_copy_GBps": round(2 * n / cp / 1e3, 1),
+                "fp8_mfma_loop_TFLOPs": round(self.lib.dsv3_probe_mfma_flops(iters) / mf / 1e6, 1),
+                "empty_launch_us": round(nl, 2),
+                "note": "measured on this GPU in this run: 1 GiB read stream; 1 GiB copy (bytes read + written); "
+                        "registers-only v_mfma_f32_16x16x128_f8f6f4 loop, 8 wavefronts per CU; empty kernel in a graph"}
+
+
 def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
@@ -108,24 +161,28 @@ def decode_bytes(m, n, k):
     return n * k + 4 * (-(-n // 128)) * (k // 128) + m * k + 4 * m * (k // 128) + 2 * m * n
 
 
-def run_extras(K, W):
+def _bw(nbytes: float, us: float, ceil_gbps: float) -> dict:
+    gbs = nbytes / us / 1e3
+    return {"us": round(us, 2), "GBps": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 3),
+            "frac_of_measured_copy": round(gbs / ceil_gbps, 3)}
+
+
+def run_extras(K, W, probes, ceil):
     out = {}
+    copy_c, read_c = ceil["hbm_copy_GBps"], ceil["hbm_read_stream_GBps"]
     x = W.activations(4096, 7168, 0, "cuda", outliers=True)
     xs = [x.clone() for _ in range(12)]                       # 12 x 58.7 MB > Infinity Cache
     us = time_graph([(lambda t=t: K.act_quant(t)) for t in xs] * 2)
-    out["act_quant_4096x7168"] = {"us": round(us, 2), "GBps": round(88.998e6 / us / 1e3, 1),
-                                  "hbm_frac": round(88.998e6 / us / 1e3 / HBM_PEAK_GBS, 3)}
+    out["act_quant_4096x7168"] = _bw(88.998e6, us, copy_c)
     del xs
     w8, s = W.random_fp8_weight(18432, 7168, 2, "cuda")
     ws_ = [w8.clone() for _ in range(5)]
     us = time_graph([(lambda t=t: K.weight_dequant(t, s)) for t in ws_] * 2)
-    out["weight_dequant_18432x7168"] = {"us": round(us, 2), "GBps": round(396.394e6 / us / 1e3, 1),
-                                        "hbm_frac": round(396.394e6 / us / 1e3 / HBM_PEAK_GBS, 3)}
+    out["weight_dequant_18432x7168"] = _bw(396.394e6, us, copy_c)
     del ws_, w8
     wb = [(torch.randn(18432, 7168, device="cuda") * 0.02).bfloat16() for _ in range(4)]   # 4 x 264 MB
     us = time_graph([(lambda t=t: K.weight_quant(t)) for t in wb] * 2)
-    out["weight_quant_18432x7168"] = {"us": round(us, 2), "GBps": round(396.394e6 / us / 1e3, 1),
-                                      "hbm_frac": round(396.394e6 / us / 1e3 / HBM_PEAK_GBS, 3)}
+    out["weight_quant_18432x7168"] = _bw(396.394e6, us, copy_c)
     del wb
     k, n = W.PREFILL_SHAPES["w2"]
     a, a_s = K.act_quant(W.activations(4096, k, 0, "cuda"))
@@ -146,10 +203,11 @@ def run_extras(K, W):
                                                 "mfma_frac": round(tf / FP8_MFMA_PEAK_TFLOPS, 3)}
     del a, a_s, wq, wsc, a2, a2_s, wsc2
     dec = {}
-    for name, (k, n) in W.DECODE_SHAPES.items():
+    for name, (k, n) in W.DECODE_SWEEP.items():
         wq, wsc = W.weight(n, k, 1, "cuda")
         copies = max(2, min(160, -(-640_000_000 // (n * k))))
         wqs = [wq.clone() for _ in range(copies)]
+        floor_us = probes.read_stream_us(n * k)               # a plain read stream over as many bytes as the weight
         for m in W.DECODE_M:
             a, a_s = K.act_quant(W.activations(m, k, m, "cuda"))
             launches = [(lambda t=t: K.fp8_gemm(a, a_s, t, wsc)) for t in wqs]
@@ -158,7 +216,9 @@ def run_extras(K, W):
             us = time_graph(launches)
             gbs = decode_bytes(m, n, k) / us / 1e3
             dec[f"{name}_{k}to{n}_M{m}"] = {"us": round(us, 2), "GBps": round(gbs, 1),
-                                            "hbm_frac": round(gbs / HBM_PEAK_GBS, 3)}
+                                            "hbm_frac": round(gbs / HBM_PEAK_GBS, 3),
+                                            "frac_of_measured_read": round(gbs / read_c, 3),
+                                            "read_stream_same_bytes_us": round(floor_us, 2)}
         del wqs
     out["decode"] = dec
     # linear() at decode sizes: act_quant + fp8_gemm as two launches against the fused single launch
@@ -183,6 +243,25 @@ def run_extras(K, W):
     out["moe_layer_T4096_balanced"] = run_moe(K, W, bias_std=0.0, expert_loop=False)
     out["wkv_b_absorb"] = run_absorb(K, W)
     return out
+
+
+def decode_roofline(dec: dict, ceil: dict) -> dict:
+    """The metric's second half in one block: the decode sweep (M = 1, 8, 32, 64 over the MLA projections) as HBM
+    fractions of its algorithmic bytes, against the 8 TB/s peak and against this GPU's measured read stream."""
+    import math
+    fr = [v["hbm_frac"] for v in dec.values()]
+    worst = min(dec, key=lambda k_: dec[k_]["hbm_frac"])
+    best = max(dec, key=lambda k_: dec[k_]["hbm_frac"])
+    geo = math.exp(sum(math.log(f) for f in fr) / len(fr))
+    return {"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s", "cells": len(fr),
+            "kernels": ["fp8_gemm_skinny_kernel (M <= 16)", "fp8_gemm_stream_kernel (M = 32, 64)",
+                        "fp8_gemm_prefill / pingpong kernel, K sliced (M >= 9 on weights >= 96 MiB)",
+                        "skinny_single kernel (M = 3..16 on weights >= 96 MiB)"],
+            "bytes": "N*K + 4*ceil(N/128)*(K/128) + M*K + 4*M*K/128 + 2*M*N per launch",
+            "frac_min": min(fr), "frac_min_cell": worst, "frac_max": max(fr), "frac_max_cell": best,
+            "frac_geomean": round(geo, 3),
+            "frac_geomean_of_measured_read": round(geo * HBM_PEAK_GBS / ceil["hbm_read_stream_GBps"], 3),
+            "measured_read_stream_GBps": ceil["hbm_read_stream_GBps"]}
 
 
 def run_absorb(K, W, token_counts=(1, 16, 64, 128, 4096)):
@@ -258,6 +337,8 @@ def run_moe(K, W, tokens: int = 4096, bias_std: float = 0.1, expert_loop: bool =
                             "weight_stream_GBps": round(wbytes / ms / 1e6, 1),
                             "mfma_frac": round(flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 4),
                             "hbm_frac": round(wbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            Mdl.MoE.grouped = True
+            res["grouped_stages_us"] = moe_stages(moe, x, Mdl)
             if expert_loop:                  # decode sizes on the same layer, one captured forward each
                 Mdl.MoE.grouped = True
                 dec = {}
@@ -274,6 +355,33 @@ def run_moe(K, W, tokens: int = 4096, bias_std: float = 0.1, expert_loop: bool =
         return res
     finally:
         Mdl.gemm_impl, Mdl.Linear.dtype, Mdl.MoE.grouped = old
+
+
+def moe_stages(moe, x, Mdl):
+    """Microseconds of each launch group of MoE._forward_grouped on fixed inputs, timed one stage at a time (same
+    ops, same arguments, same order as the layer issues them)."""
+    ops, bs = Mdl.ops, Mdl.block_size
+    w13, s13, w2, s2 = (t[:moe.n_routed_experts] for t in moe._stacked)
+    code = ops.dtype_code(torch.get_default_dtype())
+    st = {}
+
+    def t(name, fn, steps=10):
+        st[name] = round(time_loop(fn, steps, 2) * 1e3, 1)
+        return fn()
+    weights, indices = t("gate", lambda: moe.gate(x))
+    route = t("moe_route", lambda: torch.ops.dsv3fp8.moe_route(indices.contiguous(), weights.contiguous(),
+                                                                 moe.n_routed_experts, False))
+    _, a_rows, rows, w_sorted, tile_group, tile_row0, tile_rows = route
+    pairs = rows.numel()
+    xq, xs = t("act_quant", lambda: Mdl.act_quant(x, bs, None))
+    g = torch.ops.dsv3fp8.fp8_gemm_grouped
+    h = t("grouped_w1w3", lambda: g(xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, code))
+    gq, gs = t("swiglu_quant", lambda: torch.ops.dsv3fp8.swiglu_quant(h, bs, 0))
+    out = t("grouped_w2", lambda: g(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code))
+    z = t("shared_expert", lambda: moe.shared_experts(x).contiguous())
+    t("moe_combine", lambda: torch.ops.dsv3fp8.moe_combine(out, rows, w_sorted, z))
+    st["sum"] = round(sum(st.values()), 1)
+    return st
 
 
 def cpu_baseline(W, rows: int = 1024):
@@ -353,6 +461,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    probes = Probes()
+    ceil = probes.ceilings()
     line = {
         "metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "settle_ms": int(SETTLE_S * 1e3), "ms_per_step": round(ms, 4),
@@ -364,12 +474,15 @@ def main():
         "roofline": {"kernel": "fp8_gemm_two_heights_kernel", "bound": "mfma", "achieved": round(achieved, 2),
                      "peak": FP8_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4), "traffic": measured_traffic(),
-                     "launch_us": round(gemm_ms * 1e3, 2), "flops_per_launch": flops},
+                     "launch_us": round(gemm_ms * 1e3, 2), "flops_per_launch": flops,
+                     "frac_of_measured_mfma_loop": round(achieved / ceil["fp8_mfma_loop_TFLOPs"], 4)},
+        "ceilings": ceil,
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(W)
     if not args.no_extras:
-        line["extras"] = run_extras(K, W)
+        line["extras"] = run_extras(K, W, probes, ceil)
+        line["roofline_decode"] = decode_roofline(line["extras"]["decode"], ceil)
     print(json.dumps(line), flush=True)
 
 

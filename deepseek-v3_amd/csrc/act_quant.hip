@@ -50,19 +50,23 @@ template <> struct In<DSV3_F32> {
     }
 };
 
-template <int CTRL> __device__ __forceinline__ float dpp_max(float v) {
-    int o = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
-    return fmaxf(v, __builtin_bit_cast(float, o));
+// The block maximum is taken over the bit patterns of |x| as unsigned integers: for finite values and infinity that
+// is the order of the values, and a NaN (exponent all ones, mantissa non-zero) is larger than everything, so it
+// reaches the scale the way torch's amax and the reference's tl.max let it (v_max_f32 would drop it).
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_max(uint32_t v) {
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+    return umax(v, o);
 }
 
 // max over the LPB lanes that share a block; every lane ends with the result.
-template <int LPB> __device__ __forceinline__ float group_max(float v) {
+template <int LPB> __device__ __forceinline__ uint32_t group_max(uint32_t v) {
     if (LPB >= 2) v = dpp_max<0xB1>(v);    // quad_perm [1,0,3,2]
     if (LPB >= 4) v = dpp_max<0x4E>(v);    // quad_perm [2,3,0,1]
     if (LPB >= 8) v = dpp_max<0x141>(v);   // row_half_mirror
     if (LPB >= 16) v = dpp_max<0x140>(v);  // row_mirror
-    if (LPB >= 32) v = fmaxf(v, __shfl_xor(v, 16));
-    if (LPB >= 64) v = fmaxf(v, __shfl_xor(v, 32));
+    if (LPB >= 32) v = umax(v, (uint32_t)__shfl_xor((int)v, 16));
+    if (LPB >= 64) v = umax(v, (uint32_t)__shfl_xor((int)v, 32));
     return v;
 }
 
@@ -84,19 +88,21 @@ __global__ __launch_bounds__(kThreads) void act_quant_kernel(
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int64_t c = base + (int64_t)u * kThreads;
-        float amax = 0.f;
+        uint32_t abits = 0u;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(f[u][i]));
-        amax = group_max<LPB>(amax);
-        amax = fmaxf(amax, 1e-4f);
-        float sc = amax / 448.f;
+        for (int i = 0; i < 8; ++i) abits = umax(abits, f32_as_u32(f[u][i]) & 0x7fffffffu);
+        abits = group_max<LPB>(abits);
+        const bool finite = abits < 0x7f800000u;                 // the same for all lanes of the block
+        // infinity gives s = inf (finite elements quantise to 0, infinite ones to NaN), NaN gives s = NaN and a block
+        // of NaN codes: what the IEEE evaluation of the formula gives
+        float sc = abits > 0x7f800000u ? u32_as_f32(0x7fc00000u) : fmaxf(u32_as_f32(abits), 1e-4f) / 448.f;
         if (UE8M0) {
             uint32_t b = f32_as_u32(sc);
             b = ((b >> 23) + ((b & 0x7fffffu) ? 1u : 0u)) << 23;
             sc = u32_as_f32(b);
         }
         float q[8];
-        if (XD == DSV3_BF16) {
+        if (XD == DSV3_BF16 && finite) {
             const float r = 1.0f / sc;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {

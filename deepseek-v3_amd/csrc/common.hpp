@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
+#include <atomic>
 #include "../../include/dsv3_fp8.h"
 
 namespace dsv3 {
@@ -61,6 +62,21 @@ template <> __device__ __forceinline__ uint16_t cvt_out<DSV3_F16>(float v)  { re
 template <> __device__ __forceinline__ float    cvt_out<DSV3_F32>(float v)  { return v; }
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? DSV3_OK : DSV3_ERR_LAUNCH; }
+
+// More than 64 KiB of dynamic LDS has to be granted to a kernel once per device.  One LdsGrant per kernel (a
+// function-local static); the per-device flags are atomics, so concurrent first calls from several threads are
+// well defined (they may both make the idempotent attribute call).  Returns false when HIP refuses.
+struct LdsGrant {
+    std::atomic<bool> done[64];
+    bool ensure(const void* kernel, int bytes) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+        if (done[dev].load(std::memory_order_acquire)) return true;
+        if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+        done[dev].store(true, std::memory_order_release);
+        return true;
+    }
+};
 
 // Entry points of the individual kernel families (defined in the .hip files).
 int launch_act_quant(const void* x, int x_dtype, void* y, float* s, int64_t numel,

@@ -240,6 +240,7 @@ __device__ __forceinline__ void tile(
             __builtin_amdgcn_sched_barrier(0);
         };
 
+        PP_PROF_DECL
         // one K block whose LDS stage (and scale slot) ST is a compile-time constant: every LDS address of the loop is
         // a register plus an immediate
         auto block = [&](int kb, auto st_tag) {
@@ -302,7 +303,6 @@ __device__ __forceinline__ void tile(
             PP_PROF_MARK(7)
         };
 
-        PP_PROF_DECL
         int kb = 0;
         for (; kb + 1 < KB; kb += 2) {
             block(kb, std::integral_constant<int, 0>{});

@@ -642,17 +642,11 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
     constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
     if ((tm + 8) * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (tm * tn_count == 0) return DSV3_OK;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
     if constexpr (!G && TM == 256) {
         if (use_pingpong()) {
             auto pp = fp8_gemm_pingpong_kernel<CD, P2>;
-            static bool pp_granted[64] = {};
-            if (!pp_granted[dev]) {
-                if (hipFuncSetAttribute((const void*)pp, hipFuncAttributeMaxDynamicSharedMemorySize, pingpong::LDS_BYTES) != hipSuccess)
-                    return DSV3_ERR_LAUNCH;
-                pp_granted[dev] = true;
-            }
+            static LdsGrant pp_grant;
+            if (!pp_grant.ensure((const void*)pp, pingpong::LDS_BYTES)) return DSV3_ERR_LAUNCH;
             const int kbt = (int)(k / 128), per = (kbt + splits - 1) / splits;
             hipLaunchKernelGGL(pp, dim3((unsigned)(tm * tn_count), (unsigned)((kbt + per - 1) / per)), dim3(THREADS),
                                pingpong::LDS_BYTES, stream, (const uint8_t*)a, a_s, (const uint8_t*)b, b_s,
@@ -662,12 +656,8 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
         }
     }
     auto kern = fp8_gemm_prefill_kernel<CD, G, TM, S, P2>;
-    static bool granted[64] = {};
-    if (!granted[dev]) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-            return DSV3_ERR_LAUNCH;
-        granted[dev] = true;
-    }
+    static LdsGrant grant;
+    if (!grant.ensure((const void*)kern, LDS_BYTES)) return DSV3_ERR_LAUNCH;
     const int64_t grid = (G ? (tm + 7) / 8 * 8 : tm) * tn_count;       // grouped: row tiles are dealt over the 8 XCDs
     const int kb = (int)(k / 128), kb_per_split = (kb + splits - 1) / splits;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)((kb + kb_per_split - 1) / kb_per_split)), dim3(THREADS),
@@ -749,7 +739,7 @@ PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
     auto slab_cost = [&](int64_t slabs, int64_t cols) { return 300 + slabs * m * cols * 12 / 100000; };
     for (int h : {128, 256}) {
         if (forced && forced != h) continue;
-        const int64_t unit = h == 128 ? 100 : 164, tm = (m + h - 1) / h, tiles = tm * tn;
+        const int64_t unit = h == 128 ? 100 : (prefill::use_pingpong() ? 152 : 164), tm = (m + h - 1) / h, tiles = tm * tn;
         // plain or sliced over all columns
         {
             const int64_t s = slices_for(tiles), per = (kb + s - 1) / s, slabs = (kb + per - 1) / per;
@@ -778,9 +768,10 @@ PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
         for (int64_t c = 1; c < tn && c <= 32; ++c) {
             const int64_t n_tall = tm_tall * (tn - c), n_short = tm_short * c;
             const int64_t q = n_tall / kCUs, r = n_tall % kCUs;
-            // kCUs - r units carry lo = q * 164, r units hi = lo + 164; the short tiles (100 each) go to whichever
+            // kCUs - r units carry lo = q * tall, r units hi = lo + tall; the short tiles (100 each) go to whichever
             // unit is free first, level by level
-            const int64_t lo = q * 164, hi = lo + 164;
+            const int64_t tall = prefill::use_pingpong() ? 152 : 164;
+            const int64_t lo = q * tall, hi = lo + tall;
             int64_t t = lo, t_lo = lo + 100, t_hi = hi + 100, done = 0;
             while (done < n_short) {
                 if (r == 0 || t_lo <= t_hi) { t = t_lo; t_lo += 100; done += kCUs - r; }
@@ -817,14 +808,8 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
         constexpr int LDS_BYTES = LDS_OLD > pingpong::LDS_BYTES ? LDS_OLD : pingpong::LDS_BYTES;
         const bool pp = use_pingpong();
         auto kern = pp ? fp8_gemm_two_heights_kernel<CD, P2, true> : fp8_gemm_two_heights_kernel<CD, P2, false>;
-        static bool granted[2][64] = {};
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
-        if (!granted[pp][dev]) {
-            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-                return DSV3_ERR_LAUNCH;
-            granted[pp][dev] = true;
-        }
+        static LdsGrant grant[2];
+        if (!grant[pp].ensure((const void*)kern, LDS_BYTES)) return DSV3_ERR_LAUNCH;
         const int64_t n_tall = (m + 255) / 256 * p.tn_plain;
         const int64_t grid = (n_tall + 7) / 8 * 8 + (m + 127) / 128 * p.tn_short;
         if (grid > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
@@ -880,14 +865,8 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
     if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (num_tiles * tn == 0) return DSV3_OK;
     auto kern = fp8_gemm_grouped_kernel<CD, P2>;
-    static bool granted[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
-    if (!granted[dev]) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-            return DSV3_ERR_LAUNCH;
-        granted[dev] = true;
-    }
+    static LdsGrant grant;
+    if (!grant.ensure((const void*)kern, LDS_BYTES)) return DSV3_ERR_LAUNCH;
     const int64_t grid = (num_tiles + 7) / 8 * 8 * tn;                  // row tiles are dealt over the 8 XCDs
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
                        (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)num_tiles,

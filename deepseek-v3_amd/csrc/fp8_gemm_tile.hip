@@ -222,16 +222,8 @@ int launch_cfg(const void* a, const float* a_s, const void* b, const float* b_s,
     if (tm * tn > 0x7fffffff || splits > 65535) return DSV3_ERR_BAD_SHAPE;
     auto kern = fp8_gemm_tile_kernel<BM, BN, WM, WN, CD>;
     constexpr int lds_bytes = 2 * (BM + BN) * kRowStride;
-    // more than the default 64 KiB of dynamic LDS has to be granted once per device;
-    // the flag is idempotent, so a race between threads only repeats the same call
-    static bool granted[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
-    if (!granted[dev]) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-            return DSV3_ERR_LAUNCH;
-        granted[dev] = true;
-    }
+    static LdsGrant grant;                   // more than the default 64 KiB of dynamic LDS
+    if (!grant.ensure((const void*)kern, lds_bytes)) return DSV3_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn), (unsigned)splits), dim3((BM / WM) * (BN / WN) * kWave), lds_bytes, stream,
                        (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c,
                        (int)m, (int)n, (int)k, (int)tm, (int)tn, kb_per_split);

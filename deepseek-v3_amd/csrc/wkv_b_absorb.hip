@@ -398,15 +398,8 @@ int launch_wkv_b_absorb(const void* x, int64_t x_ts, int64_t x_hs, const void* w
     const dim3 grid(gx, heads, gz), block(64 * waves);
     if (!q && kv_rank == 512 && v % 128 == 0 && waves == 4) {
         constexpr int S = 4;
-        static bool granted[64];                 // 64 KiB of dynamic LDS needs the opt-in once per device
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DSV3_ERR_LAUNCH;
-        if (!granted[dev]) {
-            if (hipFuncSetAttribute((const void*)absorb_v_staged_kernel<S>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    S * kStagedStage) != hipSuccess)
-                return DSV3_ERR_LAUNCH;
-            granted[dev] = true;
-        }
+        static LdsGrant grant;                   // 64 KiB of dynamic LDS needs the opt-in once per device
+        if (!grant.ensure((const void*)absorb_v_staged_kernel<S>, S * kStagedStage)) return DSV3_ERR_LAUNCH;
         hipLaunchKernelGGL(absorb_v_staged_kernel<S>, grid, block, S * kStagedStage, st, p);
         return launch_status();
     }

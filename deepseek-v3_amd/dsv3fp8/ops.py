@@ -55,6 +55,11 @@ _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
 def _workspace(t: torch.Tensor, nbytes: int, stream: int) -> torch.Tensor:
+    # Under stream capture the scratch comes from the graph's own memory pool and lives as long as the graph: the
+    # cached buffer below is replaced when a larger one is needed, which would leave a graph that had captured it
+    # replaying into freed memory.
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(nbytes, dtype=torch.uint8, device=t.device)
     key = (t.device.index, stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:

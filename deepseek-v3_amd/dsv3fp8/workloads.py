@@ -24,6 +24,9 @@ DECODE_SHAPES = {
     "wkv_b": (512, 32768),
     "wo": (16384, 7168),
 }
+# the sweep the benchmark times: the five projections plus wq_a and wkv_a as the one stacked GEMM that the attention
+# layer launches for them (both read the same input; model.py:424-427)
+DECODE_SWEEP = dict(DECODE_SHAPES, wq_a_wkv_a_stacked=(7168, 2112))
 DECODE_M = (1, 8, 32, 64)
 # dense MLP projections for the prefill case (K -> N), M = 4096 tokens
 PREFILL_SHAPES = {"w1": (7168, 18432), "w2": (18432, 7168)}

@@ -131,3 +131,31 @@ def test_full_size_properties(K):
     mag = (y.view(torch.uint8) & 0x7F).view(4096, 56, 128)
     assert int(mag.max()) == 0x7E
     assert bool((mag.amax(-1) == 0x7E).all())
+
+
+def test_non_finite_inputs_follow_the_ieee_evaluation(K):
+    """NaN and infinity in the activations (inference/kernel.py:26-33 with tl.max / torch.amax, which propagate NaN):
+    a block with a NaN gets s = NaN and NaN codes everywhere, a block with an infinity s = inf, zeros for the finite
+    elements and NaN codes for the infinite ones; blocks beside them are untouched.  Held against oracle.act_quant
+    (NaN codes are compared as "is a NaN code": 0x7f and 0xff differ only in the sign of the NaN)."""
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(6, 512, generator=g).bfloat16()
+    x[0, 5] = float("nan")                      # block (0, 0)
+    x[1, 130] = float("inf")                    # block (1, 1)
+    x[2, 300] = float("-inf"); x[2, 301] = 7.0  # block (2, 2)
+    x[3, 10] = float("nan"); x[3, 11] = float("inf")   # NaN wins over infinity
+    x[4, 384:512] = 0                           # an all-zero block beside normal ones
+    yr, sr = oracle.act_quant(x)
+    y, s = K.act_quant(x.cuda())
+    y, s = y.cpu().view(torch.uint8), s.cpu()
+    yr = yr.view(torch.uint8)
+    assert torch.equal(torch.isnan(s), torch.isnan(sr)) and torch.equal(torch.isinf(s), torch.isinf(sr))
+    ok = torch.isfinite(sr)
+    assert torch.equal(s[ok], sr[ok])
+    nan_ref, nan_got = (yr & 0x7F) == 0x7F, (y & 0x7F) == 0x7F
+    assert torch.equal(nan_ref, nan_got)
+    assert torch.equal(y[~nan_ref], yr[~nan_ref])
+    assert bool(nan_got[0, :128].all()) and not bool(nan_got[0, 128:].any())
+    assert bool(torch.isinf(s[1, 1])) and int(nan_got[1].sum()) == 1 and bool(nan_got[1, 130])
+    assert int(((y[1, 128:256] & 0x7F) != 0).sum()) == 1                # finite / inf = a zero of either sign
+    assert bool(torch.isnan(s[3, 0])) and bool(nan_got[3, :128].all())

@@ -189,6 +189,57 @@ def test_prefill_sampled(K):
     assert torch.equal(c16.view(torch.int16), c32.to(torch.bfloat16).view(torch.int16))
 
 
+def _sampled_reference(a, a_s, w8, ws, rows, col_blocks):
+    """oracle.fp8_gemm_f32 on the sampled rows of a and whole 128-row blocks of b (the oracle needs whole scale
+    blocks); returns the reference and the column indices it covers."""
+    ref = torch.cat([oracle.fp8_gemm_f32(a[rows].cpu(), a_s[rows].cpu(), w8[b * 128:(b + 1) * 128].cpu(),
+                                         ws[b:b + 1].cpu()) for b in col_blocks], 1)
+    cols = torch.cat([torch.arange(b * 128, (b + 1) * 128) for b in col_blocks])
+    return ref, cols
+
+
+def test_prefill_w2_sampled(K):
+    """The second half of the prefill configuration at full size: M=4096, 18432 -> 7168 (448 tall tiles, 1.75
+    rounds, 144 K blocks); the oracle evaluates a sample of rows and column blocks."""
+    from dsv3fp8 import workloads
+    x = workloads.activations(4096, 18432, seed=2, device="cuda")
+    w8, ws = workloads.weight(7168, 18432, seed=3, device="cuda")
+    a, a_s = K.act_quant(x)
+    c32, c16 = _gemm_both(K, a, a_s, w8, ws)
+    rows = torch.cat([torch.arange(3, 4096, 211), torch.tensor([0, 255, 256, 4095])]).cuda()
+    ref, cols = _sampled_reference(a, a_s, w8, ws, rows, [0, 1, 27, 28, 55])
+    got = c32[rows][:, cols.cuda()].cpu()
+    rms = ref.pow(2).mean().sqrt().item()
+    assert (got - ref).abs().max().item() <= TOL * rms
+    assert torch.equal(c16.view(torch.int16), c32.to(torch.bfloat16).view(torch.int16))
+
+
+def test_prefill_pow2_full_size_sampled(K):
+    """fp8_gemm_pow2 at M=4096 on both prefill shapes: power-of-two activation scales (ue8m0) and weight block scales
+    rounded up to powers of two; sampled against the oracle and held against the general kernel everywhere."""
+    from dsv3fp8 import workloads
+    for (k, n, blocks) in ((7168, 18432, [0, 70, 143]), (18432, 7168, [0, 31, 55])):
+        x = workloads.activations(4096, k, seed=k % 13, device="cuda")
+        w8, ws = workloads.weight(n, k, seed=4, device="cuda")
+        ws2 = torch.pow(2.0, torch.ceil(torch.log2(ws)))            # the bytes stay, the scales move up to 2^e
+        a, a_s = K.act_quant(x, 128, "ue8m0")
+        old = torch.get_default_dtype()
+        try:
+            torch.set_default_dtype(torch.float32)
+            c32 = K.fp8_gemm_pow2(a, a_s, w8, ws2)
+            gen = K.fp8_gemm(a, a_s, w8, ws2)
+            torch.set_default_dtype(torch.bfloat16)
+            c16 = K.fp8_gemm_pow2(a, a_s, w8, ws2)
+        finally:
+            torch.set_default_dtype(old)
+        rows = torch.arange(7, 4096, 307).cuda()
+        ref, cols = _sampled_reference(a, a_s, w8, ws2, rows, blocks)
+        rms = ref.pow(2).mean().sqrt().item()
+        assert (c32[rows][:, cols.cuda()].cpu() - ref).abs().max().item() <= TOL * rms
+        assert (c32 - gen).abs().max().item() <= 1e-4 * rms
+        assert torch.equal(c16.view(torch.int16), c32.to(torch.bfloat16).view(torch.int16))
+
+
 def test_asserts_match_reference(K):
     a = torch.zeros(4, 256, dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn)
     a_s = torch.ones(4, 2, device="cuda")

@@ -407,3 +407,95 @@ def test_moe_forward_is_graph_capturable(K):
     finally:
         M.gemm_impl, M.Linear.dtype = old[0], old[2]
         torch.set_default_dtype(old[1])
+
+
+# ---- the mixture-of-experts configuration at its full dimensions (256 + 1 experts, 7168 -> 2048 -> 7168, 4096 tokens)
+
+@pytest.mark.parametrize("k,n", [(7168, 4096), (2048, 7168)])        # w1|w3 stacked and w2 of one expert
+def test_fp8_gemm_grouped_tile_kernel_full_dimensions(K, k, n):
+    """The grouped TILE kernel (more than 320 rows in all) on the two GEMM shapes of the layer: groups of about 128
+    rows, one of 1093 rows (five tile slots), an empty one and a 131- and a 200-row one (the 192-row
+    configuration).  The oracle evaluates sampled groups on sampled rows and whole 128-column blocks."""
+    from dsv3fp8 import ops, workloads
+    counts = [128, 97, 161, 0, 1093, 131, 200, 128, 3, 140]
+    rows, groups = sum(counts), len(counts)
+    gen = torch.Generator(device="cuda").manual_seed(k)
+    x = torch.randn(rows + 5, k, generator=gen, device="cuda").bfloat16()
+    xq, xs = K.act_quant(x)
+    a_rows = torch.randint(0, rows + 5, (rows,), generator=gen, device="cuda", dtype=torch.int32)
+    w = [workloads.weight(n, k, seed=100 + g, device="cuda") for g in range(groups)]
+    b = torch.stack([wi[0].view(torch.uint8) for wi in w]).view(FP8)
+    b_s = torch.stack([wi[1] for wi in w])
+    R, tg, t0, tr = _tables(counts, rows // ops.grouped_tile_rows() + groups)
+    out32 = torch.ops.dsv3fp8.fp8_gemm_grouped(xq, xs, a_rows, b, b_s, rows, tg, t0, tr, ops.dtype_code(torch.float32))
+    out16 = torch.ops.dsv3fp8.fp8_gemm_grouped(xq, xs, a_rows, b, b_s, rows, tg, t0, tr, ops.dtype_code(torch.bfloat16))
+    assert torch.equal(out16.float(), out32.bfloat16().float())
+    assert torch.isfinite(out32).all()
+    starts = [sum(counts[:g]) for g in range(groups)]
+    blocks = [0, n // 256, n // 128 - 1]
+    for g in (0, 2, 4, 5, 6, 8):
+        c, r0 = counts[g], starts[g]
+        pick = torch.unique(torch.cat([torch.arange(0, c, max(1, c // 24)), torch.tensor([c - 1])]))
+        idx = a_rows[r0 + pick.cuda()].long()
+        for blk in blocks:
+            ref = oracle.fp8_gemm_f32(xq[idx].cpu(), xs[idx].cpu(), w[g][0][blk * 128:(blk + 1) * 128].cpu(),
+                                      w[g][1][blk:blk + 1].cpu())
+            got = out32[r0 + pick.cuda()][:, blk * 128:(blk + 1) * 128].cpu()
+            err = (got - ref).abs().max().item()
+            assert err <= 1e-2 * ref.pow(2).mean().sqrt().item(), (g, blk, err)
+
+
+def test_moe_layer_full_configuration(K):
+    """MoE.forward at the benchmark's dimensions: 256 routed + 1 shared expert, 7168 -> 2048 -> 7168, 4096 tokens,
+    8 groups / top-4 groups / top-8 experts.  Expert e holds one of four seeded prototype weights with its scales
+    multiplied by 1 + e/512, so every expert computes something else.  oracle.moe evaluates a sample of tokens (only
+    the experts those tokens select are brought to the CPU); on the whole output: finite, and permuting the tokens
+    permutes the output bit for bit (a token's arithmetic does not depend on where it sits in its expert's list)."""
+    from dsv3fp8 import model as M, workloads
+    old = (M.gemm_impl, torch.get_default_dtype(), M.Linear.dtype)
+    torch.set_default_dtype(torch.bfloat16)
+    M.Linear.dtype, M.gemm_impl = FP8, "fp8"
+    try:
+        args = M.ModelArgs()
+        assert (args.n_routed_experts, args.dim, args.moe_inter_dim, args.n_activated_experts) == (256, 7168, 2048, 8)
+        with torch.device("cuda"):
+            moe = M.MoE(args)
+        g = torch.Generator(device="cuda").manual_seed(5)
+        protos = [(workloads.weight(args.moe_inter_dim, args.dim, 40 + i, "cuda"),
+                   workloads.weight(args.dim, args.moe_inter_dim, 50 + i, "cuda"),
+                   workloads.weight(args.moe_inter_dim, args.dim, 60 + i, "cuda")) for i in range(4)]
+        with torch.no_grad():
+            moe.gate.weight.copy_(torch.randn(args.n_routed_experts, args.dim, generator=g, device="cuda") * 0.02)
+            moe.gate.bias.copy_(torch.randn(args.n_routed_experts, generator=g, device="cuda") * 0.02)
+            for e, ex in enumerate(list(moe.experts) + [moe.shared_experts]):
+                p1, p2, p3 = protos[e % 4]
+                f = 1.0 + e / 512.0
+                for lin, (w8, sc) in ((ex.w1, p1), (ex.w2, p2), (ex.w3, p3)):
+                    lin.weight.copy_(w8)
+                    lin.scale.copy_(sc * f)
+        moe.stack_experts()
+        tokens = 4096
+        x = workloads.activations(tokens, args.dim, 6, "cuda")
+        perm = torch.randperm(tokens, generator=g, device="cuda")
+        with torch.inference_mode():
+            y = moe(x)
+            y_perm = moe(x[perm].contiguous())
+            wts, idx = moe.gate(x)
+        assert y.shape == x.shape and torch.isfinite(y.float()).all()
+        assert torch.equal(y_perm.view(torch.int16), y[perm].view(torch.int16))
+        counts = torch.bincount(idx.flatten(), minlength=args.n_routed_experts)
+        assert int(counts.sum()) == tokens * 8 and int((counts > 0).sum()) > 200
+        sample = torch.tensor([0, 1777, 4095])
+
+        def cpu(ex):
+            return tuple(t.data.cpu() for lin in (ex.w1, ex.w2, ex.w3) for t in (lin.weight, lin.scale))
+        hit = set(idx[sample.cuda()].flatten().tolist())
+        experts = [cpu(ex) if e in hit else None for e, ex in enumerate(moe.experts)]
+        ref = oracle.moe(x[sample.cuda()].cpu(), wts[sample.cuda()].cpu(), idx[sample.cuda()].cpu(), experts,
+                         cpu(moe.shared_experts))
+        rms = ref.float().pow(2).mean().sqrt().item()
+        err = (y[sample.cuda()].float().cpu() - ref.float()).abs().max().item()
+        assert err <= 5e-2 * rms + 2 ** -8 * ref.abs().max().item(), (err, rms)
+    finally:
+        M.gemm_impl, M.Linear.dtype = old[0], old[2]
+        torch.set_default_dtype(old[1])

@@ -304,6 +304,30 @@ def test_gate_invariants():
     assert torch.allclose(w.float(), want.float(), atol=0.02)
 
 
+def test_gate_route_known_answer():
+    """oracle.gate_route on logits whose routing is known in closed form (model.py:577-598).  A group's score is
+    the SUM OF ITS TWO largest biased scores (:589): group 0 holds the largest single value but a small pair, so a
+    top-1 group score would pick {0, 3} and the expected experts would not come out; the bias moves the selection
+    (:581) but the weights are the unbiased scores (:594), normalised (:596) and scaled (:597)."""
+    experts, groups = 16, 4
+    logits = torch.full((1, experts), -4.0)
+    logits[0, 4], logits[0, 5] = 2.0, 1.0            # group 1
+    logits[0, 12], logits[0, 13] = 3.0, -1.0         # group 3
+    logits[0, 0] = 3.5                                # group 0: the largest value of all, nothing beside it
+    bias = torch.zeros(experts); bias[5] = 0.5; bias[13] = 0.5
+    sg = lambda v: float(torch.tensor(v).sigmoid())
+    pair = {0: sg(3.5) + sg(-4.0), 1: sg(2.0) + sg(1.0) + 0.5, 2: 2 * sg(-4.0), 3: sg(3.0) + sg(-1.0) + 0.5}
+    top1 = {0: sg(3.5), 1: sg(1.0) + 0.5, 2: sg(-4.0), 3: sg(3.0)}
+    assert set(sorted(pair, key=pair.get)[-2:]) == {1, 3} and set(sorted(top1, key=top1.get)[-2:]) == {0, 1}   # the two rules differ
+    w, idx = oracle.gate_route(logits.bfloat16(), bias, 3, groups, 2, 1.0, "sigmoid")
+    # biased scores inside groups 1 and 3: 5 -> 1.231, 12 -> 0.953, 4 -> 0.881, 13 -> 0.769
+    assert idx.tolist() == [[5, 12, 4]]
+    s = torch.tensor([1.0, 3.0, 2.0]).bfloat16().sigmoid()
+    assert torch.equal(w[0], (s / s.sum(-1, keepdim=True)) * 1.0)
+    w25, _ = oracle.gate_route(logits.bfloat16(), bias, 3, groups, 2, 2.5, "sigmoid")
+    assert torch.equal(w25[0], (s / s.sum(-1, keepdim=True)) * 2.5)
+
+
 def test_moe_equals_dense_masked_brute_force():
     g = torch.Generator().manual_seed(8)
     t, e, dim, inter = 12, 4, 128, 128
