@@ -668,7 +668,7 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
 }
 constexpr int kGroupedTileRows = 256;     // slot height of the grouped kernel's tile table
 constexpr int64_t kCUs = 256;
-inline int env_tile_rows() { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }
+inline int env_tile_rows() { static const int v = [] { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }(); return v; }
 }  // namespace
 
 // Tile height, K slicing and the last partial round.  A K block of a 256-row tile costs about 1.64x one of a

@@ -317,6 +317,7 @@ inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
         // and one scale per thread
         int64_t slab_kb = (int64_t)kSlabChunks * waves * 64 / (m * 8);
         if (slab_kb > waves * 64 / m) slab_kb = waves * 64 / m;
+        if (slab_kb > 480 / m) slab_kb = 480 / m;              // (slab_kb m + 16) 128 + 4 slab_kb m <= 64 KiB of LDS
         if (slab_kb < 1) continue;
         const int64_t min_splits = (kb + slab_kb - 1) / slab_kb;
         if (splits < min_splits) splits = min_splits;

@@ -126,6 +126,11 @@ __global__ __launch_bounds__(64 * kTokensPerWg) void gate_route_kernel(
             // any other group size: through LDS, lane g walks group g
 #pragma unroll
             for (int s = 0; s < EPL; ++s) mine[s * 64 + lane] = sel[s];
+            // lanes below read what other lanes of the wavefront have just written: order the LDS stores before the
+            // loads for the compiler too (the hardware retires a wavefront's LDS operations in order)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             if (lane < n_groups) {
                 float top1 = ninf, top2 = ninf;
                 for (int j = 0; j < gsz; ++j) {

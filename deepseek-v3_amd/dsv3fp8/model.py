@@ -65,12 +65,14 @@ class ModelArgs:
 def _scales_are_powers_of_two(weight: torch.Tensor, scale: Optional[torch.Tensor] = None) -> bool:
     """Whether every block scale of an fp8 weight is a power of two (checkpoints made for ``scale_fmt = "ue8m0"``,
     inference/configs/config_v3.1.json:22, store them that way).  Looked at once per version of the scale tensor
-    (one device-to-host read), never while a graph is being captured."""
+    (one device-to-host read), never while a graph is being captured.  The verdict is keyed on the scale tensor's
+    storage address and version counter; a tensor made under inference_mode has no counter, so such scales must
+    not be rewritten in place after the first forward (reload them into a new module instead)."""
     scale = weight.scale if scale is None else scale
     try:
-        version = scale._version
+        version = (scale.data_ptr(), scale._version)
     except RuntimeError:            # a tensor made under inference_mode has no version counter: looked at once
-        version = -1
+        version = (scale.data_ptr(), -1)
     cached = getattr(weight, "_dsv3_pow2", None)
     if cached is not None and cached[0] == version:
         return cached[1]
@@ -181,17 +183,19 @@ def precompute_freqs_cis(args: ModelArgs) -> torch.Tensor:
     ``[max_seq_len, qk_rope_head_dim / 2]`` tensor (model.py:294-372).  Beyond ``original_seq_len`` the
     frequencies are stretched YaRN-style: pair j keeps its frequency where it completes more than ``beta_fast``
     turns over the original window, is divided by ``rope_factor`` where it completes fewer than ``beta_slow``,
-    and is blended linearly in between."""
+    and is blended linearly in between.  The binary32 expressions are evaluated in the reference's order
+    (1 / base^(j/dim); keep = 1 - ramp; f / factor * (1 - keep) + f * keep), so the table is the same bit for bit."""
     dim, base = args.qk_rope_head_dim, args.rope_theta
-    freqs = base ** (-torch.arange(0, dim, 2, dtype=torch.float32) / dim)
+    freqs = 1.0 / (base ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))
     if args.max_seq_len > args.original_seq_len:
         def pair_index(turns: float) -> float:     # the (fractional) pair that makes `turns` rotations in the window
             return dim * math.log(args.original_seq_len / (turns * 2 * math.pi)) / (2 * math.log(base))
         lo = max(math.floor(pair_index(args.beta_fast)), 0)
         hi = min(math.ceil(pair_index(args.beta_slow)), dim - 1)
         span = (hi - lo) if hi != lo else 0.001
-        stretched = ((torch.arange(dim // 2, dtype=torch.float32) - lo) / span).clamp(0, 1)   # 0: keep, 1: stretch
-        freqs = freqs / args.rope_factor * stretched + freqs * (1 - stretched)
+        ramp = torch.clamp((torch.arange(dim // 2, dtype=torch.float32) - lo) / span, 0, 1)
+        keep = 1 - ramp
+        freqs = freqs / args.rope_factor * (1 - keep) + freqs * keep
     angles = torch.outer(torch.arange(args.max_seq_len), freqs)
     return torch.polar(torch.ones_like(angles), angles)
 
@@ -207,16 +211,17 @@ def apply_rotary_emb(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
 
 
 class MLA(nn.Module):
-    """Multi-head latent attention (model.py:395-497) with the reference's two cache layouts.
+    """Host of the two ``wkv_b`` products of the absorbed multi-head latent attention (model.py:395-497).
 
-    ``attn_impl == "absorb"`` keeps the compressed latent (``kv_cache`` [b, t, kv_lora_rank]) and the shared
-    rotary key (``pe_cache``), and folds the up-projection ``wkv_b`` into the query and the output:
-    ``q_nope @ wkv_b[:, :nope]`` before the scores and ``@ wkv_b[:, -v:]^T`` after the weighted sum.  When
-    ``wkv_b`` is stored in FP8 the reference dequantises the whole weight on every call (model.py:481); here the
-    two products read the FP8 weight and its block scales directly (``torch.ops.dsv3fp8.wkv_b_absorb``), with
-    the same bf16 rounding of every dequantised weight.  ``MLA.fused = False`` selects the dequantise-then-einsum
-    sequence of the reference instead.  The score / softmax / weighted-sum einsums are bf16 torch operations as
-    in the reference: they do not touch FP8 data.
+    Only the reference's default cache layout (``attn_impl == "absorb"``) is hosted: the compressed latent
+    (``kv_cache`` [b, t, kv_lora_rank]) and the shared rotary key (``pe_cache``) are cached and the up-projection
+    ``wkv_b`` is folded into the query (``q_nope @ wkv_b[:, :nope]``, before the scores) and into the output
+    (``@ wkv_b[:, -v:]^T``, after the weighted sum).  With ``wkv_b`` in FP8 the reference dequantises the whole
+    weight on every call (model.py:481); here the two products read the FP8 weight and its block scales in place
+    (``torch.ops.dsv3fp8.wkv_b_absorb``) with the same bf16 rounding of every dequantised weight.
+    ``MLA.fused = False`` selects the dequantise-then-einsum sequence instead.  Everything between the two products
+    (scores, softmax, weighted sum) is bf16 torch arithmetic that never touches FP8 data; it is here so that the
+    products can be tested in place.  Parameter names are the checkpoint's.
 
     ``wq_a`` and ``wkv_a`` read the same input.  With FP8 weights (and ``q_lora_rank`` a multiple of the block size,
     so that both keep their own scale blocks) ``stack_a()`` lays them out as one ``[q_lora_rank + kv_lora_rank +
@@ -225,41 +230,33 @@ class MLA(nn.Module):
     """
 
     fused: bool = True
+    stacked_a: bool = True
 
     def __init__(self, args: ModelArgs):
         super().__init__()
-        self.dim = args.dim
-        self.n_heads = args.n_heads
-        self.n_local_heads = args.n_heads // world_size
-        self.q_lora_rank = args.q_lora_rank
-        self.kv_lora_rank = args.kv_lora_rank
-        self.qk_nope_head_dim = args.qk_nope_head_dim
-        self.qk_rope_head_dim = args.qk_rope_head_dim
-        self.qk_head_dim = args.qk_nope_head_dim + args.qk_rope_head_dim
-        self.v_head_dim = args.v_head_dim
-        if self.q_lora_rank == 0:
-            self.wq = ColumnParallelLinear(self.dim, self.n_heads * self.qk_head_dim)
-        else:
+        if attn_impl != "absorb":
+            raise NotImplementedError("only the absorbed cache layout (the reference's default) is hosted")
+        nope, rope, v = args.qk_nope_head_dim, args.qk_rope_head_dim, args.v_head_dim
+        self.dim, self.n_heads, self.n_local_heads = args.dim, args.n_heads, args.n_heads // world_size
+        self.q_lora_rank, self.kv_lora_rank = args.q_lora_rank, args.kv_lora_rank
+        self.qk_nope_head_dim, self.qk_rope_head_dim, self.v_head_dim, self.qk_head_dim = nope, rope, v, nope + rope
+        # projections, by their checkpoint names: query (optionally through a low-rank pair), latent + rotary key,
+        # the up-projection that gets absorbed, output
+        if self.q_lora_rank:
             self.wq_a = Linear(self.dim, self.q_lora_rank)
             self.q_norm = RMSNorm(self.q_lora_rank)
             self.wq_b = ColumnParallelLinear(self.q_lora_rank, self.n_heads * self.qk_head_dim)
-        self.wkv_a = Linear(self.dim, self.kv_lora_rank + self.qk_rope_head_dim)
-        self.kv_norm = RMSNorm(self.kv_lora_rank)
-        self.wkv_b = ColumnParallelLinear(self.kv_lora_rank, self.n_heads * (self.qk_nope_head_dim + self.v_head_dim))
-        self.wo = RowParallelLinear(self.n_heads * self.v_head_dim, self.dim)
-        self.softmax_scale = self.qk_head_dim ** -0.5
-        if args.max_seq_len > args.original_seq_len:
-            mscale = 0.1 * args.mscale * math.log(args.rope_factor) + 1.0
-            self.softmax_scale = self.softmax_scale * mscale * mscale
-        b, t, h = args.max_batch_size, args.max_seq_len, self.n_local_heads
-        if attn_impl == "naive":
-            self.register_buffer("k_cache", torch.zeros(b, t, h, self.qk_head_dim), persistent=False)
-            self.register_buffer("v_cache", torch.zeros(b, t, h, self.v_head_dim), persistent=False)
         else:
-            self.register_buffer("kv_cache", torch.zeros(b, t, self.kv_lora_rank), persistent=False)
-            self.register_buffer("pe_cache", torch.zeros(b, t, self.qk_rope_head_dim), persistent=False)
-
-    stacked_a: bool = True
+            self.wq = ColumnParallelLinear(self.dim, self.n_heads * self.qk_head_dim)
+        self.wkv_a = Linear(self.dim, self.kv_lora_rank + rope)
+        self.kv_norm = RMSNorm(self.kv_lora_rank)
+        self.wkv_b = ColumnParallelLinear(self.kv_lora_rank, self.n_heads * (nope + v))
+        self.wo = RowParallelLinear(self.n_heads * v, self.dim)
+        # 1/sqrt(d), times the YaRN magnitude correction squared when the window is extended (model.py:438-441)
+        yarn = 0.1 * args.mscale * math.log(args.rope_factor) + 1.0 if args.max_seq_len > args.original_seq_len else 1.0
+        self.softmax_scale = self.qk_head_dim ** -0.5 * yarn * yarn
+        for name, width in (("kv_cache", self.kv_lora_rank), ("pe_cache", rope)):
+            self.register_buffer(name, torch.zeros(args.max_batch_size, args.max_seq_len, width), persistent=False)
 
     def stack_a(self) -> bool:
         """wq_a over wkv_a in one buffer (scales likewise); returns whether the layers qualify.  Idempotent; the
@@ -289,50 +286,45 @@ class MLA(nn.Module):
             return torch.einsum("bshd,hdc->bshc", x, wkv_b[:, :self.qk_nope_head_dim])
         return torch.einsum("bshc,hdc->bshd", x, wkv_b[:, -self.v_head_dim:])
 
-    def forward(self, x: torch.Tensor, start_pos: int, freqs_cis: torch.Tensor, mask: Optional[torch.Tensor]):
-        bsz, seqlen, _ = x.size()
-        end_pos = start_pos + seqlen
+    def _project(self, x: torch.Tensor):
+        """Per-head queries [b, s, h, nope + rope] and the latent + rotary-key row [b, s, kv_lora_rank + rope]."""
         if self.stacked_a and gemm_impl == "fp8" and x.is_cuda and self.stack_a():
             qa, kva = torch.split(linear(x, self._wa, None, self.wq_a.scale_fmt),
                                   [self.q_lora_rank, self.kv_lora_rank + self.qk_rope_head_dim], dim=-1)
             q = self.wq_b(self.q_norm(qa))
         else:
-            q = self.wq(x) if self.q_lora_rank == 0 else self.wq_b(self.q_norm(self.wq_a(x)))
+            q = self.wq_b(self.q_norm(self.wq_a(x))) if self.q_lora_rank else self.wq(x)
             kva = self.wkv_a(x)
-        q = q.view(bsz, seqlen, self.n_local_heads, self.qk_head_dim)
-        q_nope, q_pe = torch.split(q, [self.qk_nope_head_dim, self.qk_rope_head_dim], dim=-1)
-        q_pe = apply_rotary_emb(q_pe, freqs_cis)
-        kv, k_pe = torch.split(kva, [self.kv_lora_rank, self.qk_rope_head_dim], dim=-1)
-        k_pe = apply_rotary_emb(k_pe.unsqueeze(2), freqs_cis)
-        if attn_impl == "naive":
-            q = torch.cat([q_nope, q_pe], dim=-1)
-            kv = self.wkv_b(self.kv_norm(kv)).view(bsz, seqlen, self.n_local_heads, self.qk_nope_head_dim + self.v_head_dim)
-            k_nope, v = torch.split(kv, [self.qk_nope_head_dim, self.v_head_dim], dim=-1)
-            self.k_cache[:bsz, start_pos:end_pos] = torch.cat([k_nope, k_pe.expand(-1, -1, self.n_local_heads, -1)], dim=-1)
-            self.v_cache[:bsz, start_pos:end_pos] = v
-            scores = torch.einsum("bshd,bthd->bsht", q, self.k_cache[:bsz, :end_pos]) * self.softmax_scale
-        else:
-            w = self.wkv_b.weight
-            if w.element_size() > 1:
-                wkv_b = w.view(self.n_local_heads, -1, self.kv_lora_rank)
-            elif self.fused and x.is_cuda and x.dtype == torch.bfloat16:
-                wkv_b = None
-            else:
-                wkv_b = weight_dequant(w, self.wkv_b.scale, block_size).view(self.n_local_heads, -1, self.kv_lora_rank)
-            q_nope = self._absorb(q_nope, ops._lib.ABSORB_Q, wkv_b)
-            self.kv_cache[:bsz, start_pos:end_pos] = self.kv_norm(kv)
-            self.pe_cache[:bsz, start_pos:end_pos] = k_pe.squeeze(2)
-            scores = (torch.einsum("bshc,btc->bsht", q_nope, self.kv_cache[:bsz, :end_pos]) +
-                      torch.einsum("bshr,btr->bsht", q_pe, self.pe_cache[:bsz, :end_pos])) * self.softmax_scale
+        return q.unflatten(-1, (self.n_local_heads, self.qk_head_dim)), kva
+
+    def _dequantised_wkv_b(self, x: torch.Tensor) -> Optional[torch.Tensor]:
+        """[h, nope+v, c] weight for the einsum path, or None when the products read the FP8 weight in place."""
+        w = self.wkv_b.weight
+        if w.element_size() == 1:
+            if self.fused and x.is_cuda and x.dtype == torch.bfloat16:
+                return None
+            w = weight_dequant(w, self.wkv_b.scale, block_size)
+        return w.view(self.n_local_heads, -1, self.kv_lora_rank)
+
+    def forward(self, x: torch.Tensor, start_pos: int, freqs_cis: torch.Tensor, mask: Optional[torch.Tensor]):
+        b, s = x.size(0), x.size(1)
+        t = start_pos + s
+        q, kva = self._project(x)
+        wkv_b = self._dequantised_wkv_b(x)
+        # this step's rows of the two caches
+        self.kv_cache[:b, start_pos:t] = self.kv_norm(kva[..., :self.kv_lora_rank])
+        self.pe_cache[:b, start_pos:t] = apply_rotary_emb(kva[..., self.kv_lora_rank:].unsqueeze(2), freqs_cis).squeeze(2)
+        latent, rope_keys = self.kv_cache[:b, :t], self.pe_cache[:b, :t]
+        # scores over the latent (query folded through wkv_b) plus the rotary part; softmax in binary32
+        q_latent = self._absorb(q[..., :self.qk_nope_head_dim], ops._lib.ABSORB_Q, wkv_b)
+        q_rope = apply_rotary_emb(q[..., self.qk_nope_head_dim:], freqs_cis)
+        scores = torch.einsum("bshc,btc->bsht", q_latent, latent) + torch.einsum("bshr,btr->bsht", q_rope, rope_keys)
+        scores = scores * self.softmax_scale
         if mask is not None:
-            scores += mask.unsqueeze(1)
-        scores = scores.softmax(dim=-1, dtype=torch.float32).type_as(x)
-        if attn_impl == "naive":
-            x = torch.einsum("bsht,bthd->bshd", scores, self.v_cache[:bsz, :end_pos])
-        else:
-            x = torch.einsum("bsht,btc->bshc", scores, self.kv_cache[:bsz, :end_pos])
-            x = self._absorb(x, ops._lib.ABSORB_V, wkv_b)
-        return self.wo(x.flatten(2))
+            scores = scores + mask.unsqueeze(1)
+        probs = scores.softmax(dim=-1, dtype=torch.float32).type_as(x)
+        out = self._absorb(torch.einsum("bsht,btc->bshc", probs, latent), ops._lib.ABSORB_V, wkv_b)
+        return self.wo(out.flatten(2))
 
 
 class MLP(nn.Module):
@@ -513,7 +505,12 @@ class MoE(nn.Module):
 
     def _grouped_ok(self, x: torch.Tensor) -> bool:
         ex = self.experts[self.experts_start_idx]
-        return (self.grouped and gemm_impl == "fp8" and world_size == 1 and x.is_cuda
+        inter = ex.w1.out_features
+        pairs = x.size(0) * self.n_activated_experts
+        # the grouped kernels' limits: up to 16 experts per token, 32-bit offsets into the gathered rows and into x
+        fits = (0 < x.size(0) and self.n_activated_experts <= 16 and pairs * max(inter, self.dim) < 2 ** 32
+                and x.size(0) * self.dim < 2 ** 32)
+        return (self.grouped and fits and gemm_impl == "fp8" and world_size == 1 and x.is_cuda
                 and ex.w1.weight.element_size() == 1 and x.dtype == torch.bfloat16
                 and torch.get_default_dtype() == torch.bfloat16
                 and ex.w1.out_features % block_size == 0 and self.dim % block_size == 0)

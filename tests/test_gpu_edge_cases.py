@@ -76,3 +76,47 @@ def test_activation_matrix_beyond_4_gib(K):
     assert (got - ref).abs().max().item() <= 1e-2 * ref.pow(2).mean().sqrt().item()
     del a, a_s, c
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("m,k", [(2, 32768), (1, 61568)])
+def test_few_rows_and_a_very_long_k(m, k):
+    """K beyond every DeepSeek-V3 projection at one and two rows: the activation slab of the few-row kernel is capped
+    at what 64 KiB of LDS holds (more K splits instead of a refused launch)."""
+    import dsv3fp8 as K
+    g = torch.Generator().manual_seed(k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w8, ws = oracle.block_quant_weight((torch.randn(256, k, generator=g) * 0.02).bfloat16())
+    a, a_s = oracle.act_quant(x)
+    ref = oracle.fp8_gemm_f32(a, a_s, w8, ws)
+    got = K.fp8_gemm_f32(a.cuda(), a_s.cuda(), w8.cuda(), ws.cuda()).cpu()
+    assert (got - ref).abs().max().item() <= 1e-2 * ref.pow(2).mean().sqrt().item()
+
+
+def test_moe_beyond_the_grouped_limits_takes_the_expert_loop():
+    """17 experts per token is more than the grouped bookkeeping handles (16): MoE.forward falls back to the
+    reference's expert loop instead of raising, and an empty batch returns an empty result."""
+    from dsv3fp8 import model as M
+    old = (M.gemm_impl, torch.get_default_dtype(), M.Linear.dtype)
+    torch.set_default_dtype(torch.bfloat16)
+    M.Linear.dtype, M.gemm_impl = torch.float8_e4m3fn, "fp8"
+    try:
+        args = M.ModelArgs(dim=256, inter_dim=512, moe_inter_dim=128, n_routed_experts=32, n_shared_experts=1,
+                           n_activated_experts=17, n_expert_groups=1, n_limited_groups=1, route_scale=1.0)
+        with torch.device("cuda"):
+            moe = M.MoE(args)
+        g = torch.Generator().manual_seed(3)
+        with torch.no_grad():
+            moe.gate.weight.copy_((torch.randn(32, 256, generator=g) * 0.05).bfloat16().cuda())
+            for lin in [l for ex in list(moe.experts) + [moe.shared_experts] for l in (ex.w1, ex.w2, ex.w3)]:
+                w8, s = oracle.block_quant_weight((torch.randn(lin.out_features, lin.in_features, generator=g) * 0.05).bfloat16())
+                lin.weight.copy_(w8.cuda()); lin.scale.copy_(s.cuda())
+        x = torch.randn(9, 256, generator=g).bfloat16().cuda()
+        with torch.inference_mode():
+            assert not moe._grouped_ok(x)
+            y = moe(x)
+            assert y.shape == x.shape and torch.isfinite(y.float()).all()
+            empty = moe(x[:0])
+            assert empty.shape == (0, 256)
+    finally:
+        M.gemm_impl, M.Linear.dtype = old[0], old[2]
+        torch.set_default_dtype(old[1])

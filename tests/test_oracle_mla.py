@@ -127,3 +127,37 @@ def test_mla_absorbed_equals_textbook_attention():
     # the caches hold the normalised latent and the rotated shared key of the positions just written
     assert (kv_cache[:, :seqlen].double() - lat).abs().max() < 0.1 and kv_cache[:, seqlen:].abs().max() == 0
     assert (pe_cache[:, :seqlen].double() - k_pe.squeeze(2)).abs().max() < 0.1
+
+
+def test_rotary_table_equals_the_reference_expressions_bit_for_bit():
+    """precompute_freqs_cis against the reference's expressions written out literally (model.py:297-372): the same
+    binary32 operations in the same order, for the extended window (YaRN) and for the plain one."""
+    import math
+    import sys
+    from pathlib import Path
+    sys.path.insert(0, str(Path(__file__).resolve().parent.parent / "deepseek-v3_amd"))
+    try:
+        from dsv3fp8 import model as M
+    except ImportError:
+        import pytest
+        pytest.skip("the package needs its HIP library to import")
+    for max_seq_len in (4096 * 4, 4096):
+        args = M.ModelArgs(max_seq_len=max_seq_len)
+        dim, base, factor = args.qk_rope_head_dim, args.rope_theta, args.rope_factor
+
+        def correction_dim(num_rotations):
+            return dim * math.log(args.original_seq_len / (num_rotations * 2 * math.pi)) / (2 * math.log(base))
+        freqs = 1.0 / (base ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))
+        if max_seq_len > args.original_seq_len:
+            low = max(math.floor(correction_dim(args.beta_fast)), 0)
+            high = min(math.ceil(correction_dim(args.beta_slow)), dim - 1)
+            if low == high:
+                high += 0.001
+            ramp = torch.clamp((torch.arange(dim // 2, dtype=torch.float32) - low) / (high - low), 0, 1)
+            smooth = 1 - ramp
+            freqs = freqs / factor * (1 - smooth) + freqs * smooth
+        t = torch.arange(max_seq_len)
+        f = torch.outer(t, freqs)
+        want = torch.polar(torch.ones_like(f), f)
+        got = M.precompute_freqs_cis(args)
+        assert torch.equal(torch.view_as_real(got), torch.view_as_real(want))
