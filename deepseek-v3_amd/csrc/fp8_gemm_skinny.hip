@@ -28,6 +28,7 @@ namespace skinny {
 
 constexpr int kMaxWaves = 16;
 
+
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
     v8i r = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
     return r;
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         void* __restrict__ out, int out_dtype,      // out_dtype: dsv3_dtype of `out` (F32 slabs when gridDim.y > 1)
-        int M, int N, int K, int kb_per_wg, int ue8m0) {
+        int M, int N, int K, int kb_per_wg, int ue8m0, uint64_t m_magic) {     // m_magic = ceil(2^32 / M)
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -118,12 +119,16 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
     v4i stage[kSlabChunks];
     v4u raw[QF ? kSlabChunks : 1][2];                          // QF: the 16 bf16 values behind each chunk
     float stage_q[QF ? kSlabChunks : 1];                       // QF: weight-block scale of the chunk's K block
-    float stage_s = 0.f;
+    // the two factors of a (row, K block) scale stay apart until the slab is written: multiplying them here would
+    // put a wait for these loads in front of the weight loads below
+    float stage_sa = 0.f, stage_sb = 0.f;
+    // x / M and x % M for x < 2^16 without an integer division (M is a run-time value)
+    auto div_m = [&](int x) { return (int)(((uint64_t)(uint32_t)x * m_magic) >> 32); };
 #pragma unroll
     for (int i = 0; i < kSlabChunks; ++i) {
         const int c = tid + i * (int)blockDim.x;
         if (c < chunks) {
-            const int ch = c & 7, R = c >> 3, row = R % M, kb = R / M;
+            const int ch = c & 7, R = c >> 3, kb = div_m(R), row = R - kb * M;
             if (QF) {
                 const v4u* src = (const v4u*)(a + 2 * ((size_t)row * K + (size_t)(wg_kb0 + kb) * 128 + ch * 16));
                 raw[i][0] = src[0];
@@ -137,9 +142,11 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
             stage_q[i] = 0.f;
         }
     }
-    if (!QF && tid < wg_nkb * M)   // scale of (row, K block) with the weight block's scale already folded in
-        stage_s = a_s[(size_t)(tid % M) * KB + wg_kb0 + tid / M] * b_s[(size_t)min(n0 >> 7, (N - 1) >> 7) * KB + wg_kb0 + tid / M];
-
+    if (!QF && tid < wg_nkb * M) {  // scale of (row, K block) and the weight block's scale
+        const int kb = div_m(tid), row = tid - kb * M;
+        stage_sa = a_s[(size_t)row * KB + wg_kb0 + kb];
+        stage_sb = b_s[(size_t)min(n0 >> 7, (N - 1) >> 7) * KB + wg_kb0 + kb];
+    }
     // ---- start the weight stream: the first NPF K blocks of every strip
     v4i wlo[NPF][S], whi[NPF][S];
     auto fetch = [&](int p, int k) {
@@ -152,7 +159,6 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
 #pragma unroll
     for (int p = 0; p < NPF; ++p)
         if (p < nkb) fetch(p, p);
-
     if (QF) {
         // the 8 lanes that hold the chunks of one (row, K block) are consecutive and aligned: amax by DPP
 #pragma unroll
@@ -205,7 +211,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
                 *(v4i*)(act + R * 128 + ((ch ^ swz(R)) * 16)) = stage[i];
             }
         }
-        if (tid < wg_nkb * M) act_s[tid] = stage_s;
+        if (tid < wg_nkb * M) act_s[tid] = stage_sa * stage_sb;
     }
     __syncthreads();
 
@@ -264,13 +270,19 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
 #pragma unroll
         for (int j = 0; j < MT; ++j) red[(wave * TILES + s * MT + j) * 64 + lane] = acc[s][j];
     __syncthreads();
-
     const size_t slab = (size_t)blockIdx.y * M * N;          // split-K slab of the fp32 workspace (0 when gridDim.y == 1)
     for (int slot = tid; slot < TILES * 64; slot += blockDim.x) {
+        // the partial sums of the wavefronts, added in wavefront order; read four at a time so that the LDS latency
+        // is paid once per four and not once per wavefront (a missing wavefront re-reads the last one, weight 0)
         v4f v = red[slot];
-        for (int w = 1; w < n_waves; ++w) {
-            const v4f u = red[w * TILES * 64 + slot];
-            v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
+        for (int w0 = 1; w0 < n_waves; w0 += 4) {
+            v4f u[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) u[i] = red[min(w0 + i, n_waves - 1) * TILES * 64 + slot];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (w0 + i < n_waves) { v[0] += u[i][0]; v[1] += u[i][1]; v[2] += u[i][2]; v[3] += u[i][3]; }
+            }
         }
         const int t = slot >> 6, l = slot & 63;
         const int s = t / MT, j = t % MT;
@@ -278,6 +290,12 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
         const int n = n0 + s * 16 + (l >> 4) * 4;
         if (m >= M) continue;
         const size_t idx = slab + (size_t)m * N + n;
+        if (n + 3 < N && (N & 3) == 0) {                      // four results in one store
+            if (out_dtype == DSV3_F32) *(v4f*)((float*)out + idx) = v;
+            else if (out_dtype == DSV3_BF16) *(v2u*)((uint16_t*)out + idx) = v2u{ pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]) };
+            else *(v2u*)((uint16_t*)out + idx) = v2u{ pack_f16(v[0], v[1]), pack_f16(v[2], v[3]) };
+            continue;
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             if (n + e >= N) break;
@@ -341,7 +359,8 @@ void launch_cfg(const Plan& p, const void* a, const float* a_s, const void* b, c
     const size_t slab_bytes = ((size_t)p.kb_per_wg * m + 16) * 128 + (size_t)p.kb_per_wg * m * 4;
     const size_t lds = red_bytes > slab_bytes ? red_bytes : slab_bytes;
     hipLaunchKernelGGL((fp8_gemm_skinny_kernel<MT, S, NPF, QF>), dim3(groups, (unsigned)p.splits), dim3(p.waves * kWave), lds, st,
-                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, out_dtype, m, n, k, p.kb_per_wg, ue8m0);
+                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, out_dtype, m, n, k, p.kb_per_wg, ue8m0,
+                       (uint64_t)(((1ull << 32) + (uint64_t)m - 1) / (uint64_t)m));
 }
 
 }  // namespace skinny
