@@ -150,11 +150,12 @@ __device__ __forceinline__ void tile(
         copy16(m2_base[t] + (uint32_t)kb * 128u, m2_src[t], lds_addr_of(lds + m2_dst[t] + stage * STAGE));
     };
     // scales of a K block: wavefronts 0-3 copy a_s[row, kb] of 64 tile rows each, wavefront 4 the b_s rows of the two
-    // column halves (wavefronts 5-7 repeat that into slots nobody reads: no branch in the loop)
+    // column halves (lanes 0 and 1; its other lanes and wavefronts 5-7 repeat an address already requested, so that
+    // every wavefront issues the same number of copies per block without asking the memory pipeline for more lines)
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
     const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT
-                                      : (uint32_t)min(n0 / 128 + lane, nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
+                                      : (uint32_t)min(n0 / 128 + (wave == 4 ? min(lane, 1) : 0), nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
     auto issue_scales = [&](int kb, int slot) {
         copy4(sc_base + (uint32_t)kb, sc_off * 4u, lds_addr_of(lds + LDS_SC + slot * SC_SLOT + wave * 256));
     };
