@@ -51,7 +51,8 @@ class Probes:
         L = self.lib = C.CDLL(str(path))
         L.dsv3_probe_read_stream.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
         L.dsv3_probe_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
-        L.dsv3_probe_mfma.argtypes = [C.c_int, C.c_void_p, C.c_void_p]
+        L.dsv3_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.dsv3_probe_mix.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         L.dsv3_probe_mfma_flops.restype = C.c_double
         L.dsv3_probe_mfma_flops.argtypes = [C.c_int]
         L.dsv3_probe_null.argtypes = [C.c_void_p]
@@ -76,20 +77,55 @@ class Probes:
             launches = launches * (-(-40 // len(launches)))
         return time_graph(launches)
 
+    def mix_gbps(self, dst, rd: int, wr: int) -> float:
+        """GB/s (bytes read + written) of a stream that reads rd and writes wr bytes per unit, over ~1 GiB."""
+        import ctypes as C
+        n_read = self.pool.numel() if rd >= wr else self.pool.numel() // 2
+        done = C.c_size_t(0)
+        call = lambda: self.lib.dsv3_probe_mix(self.pool.data_ptr(), dst.data_ptr(), n_read, rd, wr, C.byref(done), self._st())
+        assert call() == 0
+        us = time_graph([call] * 4)
+        return (done.value + done.value * wr // rd) / us / 1e3
+
+    def mix_same_size_us(self, rd: int, wr: int, bytes_read: int, copies: int) -> float:
+        """Microseconds per launch of the rd : wr stream over `bytes_read` input bytes, sources and destinations
+        rotating like the measured kernel's (so neither side is served by the Infinity Cache)."""
+        copies = max(1, min(copies, self.pool.numel() // bytes_read))
+        bytes_written = bytes_read * wr // rd
+        dst = torch.empty(copies * bytes_written, dtype=torch.uint8, device="cuda")
+        calls = [(lambda i=i: self.lib.dsv3_probe_mix(self.pool.data_ptr() + i * bytes_read, dst.data_ptr() + i * bytes_written,
+                                                      bytes_read, rd, wr, None, self._st())) for i in range(copies)]
+        assert calls[0]() == 0
+        us = time_graph(calls * 2)
+        del dst
+        return us
+
+    def mfma_tflops(self, mode: int, iters: int = 4000) -> float:
+        us = time_graph([lambda: self.lib.dsv3_probe_mfma(iters, mode, self.pool.data_ptr(), self.sink.data_ptr(), self._st())] * 10)
+        return self.lib.dsv3_probe_mfma_flops(iters) / us / 1e6
+
     def ceilings(self) -> dict:
         n = self.pool.numel()
         dst = torch.empty_like(self.pool)
         rd = time_graph([lambda: self.read(0, n)] * 4)
         cp = time_graph([lambda: self.lib.dsv3_probe_copy(self.pool.data_ptr(), dst.data_ptr(), n, 0, self._st())] * 4)
+        r2w1 = self.mix_gbps(dst, 2, 1)
+        r1w2 = self.mix_gbps(dst, 1, 2)
         del dst
-        iters = 2000
-        mf = time_graph([lambda: self.lib.dsv3_probe_mfma(iters, self.sink.data_ptr(), self._st())] * 10)
         nl = time_graph([lambda: self.lib.dsv3_probe_null(self._st())] * 100)
         return {"hbm_read_stream_GBps": round(n / rd / 1e3, 1), "hbm_copy_GBps": round(2 * n / cp / 1e3, 1),
-                "fp8_mfma_loop_TFLOPs": round(self.lib.dsv3_probe_mfma_flops(iters) / mf / 1e6, 1),
+                "hbm_read2_write1_GBps": round(r2w1, 1), "hbm_read1_write2_GBps": round(r1w2, 1),
+                "fp8_mfma_loop_TFLOPs": round(self.mfma_tflops(0), 1),
+                "fp8_mfma_loop_changing_operands_TFLOPs": round(self.mfma_tflops(1), 1),
+                "fp8_mfma_loop_with_fold_TFLOPs": round(self.mfma_tflops(2), 1),
                 "empty_launch_us": round(nl, 2),
-                "note": "measured on this GPU in this run: 1 GiB read stream; 1 GiB copy (bytes read + written); "
-                        "registers-only v_mfma_f32_16x16x128_f8f6f4 loop, 8 wavefronts per CU; empty kernel in a graph"}
+                "note": "measured on this GPU in this run: 1 GiB read stream; 1 GiB copy (bytes read + written); streams "
+                        "that read two bytes per byte written (the mix of act_quant and weight_quant) and one per two "
+                        "written (weight_dequant); registers-only v_mfma_f32_16x16x128_f8f6f4 loops, 8 wavefronts per "
+                        "CU: one operand pair for all instructions, 4 x 4 fragments of random bytes accumulated in the "
+                        "matrix core (what power-of-two scales allow), and the same with every product folded into "
+                        "its accumulator by four FMAs (what binary32 block scales need) -- the chip is power limited, "
+                        "so the rate falls as operands toggle and as vector work is added; empty kernel in a graph"}
 
 
 def _events(n):
@@ -161,10 +197,12 @@ def decode_bytes(m, n, k):
     return n * k + 4 * (-(-n // 128)) * (k // 128) + m * k + 4 * m * (k // 128) + 2 * m * n
 
 
-def _bw(nbytes: float, us: float, ceil_gbps: float) -> dict:
+def _bw(nbytes: float, us: float, copy_gbps: float, mix_us: float) -> dict:
+    """mix_us: a plain stream of the same size and read : write ratio as this kernel, measured the same way."""
     gbs = nbytes / us / 1e3
     return {"us": round(us, 2), "GBps": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 3),
-            "frac_of_measured_copy": round(gbs / ceil_gbps, 3)}
+            "frac_of_measured_copy": round(gbs / copy_gbps, 3),
+            "plain_stream_same_size_and_mix_us": round(mix_us, 2), "frac_of_that_stream": round(mix_us / us, 3)}
 
 
 def run_extras(K, W, probes, ceil):
@@ -173,16 +211,16 @@ def run_extras(K, W, probes, ceil):
     x = W.activations(4096, 7168, 0, "cuda", outliers=True)
     xs = [x.clone() for _ in range(12)]                       # 12 x 58.7 MB > Infinity Cache
     us = time_graph([(lambda t=t: K.act_quant(t)) for t in xs] * 2)
-    out["act_quant_4096x7168"] = _bw(88.998e6, us, copy_c)
+    out["act_quant_4096x7168"] = _bw(88.998e6, us, copy_c, probes.mix_same_size_us(2, 1, 4096 * 7168 * 2, 12))
     del xs
     w8, s = W.random_fp8_weight(18432, 7168, 2, "cuda")
     ws_ = [w8.clone() for _ in range(5)]
     us = time_graph([(lambda t=t: K.weight_dequant(t, s)) for t in ws_] * 2)
-    out["weight_dequant_18432x7168"] = _bw(396.394e6, us, copy_c)
+    out["weight_dequant_18432x7168"] = _bw(396.394e6, us, copy_c, probes.mix_same_size_us(1, 2, 18432 * 7168, 6))
     del ws_, w8
     wb = [(torch.randn(18432, 7168, device="cuda") * 0.02).bfloat16() for _ in range(4)]   # 4 x 264 MB
     us = time_graph([(lambda t=t: K.weight_quant(t)) for t in wb] * 2)
-    out["weight_quant_18432x7168"] = _bw(396.394e6, us, copy_c)
+    out["weight_quant_18432x7168"] = _bw(396.394e6, us, copy_c, probes.mix_same_size_us(2, 1, 18432 * 7168 * 2, 4))
     del wb
     k, n = W.PREFILL_SHAPES["w2"]
     a, a_s = K.act_quant(W.activations(4096, k, 0, "cuda"))
@@ -475,7 +513,8 @@ def main():
                      "peak": FP8_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4), "traffic": measured_traffic(),
                      "launch_us": round(gemm_ms * 1e3, 2), "flops_per_launch": flops,
-                     "frac_of_measured_mfma_loop": round(achieved / ceil["fp8_mfma_loop_TFLOPs"], 4)},
+                     "frac_of_measured_mfma_loop": round(achieved / ceil["fp8_mfma_loop_TFLOPs"], 4),
+                     "frac_of_measured_mfma_loop_with_fold": round(achieved / ceil["fp8_mfma_loop_with_fold_TFLOPs"], 4)},
         "ceilings": ceil,
     }
     if not args.no_cpu:

@@ -155,14 +155,6 @@ __device__ __forceinline__ void prefill_tile(
     // wavefront w issues A loads t*8 + w (t < A_LOADS) and B loads t*8 + w (t < B_LOADS).
     // Lane l of a load -> row 8q + l/8, LDS chunk l%8, global chunk (l%8)^f(row).
     uint32_t src_off[A_LOADS + B_LOADS];
-#pragma unroll
-    for (int t = 0; t < A_LOADS + B_LOADS; ++t) {
-        const int q = (t < A_LOADS ? t : t - A_LOADS) * 8 + wave;
-        const int row = q * 8 + (lane >> 3);                     // row inside A or B
-        const int ch = (lane & 7) ^ swz(row);
-        if (t < A_LOADS) src_off[t] = a_row(row) * (uint32_t)K + ch * 16;
-        else             src_off[t] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + ch * 16;
-    }
     // load t of K block kb into LDS stage `stage`: t < A_LOADS is the activation part, the rest the weight part
     auto issue_load = [&](int t, int kb, int stage) {
         const bool is_a = t < A_LOADS;
@@ -172,6 +164,28 @@ __device__ __forceinline__ void prefill_tile(
         __builtin_amdgcn_global_load_lds((gptr_t)(base + src_off[t] + (uint32_t)kb * 128u),
                                          (lptr_t)(lds + dst), 16, 0, 0);
     };
+    // The weight part of K block 0 is requested right here, ahead of everything that depends on the row map: a
+    // group's weights come from HBM, the longest wait of the tile's start, and a gathered row number is itself a
+    // dependent load.  The row numbers are requested first (older loads return first, so waiting for them does not
+    // wait for the copies behind them), then the four weight copies, then the activation addresses are formed.
+    uint32_t a_src_row[A_LOADS];
+#pragma unroll
+    for (int t = 0; t < A_LOADS; ++t) a_src_row[t] = a_row((t * 8 + wave) * 8 + (lane >> 3));
+    const uint32_t a_scale_row = a_row(wave * 64 + lane);
+#pragma unroll
+    for (int t = A_LOADS; t < A_LOADS + B_LOADS; ++t) {
+        const int row = ((t - A_LOADS) * 8 + wave) * 8 + (lane >> 3);
+        src_off[t] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + (((lane & 7) ^ swz(row)) * 16);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = A_LOADS; t < A_LOADS + B_LOADS; ++t) issue_load(t, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < A_LOADS; ++t) {
+        const int row = (t * 8 + wave) * 8 + (lane >> 3);
+        src_off[t] = a_src_row[t] * (uint32_t)K + (((lane & 7) ^ swz(row)) * 16);
+    }
 
     // ---- fragment read addresses.  A lane reads row (lane&15) of a 16-row sub-tile and the 32 bytes
     // at K offset 32*(lane>>4), i.e. chunks 2*(lane>>4) and 2*(lane>>4)+1, permuted by f(row).
@@ -190,13 +204,14 @@ __device__ __forceinline__ void prefill_tile(
     // requested with the tiles, read back after the block's barrier.  An ordinary global load inside the K
     // loop is not an option: issued behind the wavefront's outstanding direct-to-LDS loads it holds the
     // wavefront until those have returned -- a memory round trip per K block, measured at 30% of the kernel.
-    // Wavefronts 0-3 fetch a_s[row, kb] of 64 tile rows each (rows past the tile repeat its last row), wavefront 4
-    // the b_s rows of the two column halves (wavefronts 5-7 repeat that into slots nobody reads, which keeps the
-    // loop free of branches).
+    // Wavefronts 0-3 fetch a_s[row, kb] of 64 tile rows each (rows past the tile repeat its last row), lanes 0 and 1
+    // of wavefront 4 the b_s rows of the two column halves; every other lane of wavefronts 4-7 repeats the first of
+    // those addresses into slots nobody reads, which keeps the loop free of branches and costs one cache line per
+    // instruction instead of 64.
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
-    const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT
-                                      : (uint32_t)min(n0 / 128 + lane, nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
+    const uint32_t sc_off = (wave < 4 ? a_scale_row * (uint32_t)KBT
+                                      : (uint32_t)min(n0 / 128 + (wave == 4 ? min(lane, 1) : 0), nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
     auto issue_scales = [&](int kb, int stage) {
         __builtin_amdgcn_global_load_lds((gptr_t)(sc_base + sc_off + (uint32_t)kb),
                                          (lptr_t)(lds + LDS_SC + stage * SC_STAGE + wave * 256), 4, 0, 0);
@@ -247,13 +262,18 @@ __device__ __forceinline__ void prefill_tile(
 #define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
     auto pipeline = [&](auto ja_tag) {
         constexpr int JA = decltype(ja_tag)::value;
-        // prologue: block 0 completely, wait, barrier; then the blocks the steady state expects to be in flight:
-        // 1 .. S-2 completely and the activation part + scales of block S-1
+        // prologue: the rest of block 0 (its weight part is in flight already), then the blocks the steady state
+        // expects to be in flight -- 1 .. S-2 completely and the activation part + scales of block S-1 -- and only
+        // then the wait for block 0: everything requested after it may stay in flight across the barrier
 #pragma unroll
-        for (int t = 0; t < A_LOADS + B_LOADS; ++t) issue_load(t, 0, 0);
+        for (int t = 0; t < A_LOADS; ++t) issue_load(t, 0, 0);
         issue_scales(0, 0);
-        __builtin_amdgcn_s_waitcnt(0x0f70);             // vmcnt(0)
-        wg_barrier();
+        constexpr int kLater = [] {
+            int n = 0;
+            for (int blk = 1; blk < SS; ++blk) n += (blk < S ? A_LOADS + 1 : 0) + (blk < SB - 1 ? B_LOADS : 0);
+            return n;
+        }();
+        static_assert(kLater < 16, "vmcnt immediate");
 #pragma unroll
         for (int blk = 1; blk < SS; ++blk) {
             if (blk < S) {
@@ -266,6 +286,8 @@ __device__ __forceinline__ void prefill_tile(
                 for (int t = A_LOADS; t < A_LOADS + B_LOADS; ++t) issue_load(t, min(blk, KB - 1), blk);
             }
         }
+        __builtin_amdgcn_s_waitcnt(0x0f70 | kLater);
+        wg_barrier();
         if constexpr (JA == 0) {
             int st_a = 0, st_b = 0, st_s = 0;
             for (int kb = 0; kb < KB; ++kb) {

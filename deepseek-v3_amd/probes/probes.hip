@@ -1,5 +1,5 @@
 // Measurement probes for the benchmark (libdsv3probe.so): kernels of known traffic / arithmetic that give the
-// ceilings this GPU sustains -- a read stream, a copy, an fp8 MFMA loop and an empty launch.  They are not part of
+// ceilings this GPU sustains -- a read stream, a copy, read/write mixes, fp8 MFMA loops and an empty launch.  They are not part of
 // libdsv3fp8.so and nothing in the product path calls them.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -47,24 +47,69 @@ __global__ __launch_bounds__(kThreads) void copy_kernel(const v4i* __restrict__ 
     }
 }
 
-// 8 wavefronts per compute unit, 16 independent accumulator tiles each, nothing but v_mfma_f32_16x16x128_f8f6f4 on
-// registers: the fp8 matrix rate the chip sustains under its power limit.  Operands are pseudo-random bytes.
-__global__ __launch_bounds__(512, 1) void mfma_kernel(int iters, float* sink) {
-    const int lane = threadIdx.x & 63;
-    v8i a, b;
-    for (int i = 0; i < 8; ++i) {
-        a[i] = (int)((lane * 2654435761u + i * 40503u + blockIdx.x * 97u) | 0x01010101u) & 0x7b7b7b7b;
-        b[i] = (int)((lane * 2246822519u + i * 3266489917u) | 0x01010101u) & 0x7b7b7b7b;
+// Streams with the read : write mix of the quantisation kernels: every lane reads RD 16-byte pieces and writes WR
+// (act_quant and weight_quant read two bytes per byte written, weight_dequant writes two per byte read).
+template <int RD, int WR>
+__global__ __launch_bounds__(kThreads) void mix_kernel(const v4i* __restrict__ src, v4i* __restrict__ dst, size_t steps) {
+    constexpr int U = 4;
+    for (size_t st = blockIdx.x; st < steps; st += gridDim.x) {
+        v4i v[U][RD];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int r = 0; r < RD; ++r)
+                v[u][r] = __builtin_nontemporal_load(src + ((st * U + u) * RD + r) * kThreads + threadIdx.x);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            v4i x = v[u][0];
+#pragma unroll
+            for (int r = 1; r < RD; ++r) x ^= v[u][r];
+#pragma unroll
+            for (int w = 0; w < WR; ++w)
+                __builtin_nontemporal_store(x + (v4i){w, w, w, w}, dst + ((st * U + u) * WR + w) * kThreads + threadIdx.x);
+        }
     }
-    v4f acc[16];
-    for (int i = 0; i < 16; ++i) acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+}
+
+// 8 wavefronts per compute unit, nothing but v_mfma_f32_16x16x128_f8f6f4 on registers: the fp8 matrix rate the chip
+// sustains under its power limit.  MODE 0: one operand pair for all 16 accumulator tiles (the operand buses do not
+// toggle between instructions: the most the matrix cores issue).  MODE 1: 4 x 4 different fragments of random
+// bytes, accumulated inside the matrix core (what a GEMM with power-of-two scales issues).  MODE 2: the same
+// fragments, every product folded into its accumulator by four FMAs (what a GEMM with binary32 block scales
+// issues per 16 x 16 x 128 product).
+template <int MODE>
+__global__ __launch_bounds__(512, 1) void mfma_kernel(int iters, const int* __restrict__ rnd, float* sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    v8i a[4], b[4];
+    for (int f = 0; f < 4; ++f)
+        for (int i = 0; i < 8; ++i) {
+            const unsigned idx = (((blockIdx.x * 8 + wave) * 64 + lane) * 64 + f * 8 + i) & 0xfffff;
+            a[f][i] = rnd[idx] & 0x7b7b7b7b;                              // no NaN codes
+            b[f][i] = rnd[(idx + 32) & 0xfffff] & (int)0xfbfbfbfb;
+        }
+    if (MODE == 0) for (int f = 1; f < 4; ++f) { a[f] = a[0]; b[f] = b[0]; }
+    v4f acc[4][4];
+    for (int i = 0; i < 4; ++i) for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    const float sc = 1.0f + lane * 1e-7f;
+    v4f prev = {0.f, 0.f, 0.f, 0.f};
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int t = 0; t < 16; ++t)
-            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[t], 0, 0, 0, 0, 0, 0);
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (MODE == 2) {
+                    const v4f z = {0.f, 0.f, 0.f, 0.f};
+                    const v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[i], b[j], z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(prev[e], sc, acc[i][j][e]);
+                    prev = p;
+                } else {
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[i], b[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                }
+            }
     }
-    float r = 0.f;
-    for (int i = 0; i < 16; ++i) r += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    float r = prev[0];
+    for (int i = 0; i < 4; ++i) for (int j = 0; j < 4; ++j) r += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
     if (r == 12345.678f) sink[blockIdx.x] = r;
 }
 
@@ -97,10 +142,27 @@ int dsv3_probe_copy(const void* src, void* dst, size_t bytes, int grid, void* st
     return status();
 }
 
-// flops of one launch: 256 workgroups x 8 wavefronts x iters x 16 x 65536
-int dsv3_probe_mfma(int iters, float* sink, void* stream) {
-    if (!sink || iters <= 0) return 2;
-    hipLaunchKernelGGL(mfma_kernel, dim3(256), dim3(512), 0, (hipStream_t)stream, iters, sink);
+// reads rd and writes wr 16-byte pieces per lane and step (rd : wr = 2 : 1 or 1 : 2); bytes_read is rounded down to
+// whole steps and returned through *done_read (bytes written = that * wr / rd)
+int dsv3_probe_mix(const void* src, void* dst, size_t bytes_read, int rd, int wr, size_t* done_read, void* stream) {
+    if (!src || !dst || !((rd == 2 && wr == 1) || (rd == 1 && wr == 2))) return 2;
+    const size_t per_step = (size_t)kThreads * 4 * rd * 16;
+    const size_t steps = bytes_read / per_step;
+    if (steps == 0) return 2;
+    if (done_read) *done_read = steps * per_step;
+    const unsigned g = (unsigned)(steps < 4096 ? steps : 4096);
+    if (rd == 2) hipLaunchKernelGGL((mix_kernel<2, 1>), dim3(g), dim3(kThreads), 0, (hipStream_t)stream, (const v4i*)src, (v4i*)dst, steps);
+    else         hipLaunchKernelGGL((mix_kernel<1, 2>), dim3(g), dim3(kThreads), 0, (hipStream_t)stream, (const v4i*)src, (v4i*)dst, steps);
+    return status();
+}
+
+// flops of one launch: 256 workgroups x 8 wavefronts x iters x 16 x 65536.  rnd: 4 MiB of random bytes.
+// mode 0: constant operands, 1: changing random operands, 2: changing random operands + the fold's four FMAs
+int dsv3_probe_mfma(int iters, int mode, const void* rnd, float* sink, void* stream) {
+    if (!sink || !rnd || iters <= 0 || mode < 0 || mode > 2) return 2;
+    if (mode == 0) hipLaunchKernelGGL(mfma_kernel<0>, dim3(256), dim3(512), 0, (hipStream_t)stream, iters, (const int*)rnd, sink);
+    if (mode == 1) hipLaunchKernelGGL(mfma_kernel<1>, dim3(256), dim3(512), 0, (hipStream_t)stream, iters, (const int*)rnd, sink);
+    if (mode == 2) hipLaunchKernelGGL(mfma_kernel<2>, dim3(256), dim3(512), 0, (hipStream_t)stream, iters, (const int*)rnd, sink);
     return status();
 }
 double dsv3_probe_mfma_flops(int iters) { return 256.0 * 8.0 * iters * 16.0 * 65536.0; }
