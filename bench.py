@@ -299,7 +299,14 @@ def decode_roofline(dec: dict, ceil: dict) -> dict:
             "frac_min": min(fr), "frac_min_cell": worst, "frac_max": max(fr), "frac_max_cell": best,
             "frac_geomean": round(geo, 3),
             "frac_geomean_of_measured_read": round(geo * HBM_PEAK_GBS / ceil["hbm_read_stream_GBps"], 3),
-            "measured_read_stream_GBps": ceil["hbm_read_stream_GBps"]}
+            "measured_read_stream_GBps": ceil["hbm_read_stream_GBps"],
+            # launch time of a plain read stream over exactly the weight's bytes, divided by the GEMM's launch time
+            # (both in the same kind of graph over rotating buffers): what is left once the floor of a launch this
+            # short is taken out
+            "read_stream_same_bytes_over_gemm_time_geomean": round(math.exp(sum(
+                math.log(v["read_stream_same_bytes_us"] / v["us"]) for v in dec.values()) / len(dec)), 3),
+            "read_stream_same_bytes_over_gemm_time_M1": {k_: round(v["read_stream_same_bytes_us"] / v["us"], 3)
+                                                          for k_, v in dec.items() if k_.endswith("_M1")}}
 
 
 def run_absorb(K, W, token_counts=(1, 16, 64, 128, 4096)):
