@@ -728,8 +728,16 @@ __global__ __launch_bounds__(256) void slab_reduce_kernel(
     const int col = (int)(i - row * w);
     typename OutT<CD>::type* dst = c + row * n + n0 + col;
     if ((w & 3) == 0 && (n & 3) == 0) {
+        // all (up to eight) slabs' partial sums are requested before the first addition: a load-then-add loop pays a
+        // round trip to L2 per slab.  Slabs past the last are requested again from the last and left out of the sum.
         v4f v = {0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < slabs; ++s) v += *(const v4f*)(ws + (int64_t)s * mw + i);
+        for (int s0 = 0; s0 < slabs; s0 += 8) {
+            v4f t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = *(const v4f*)(ws + (int64_t)min(s0 + u, slabs - 1) * mw + i);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v = s0 + u < slabs ? v + t[u] : v;
+        }
         if (CD == DSV3_F32) *(v4f*)dst = v;
         else if (CD == DSV3_BF16) *(v2u*)dst = v2u{ pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]) };
         else *(v2u*)dst = v2u{ pack_f16(v[0], v[1]), pack_f16(v[2], v[3]) };

@@ -6,11 +6,13 @@
 // the workgroup's K range; their weights go straight from global memory into the MFMA register layout through a
 // ring of NPF K blocks whose loads and waits are written out explicitly (inline asm), so that exactly NPF-1
 // blocks stay in flight behind the one being multiplied.  The fifth wavefront is the PRODUCER: it copies the
-// activations the consumers share (chunks of KC K blocks x 16*MT rows, plus their scales) into double-buffered
-// LDS with global_load_lds_dwordx4.  Keeping the two streams in different wavefronts matters because vector
-// loads retire in issue order per wavefront: an activation load in a consumer's queue would force its weight
-// ring to drain at every chunk boundary.  One fence-free workgroup barrier per chunk hands a filled buffer to
-// the consumers and an emptied one back to the producer.
+// activations the consumers share (chunks of KC K blocks x 16*MT rows, plus their scales and the weight scales of
+// those K blocks) into a ring of LDS buffers with global_load_lds, AHEAD chunks ahead of the one the consumers
+// read, so that a chunk's trip from L2 is hidden behind the chunks before it (with one chunk in flight at a time
+// the chunks' round trips added up to half of the kernel).  Keeping the two streams in different wavefronts matters
+// because vector loads retire in issue order per wavefront: an activation load in a consumer's queue would force
+// its weight ring to drain at every chunk boundary.  One fence-free workgroup barrier per chunk hands a filled
+// buffer to the consumers and tells the producer that the chunk before it has been read.
 #include "common.hpp"
 #include <type_traits>
 
@@ -60,18 +62,39 @@ DSV3_WAITFOR(0) DSV3_WAITFOR(2) DSV3_WAITFOR(4) DSV3_WAITFOR(6) DSV3_WAITFOR(8) 
 #undef DSV3_WAITFOR
 
 // MT: 16-row activation sub-tiles (M <= 16*MT); NPF: ring depth in K blocks (divides the workgroup's K range);
-// KC: K blocks per activation chunk (divides NPF or is a multiple of it -- only has to divide the K range).
-template <int MT, int NPF, int KC>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void fp8_gemm_stream_kernel(
+// KC: K blocks per activation chunk (divides NPF or is a multiple of it -- only has to divide the K range);
+// AHEAD: chunks requested ahead of the one being waited for; NBUF >= AHEAD + 2 LDS buffers (when the producer
+// requests chunk c + AHEAD it has passed barrier c - 1, so the consumers are done with chunk c - 2 and older).
+template <int KC, int ROWS> struct ChunkCfg {
+    static constexpr int BYTES = KC * ROWS * 128;
+    static constexpr int DMA = BYTES / 1024;               // 1 KiB global_load_lds instructions per chunk
+    static constexpr int SC_DMA = (KC * ROWS + 63) / 64;   // 4-byte copies of the activation scales
+    static constexpr int PER = DMA + SC_DMA + 1;           // ... plus one for the weight scales
+};
+constexpr size_t lds_bytes(int kc, int rows, int nbuf) { return (size_t)nbuf * ((size_t)kc * rows * (128 + 4) + 64 * 4); }
+
+template <int N> struct ProducerWait;   // vmcnt(N)
+#define DSV3_PWAIT(N_) template <> struct ProducerWait<N_> { static __device__ __forceinline__ void on() { asm volatile("s_waitcnt vmcnt(" #N_ ")" ::: "memory"); } };
+DSV3_PWAIT(0) DSV3_PWAIT(19) DSV3_PWAIT(38) DSV3_PWAIT(57)
+#undef DSV3_PWAIT
+
+// WPE: wavefronts per SIMD the register budget is sized for (4: three workgroups of five wavefronts per compute unit,
+// 128 VGPRs; 3: one workgroup of nine, 168 VGPRs: room to read a K block's activation fragments before the wait for
+// its weights)
+template <int MT, int NPF, int KC, int AHEAD, int NBUF, int WPE = (NBUF >= 5 ? 3 : 4)>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void fp8_gemm_stream_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         void* __restrict__ out, int out_dtype,      // F32 slabs [gridDim.y][M][N] when gridDim.y > 1, else c
         int M, int N, int K, int nkb) {             // nkb: K blocks per workgroup, a multiple of NPF and of KC
     constexpr int ROWS = 16 * MT;
-    constexpr int CHUNK_BYTES = KC * ROWS * 128;
-    constexpr int DMA = CHUNK_BYTES / 1024;                // 1 KiB global_load_lds instructions per chunk
+    using CC = ChunkCfg<KC, ROWS>;
+    constexpr int CHUNK_BYTES = CC::BYTES, DMA = CC::DMA, SC_DMA = CC::SC_DMA, PER = CC::PER;
+    static_assert(NBUF >= AHEAD + 2 && AHEAD <= 3 && PER == 19, "ring of chunk buffers; the producer's counted waits");
+    static_assert((KC * ROWS) % 64 == 0, "whole wavefront copies of the activation scales");
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-    float* lds_s = (float*)(lds + 2 * CHUNK_BYTES);        // [2][KC*ROWS]: a_s * b_s
+    float* lds_as = (float*)(lds + NBUF * CHUNK_BYTES);    // [NBUF][KC*ROWS]: a_s of the chunk's rows and K blocks
+    float* lds_bs = lds_as + NBUF * (KC * ROWS);           // [NBUF][64]: b_s of the chunk's K blocks (first KC entries)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -82,9 +105,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
     const int consumers = (int)(blockDim.x >> 6) - 1, group_rows = consumers * 16;
     if (wave == consumers) {
         // ------------------------------------------------------------------ producer
+        // Everything goes global -> LDS without passing through registers: an ordinary load issued behind
+        // direct-to-LDS loads would hold the wavefront until those have landed.
         const float* bs_src = b_s + (size_t)min((int)(blockIdx.x * group_rows) >> 7, (N - 1) >> 7) * KB + kb0;
-        for (int c = 0; c < nchunks; ++c) {
-            const int buf = c & 1;
+        auto request = [&](int c) {
+            const int buf = c % NBUF;
 #pragma unroll
             for (int i = 0; i < DMA; ++i) {
                 const int R = i * 8 + (lane >> 3);                     // slab row = kbl*ROWS + m
@@ -92,12 +117,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
                 const uint8_t* src = a + (size_t)m * K + (size_t)(kb0 + kb) * 128 + (((lane & 7) ^ swz(R)) * 16);
                 __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + buf * CHUNK_BYTES + i * 1024), 16, 0, 0);
             }
-            for (int idx = lane; idx < KC * ROWS; idx += kWave) {
+#pragma unroll
+            for (int i = 0; i < SC_DMA; ++i) {
+                const int idx = i * 64 + lane;
                 const int m = min(idx % ROWS, M - 1), kb = c * KC + idx / ROWS;
-                lds_s[buf * (KC * ROWS) + idx] = a_s[(size_t)m * KB + kb0 + kb] * bs_src[kb];
+                __builtin_amdgcn_global_load_lds((gptr_t)(a_s + (size_t)m * KB + kb0 + kb),
+                                                 (lptr_t)(lds_as + buf * (KC * ROWS) + i * 64), 4, 0, 0);
             }
-            __builtin_amdgcn_s_waitcnt(0x0f70);                        // vmcnt(0): the chunk has landed
-            wg_barrier();                                              // barrier #c: chunk c is ready, chunk c-1 is consumed
+            __builtin_amdgcn_global_load_lds((gptr_t)(bs_src + c * KC + min(lane, KC - 1)), (lptr_t)(lds_bs + buf * 64), 4, 0, 0);
+        };
+        for (int c = 0; c < AHEAD && c < nchunks; ++c) request(c);
+        for (int c = 0; c < nchunks; ++c) {
+            if (c + AHEAD < nchunks) request(c + AHEAD);
+            // chunk c has landed when at most the chunks requested after it are outstanding
+            const int later = min(AHEAD, nchunks - 1 - c);
+            if (AHEAD >= 3 && later == 3) ProducerWait<57>::on();
+            else if (AHEAD >= 2 && later == 2) ProducerWait<38>::on();
+            else if (AHEAD >= 1 && later == 1) ProducerWait<19>::on();
+            else ProducerWait<0>::on();
+            wg_barrier();                                              // barrier #c: chunk c is ready, chunk c-1 has been read
         }
         return;
     }
@@ -123,21 +161,33 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
     auto step = [&](auto left_tag, int p_, v4i& lo, v4i& hi, int kbl) {
         (void)p_;
         constexpr int LEFT = decltype(left_tag)::value;
-        WaitFor<2 * LEFT>::on(lo, hi);
-        const v8i wf = untangle(lo, hi);
-        const int c = kbl / KC, t = kbl % KC;
-        const uint8_t* act = lds + (c & 1) * CHUNK_BYTES;
-        const float* sc_base = lds_s + (c & 1) * (KC * ROWS);
-#pragma unroll
-        for (int j = 0; j < MT; ++j) {
+        // With registers to spare (WPE == 3) the block's activation fragments and scales are read from LDS before the
+        // wait for its weights, so the LDS latency of MT dependent read -> MFMA pairs is not paid behind that wait.
+        constexpr bool EARLY = WPE == 3;
+        const int c = kbl / KC, t = kbl % KC, buf = c % NBUF;
+        const uint8_t* act = lds + buf * CHUNK_BYTES;
+        const float* sc_base = lds_as + buf * (KC * ROWS);
+        auto fragment = [&](int j) {
             const int R = t * ROWS + j * 16 + fr, fx = swz(R);
             const uint8_t* r = act + R * 128;
-            const v8i af = join(*(const v4i*)(r + ((fq ^ fx) * 16)), *(const v4i*)(r + (((4 + fq) ^ fx) * 16)));
-            const float sc = sc_base[R];
-            const v4f z = {0.f, 0.f, 0.f, 0.f};
-            const v4f p4 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, z, 0, 0, 0, 0, 0, 0);
+            return join(*(const v4i*)(r + ((fq ^ fx) * 16)), *(const v4i*)(r + (((4 + fq) ^ fx) * 16)));
+        };
+        v8i af[MT];
+        float sc[MT];
+        const float bs = lds_bs[buf * 64 + t];
+        if (EARLY) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[j][e] = __builtin_fmaf(p4[e], sc, acc[j][e]);
+            for (int j = 0; j < MT; ++j) { af[j] = fragment(j); sc[j] = sc_base[t * ROWS + j * 16 + fr] * bs; }
+        }
+        WaitFor<2 * LEFT>::on(lo, hi);
+        const v8i wf = untangle(lo, hi);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            if (!EARLY) { af[j] = fragment(j); sc[j] = sc_base[t * ROWS + j * 16 + fr] * bs; }
+            const v4f z = {0.f, 0.f, 0.f, 0.f};
+            const v4f p4 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af[j], z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[j][e] = __builtin_fmaf(p4[e], sc[j], acc[j][e]);
         }
     };
 
@@ -167,8 +217,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
         const int m = j * 16 + fr, n = n0 + fq * 4;
         if (m >= M) continue;
         const size_t idx = slab + (size_t)m * N + n;
-        if (out_dtype == DSV3_F32 && (N & 3) == 0 && n + 3 < N) {        // split-K slabs: one 16-byte store
-            *(v4f*)((float*)out + idx) = acc[j];
+        if ((N & 3) == 0 && n + 3 < N) {                                 // four results per store
+            if (out_dtype == DSV3_F32)       *(v4f*)((float*)out + idx) = acc[j];
+            else if (out_dtype == DSV3_BF16) *(v2u*)((uint16_t*)out + idx) = v2u{ pack_bf16(acc[j][0], acc[j][1]), pack_bf16(acc[j][2], acc[j][3]) };
+            else                             *(v2u*)((uint16_t*)out + idx) = v2u{ pack_f16(acc[j][0], acc[j][1]), pack_f16(acc[j][2], acc[j][3]) };
             continue;
         }
 #pragma unroll
@@ -184,31 +236,39 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
 struct Plan { bool ok; int mt, npf, splits, nkb, consumers; };
 
 // Usable when N gives enough groups of 64 (128) rows and the K range splits evenly into ring-sized pieces.
-inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
+// mt_min: smallest number of 16-row sub-tiles to plan for (a launch of up to 16 rows may run as two sub-tiles when the
+// K range does not divide into the one-sub-tile configuration's chunks of eight blocks).
+inline Plan make_plan_mt(int64_t m, int64_t n, int64_t k, int mt_min) {
     Plan p{};
     p.ok = false;
-    // (M <= 16 and short K ranges are served better by the kernels that split K inside the workgroup)
-    if (m <= 16 || m > 64 || k < 1024 || k % 128 || n * k >= (1ll << 32)) return p;
+    // (one and two rows and short K ranges are served better by the kernel that splits K inside the workgroup)
+    if (m < 3 || m > 64 || k < 1024 || k % 128 || n * k >= (1ll << 32)) return p;
     p.mt = (int)((m + 15) / 16);
+    if (p.mt < mt_min) p.mt = mt_min;
     if (p.mt == 3) p.mt = 4;                                    // 3 sub-tiles run as 4 (chunk size stays a power of two)
-    // eight consumer wavefronts share an activation chunk where N gives enough groups of 128 rows (half the
-    // activation traffic per weight byte: wq_b 1536 -> 24576 at 64 rows 18.0 -> 16.9 us, wq_a 15.1 -> 14.3), four
-    // otherwise (wkv_a 7168 -> 576: 11.0 against 12.5 us)
-    p.consumers = n >= 1024 ? 8 : 4;
+    // eight consumer wavefronts share an activation chunk where N gives a chip's worth of 128-row groups without
+    // splitting K (half the activation traffic per weight byte: wq_b 1536 -> 24576 at 64 rows 13.2 -> 11.6 us), four
+    // otherwise (7168 -> 1536 at 64 rows: 9.8 against 11.3 us, 7168 -> 576: 8.4 against 9.7 us)
+    p.consumers = n >= 8192 ? 8 : 4;
     const int64_t kb = k / 128, groups = (n + 16 * p.consumers - 1) / (16 * p.consumers);
-    if (groups < 4) return p;                                   // a handful of rows: not worth a streaming plan
+    // a handful of weight rows is not worth a streaming plan, and up to 16 activation rows only pay with 16 groups
+    // or more (7168 -> 1536 at 8 rows: 7.1 against 8.2 us on the M <= 16 kernel; 7168 -> 576, 9 groups: 6.8 against 6.6)
+    if (groups < (m <= 16 ? 16 : 4)) return p;
     const int64_t capacity = 256 * (p.consumers == 4 ? 3 : 1);     // resident workgroups (3 per CU with five wavefronts, 1 with nine)
-    // K blocks per workgroup: a divisor of kb that is a multiple of the ring depth; take the split count that
-    // fills one round best
+    // K blocks per workgroup: a divisor of kb that is a multiple of the ring depth.  Every K slice costs a slab of
+    // partial sums and every workgroup a start-up, so the longest range that still gives half a chip of workgroups
+    // wins (7168 -> 1536 at 64 rows: 7 slices of 8 blocks 9.8 us, 14 of 4 12.1 us, 2 of 28 17.3 us); where no range
+    // gives that many, the one with the most workgroups (7168 -> 576: 14 slices of 4 blocks).
     int best_nkb = 0, best_npf = 0;
     int64_t best_wgs = 0;
     for (int npf : {8, 4}) {
         if (npf == 8 && p.mt > 1) continue;                     // the deeper ring only fits the register budget with one sub-tile
+        if (npf == 4 && p.mt == 1) continue;                    // one sub-tile: chunks of eight K blocks only
         for (int64_t nkb = npf; nkb <= kb; nkb += npf) {
             if (kb % nkb) continue;
             const int64_t wgs = groups * (kb / nkb);
             if (wgs > capacity && (kb / nkb) > 1) continue;
-            if (wgs > best_wgs) { best_wgs = wgs; best_nkb = (int)nkb; best_npf = npf; }
+            if (wgs >= 128 || wgs > best_wgs) { best_wgs = wgs >= 128 ? 128 : wgs; best_nkb = (int)nkb; best_npf = npf; }
         }
         if (best_nkb) break;
     }
@@ -220,15 +280,36 @@ inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
     return p;
 }
 
+inline Plan make_plan(int64_t m, int64_t n, int64_t k) {
+    Plan p = make_plan_mt(m, n, k, 1);
+    // 9 .. 16 rows on a K range without chunks of eight blocks (1536 -> 24576: 12 blocks): two sub-tiles, the second
+    // one padding -- 12.4 us on the M <= 16 kernel, whose activation slab grows with the rows
+    if (!p.ok && m >= 9 && m <= 16) p = make_plan_mt(m, n, k, 2);
+    return p;
+}
+
 template <int MT, int NPF>
-void launch_cfg(const Plan& p, const void* a, const float* a_s, const void* b, const float* b_s,
+int launch_cfg(const Plan& p, const void* a, const float* a_s, const void* b, const float* b_s,
                 void* out, int od, int m, int n, int k, hipStream_t st) {
     constexpr int KC = MT == 1 ? (NPF < 8 ? NPF : 8) : (MT == 2 ? 4 : 2);
-    const size_t lds = 2 * (size_t)KC * 16 * MT * (128 + 4);
     const int group_rows = 16 * p.consumers;
     const dim3 grid((unsigned)((n + group_rows - 1) / group_rows), (unsigned)p.splits);
-    hipLaunchKernelGGL((fp8_gemm_stream_kernel<MT, NPF, KC>), grid, dim3((p.consumers + 1) * kWave), lds, st,
-                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, od, m, n, k, p.nkb);
+    if (p.consumers == 8) {
+        // one workgroup per compute unit anyway (nine wavefronts): five buffers, three chunks ahead
+        auto kern = fp8_gemm_stream_kernel<MT, NPF, KC, 3, 5>;
+        constexpr size_t lds = lds_bytes(KC, 16 * MT, 5);
+        static LdsGrant grant;
+        if (!grant.ensure((const void*)kern, (int)lds)) return DSV3_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, dim3(9 * kWave), lds, st, (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, od, m, n, k, p.nkb);
+    } else {
+        // three workgroups of five wavefronts per compute unit: three buffers (51 KiB), one chunk ahead
+        auto kern = fp8_gemm_stream_kernel<MT, NPF, KC, 1, 3>;
+        constexpr size_t lds = lds_bytes(KC, 16 * MT, 3);
+        static LdsGrant grant;
+        if (!grant.ensure((const void*)kern, (int)lds)) return DSV3_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, dim3(5 * kWave), lds, st, (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, od, m, n, k, p.nkb);
+    }
+    return launch_status();
 }
 
 }  // namespace stream
@@ -248,14 +329,12 @@ int launch_stream(const void* a, const float* a_s, const void* b, const float* b
     void* out = p.splits > 1 ? ws : c;
     const int od = p.splits > 1 ? (int)DSV3_F32 : c_dtype;
     *splits_out = p.splits;
-#define DSV3_CASE(MT_, NPF_) launch_cfg<MT_, NPF_>(p, a, a_s, b, b_s, out, od, (int)m, (int)n, (int)k, st); break
     switch (p.mt * 10 + p.npf) {
-        case 24: DSV3_CASE(2, 4);
-        case 44: DSV3_CASE(4, 4);
+        case 18: return launch_cfg<1, 8>(p, a, a_s, b, b_s, out, od, (int)m, (int)n, (int)k, st);
+        case 24: return launch_cfg<2, 4>(p, a, a_s, b, b_s, out, od, (int)m, (int)n, (int)k, st);
+        case 44: return launch_cfg<4, 4>(p, a, a_s, b, b_s, out, od, (int)m, (int)n, (int)k, st);
         default: return DSV3_ERR_BAD_SHAPE;
     }
-#undef DSV3_CASE
-    return launch_status();
 }
 
 }  // namespace dsv3

@@ -204,16 +204,46 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave, 2) void fp8_gemm_til
     }
 }
 
-// Sums the split-K slabs in a fixed order and converts to the output type.
+// Sums the split-K slabs in a fixed order (slab 0 first) and converts to the output type.  A thread owns four
+// consecutive outputs and requests eight slabs' worth of partial sums before it adds the first: written as a loop of
+// load-then-add, every slab cost a round trip to L2 (0.6-0.8 us each on the decode shapes, measured).  Slabs past the
+// last one are requested again from the last slab and left out of the sum (no "+ 0": a sum that is -0 stays -0).
 template <int CD>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(
         const float* __restrict__ ws, typename OutT<CD>::type* __restrict__ c, int64_t mn, int splits) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= mn) return;
-    float v = 0.f;
-    for (int s = 0; s < splits; ++s) v += ws[(int64_t)s * mn + i];
-    c[i] = cvt_out<CD>(v);
+    constexpr int U = 8;
+    if ((mn & 3) == 0) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < splits; s += U) {
+            v4f t[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) t[u] = *(const v4f*)(ws + (int64_t)min(s + u, splits - 1) * mn + i);
+#pragma unroll
+            for (int u = 0; u < U; ++u) v = s + u < splits ? v + t[u] : v;
+        }
+        if (CD == DSV3_F32) *(v4f*)(c + i) = v;
+        else if (CD == DSV3_BF16) *(v2u*)(c + i) = v2u{ pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]) };
+        else *(v2u*)(c + i) = v2u{ pack_f16(v[0], v[1]), pack_f16(v[2], v[3]) };
+        return;
+    }
+    const int64_t left = mn - i;                    // 1 .. 4 outputs when mn is not a multiple of four
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < splits; s += U) {
+        float t[U][4];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[u][e] = ws[(int64_t)min(s + u, splits - 1) * mn + i + (e < left ? e : 0)];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = s + u < splits ? v[e] + t[u][e] : v[e];
+    }
+    for (int e = 0; e < 4 && e < left; ++e) c[i + e] = cvt_out<CD>(v[e]);
 }
+inline unsigned splitk_reduce_grid(int64_t mn) { return (unsigned)(((mn + 3) / 4 + 255) / 256); }
 
 template <int BM, int BN, int WM, int WN, int CD>
 int launch_cfg(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
@@ -288,7 +318,7 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
                  int64_t m, int64_t n, int64_t k, void* ws, hipStream_t st, bool pow2) {
     if (k == 0) {   // empty sum: c = 0
         const int64_t mn0 = m * n;
-        hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn0 + 255) / 256)), dim3(256), 0, st,
+        hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3(splitk_reduce_grid(mn0)), dim3(256), 0, st,
                            (const float*)nullptr, (typename OutT<CD>::type*)c, mn0, 0);
         return launch_status();
     }
@@ -303,7 +333,7 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
                                   : launch_skinny(a, a_s, b, b_s, c, CD, m, n, k, ws, &splits, st);
         if (rc != DSV3_OK || splits == 1) return rc;
         const int64_t mn = m * n;
-        hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
+        hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3(splitk_reduce_grid(mn)), dim3(256), 0, st,
                            (const float*)ws, (typename OutT<CD>::type*)c, mn, splits);
         return launch_status();
     }
@@ -320,7 +350,7 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
     else            rc = launch_cfg<64, 128, 64, 32, DSV3_F32>(a, a_s, b, b_s, ws, m, n, k, p.splits, p.kb_per_split, st);
     if (rc != DSV3_OK) return rc;
     const int64_t mn = m * n;
-    hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
+    hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3(splitk_reduce_grid(mn)), dim3(256), 0, st,
                        (const float*)ws, (typename OutT<CD>::type*)c, mn, p.splits);
     return launch_status();
 }
@@ -330,10 +360,12 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
 // linear() of the reference for few rows (inference/model.py:159-160: act_quant, then fp8_gemm) as ONE launch:
 // the M <= 16 weight-streaming kernel quantises the bf16 activations itself.  Same workspace as fp8_gemm.
 // Every workgroup quantises the rows of its own K range again, so the fusion pays while the activation matrix is
-// small (16 rows x 16384: 51 us fused against 44 us in two launches; 8 rows: equal; fewer: 1 - 3 us saved).
+// small (16 rows x 16384: 51 us fused against 44 us in two launches; 8 rows: equal; fewer: 1 - 3 us saved).  Shapes
+// that fp8_gemm itself sends to another kernel (3+ rows on long K ranges: the activation-streaming kernel) are not
+// fused, so that the one call and the two calls always give the same bits.
 bool linear_fp8_supported(int64_t m, int64_t n, int64_t k) {
     return forced_kernel() != 1 && k % 128 == 0 && skinny_supported(m, n, k) && !to_large_m_kernel(m, n, k) &&
-           !(forced_kernel() == 0 && single_group_stream(m, n, k)) && m * k <= 131072;
+           !(forced_kernel() == 0 && single_group_stream(m, n, k)) && !stream_supported(m, n, k) && m * k <= 131072;
 }
 
 int launch_linear_fp8(const void* x, const void* b, const float* b_s, void* c, int c_dtype, int64_t m, int64_t n,
@@ -344,9 +376,9 @@ int launch_linear_fp8(const void* x, const void* b, const float* b_s, void* c, i
     if (rc != DSV3_OK || splits == 1) return rc;
     const int64_t mn = m * n;
     switch (c_dtype) {
-        case DSV3_BF16: hipLaunchKernelGGL((splitk_reduce_kernel<DSV3_BF16>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st, (const float*)ws, (uint16_t*)c, mn, splits); break;
-        case DSV3_F16:  hipLaunchKernelGGL((splitk_reduce_kernel<DSV3_F16>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st, (const float*)ws, (uint16_t*)c, mn, splits); break;
-        default:        hipLaunchKernelGGL((splitk_reduce_kernel<DSV3_F32>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st, (const float*)ws, (float*)c, mn, splits); break;
+        case DSV3_BF16: hipLaunchKernelGGL((splitk_reduce_kernel<DSV3_BF16>), dim3(splitk_reduce_grid(mn)), dim3(256), 0, st, (const float*)ws, (uint16_t*)c, mn, splits); break;
+        case DSV3_F16:  hipLaunchKernelGGL((splitk_reduce_kernel<DSV3_F16>), dim3(splitk_reduce_grid(mn)), dim3(256), 0, st, (const float*)ws, (uint16_t*)c, mn, splits); break;
+        default:        hipLaunchKernelGGL((splitk_reduce_kernel<DSV3_F32>), dim3(splitk_reduce_grid(mn)), dim3(256), 0, st, (const float*)ws, (float*)c, mn, splits); break;
     }
     return launch_status();
 }

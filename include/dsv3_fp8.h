@@ -196,9 +196,9 @@ int dsv3_fp8_gemm_grouped_tile_rows(void);
  * The FP8 branch of linear() for few rows, act_quant followed by fp8_gemm (inference/model.py:159-160), in one
  * launch: the weight-streaming kernel quantises the bf16 activations x [m,k] itself, with act_quant's arithmetic
  * (inference/kernel.py:23-35), so c equals dsv3_act_quant + dsv3_fp8_gemm bit for bit.  Implemented where
- * dsv3_linear_fp8_fused(m, n, k) returns non-zero (m <= 16 and m*k <= 131072 today, one or two rows on weights of 96 MiB
- * and more); other shapes return DSV3_ERR_BAD_SHAPE and the
- * caller issues the two calls.  x_dtype must be DSV3_BF16, block_size 128; workspace as for dsv3_fp8_gemm.
+ * dsv3_linear_fp8_fused(m, n, k) returns non-zero (today: shapes that dsv3_fp8_gemm sends to its M <= 16 kernel with
+ * m*k <= 131072 -- one and two rows everywhere, up to 16 rows on short K ranges or narrow weights); other shapes
+ * return DSV3_ERR_BAD_SHAPE and the caller issues the two calls.  x_dtype must be DSV3_BF16, block_size 128; workspace as for dsv3_fp8_gemm.
  */
 int dsv3_linear_fp8_fused(int64_t m, int64_t n, int64_t k);
 int dsv3_linear_fp8(const void* x, int x_dtype, const void* b, const float* b_s, void* c, int c_dtype,
