@@ -242,7 +242,7 @@ inline Plan make_plan_mt(int64_t m, int64_t n, int64_t k, int mt_min) {
     Plan p{};
     p.ok = false;
     // (one and two rows and short K ranges are served better by the kernel that splits K inside the workgroup)
-    if (m < 3 || m > 64 || k < 1024 || k % 128 || n * k >= (1ll << 32)) return p;
+    if (m < 3 || m > 64 || k < 512 || k % 128 || n * k >= (1ll << 32)) return p;
     p.mt = (int)((m + 15) / 16);
     if (p.mt < mt_min) p.mt = mt_min;
     if (p.mt == 3) p.mt = 4;                                    // 3 sub-tiles run as 4 (chunk size stays a power of two)
