@@ -261,6 +261,7 @@ inline Plan make_plan_mt(int64_t m, int64_t n, int64_t k, int mt_min) {
     // gives that many, the one with the most workgroups (7168 -> 576: 14 slices of 4 blocks).
     int best_nkb = 0, best_npf = 0;
     int64_t best_wgs = 0;
+    constexpr int64_t enough = 128;
     for (int npf : {8, 4}) {
         if (npf == 8 && p.mt > 1) continue;                     // the deeper ring only fits the register budget with one sub-tile
         if (npf == 4 && p.mt == 1) continue;                    // one sub-tile: chunks of eight K blocks only
@@ -268,7 +269,7 @@ inline Plan make_plan_mt(int64_t m, int64_t n, int64_t k, int mt_min) {
             if (kb % nkb) continue;
             const int64_t wgs = groups * (kb / nkb);
             if (wgs > capacity && (kb / nkb) > 1) continue;
-            if (wgs >= 128 || wgs > best_wgs) { best_wgs = wgs >= 128 ? 128 : wgs; best_nkb = (int)nkb; best_npf = npf; }
+            if (wgs >= enough || wgs > best_wgs) { best_wgs = wgs >= enough ? enough : wgs; best_nkb = (int)nkb; best_npf = npf; }
         }
         if (best_nkb) break;
     }

@@ -304,13 +304,17 @@ int forced_kernel() {
 }
 
 // Which problems go to the large-M kernel (K range cut into slices when the tiles do not fill the chip): every M
-// above 64, and M = 9 .. 64 when the weight is large (>= 96 MiB).  There it runs at a flat ~30 us per 117-132 MB
-// from 2 to 64 rows, while the M <= 16 streaming kernel grows with M (its K splits multiply with the rows it has
-// to stage: 31 us at 8 rows, 42-50 us at 16) and the M = 32 .. 64 streaming kernel takes 35-42 us; for the
-// smaller decode weights the streaming and tile kernels are faster.
+// above 64, and M = 9 .. 64 when the weight is large (>= 96 MiB).  There it runs at a flat 32-34 us per 117-132 MB
+// from 9 to 64 rows, while the M <= 16 streaming kernel grows with M (its K splits multiply with the rows it has
+// to stage: 31 us at 8 rows, 42-50 us at 16).  Exception: up to 32 rows on a large weight of fewer than 8192 rows go
+// to the activation-streaming kernel in its four-consumer form, two K slices (16384 -> 7168 at 17 / 32 rows 27.3 /
+// 29.1 against 33.3 / 31.6 us, 18432 -> 7168 28.6 / 29.2 against 36.4 / 32.7; at 48-64 rows and on wider weights the
+// large-M kernel is equal or faster).  For the smaller decode weights the streaming and tile kernels are faster.
 bool to_large_m_kernel(int64_t m, int64_t n, int64_t k) {
     if (!prefill_supported(m, n, k)) return false;
-    return m > 64 || (m > 8 && n * k >= (96ll << 20));
+    if (m > 64) return true;
+    if (m <= 8 || n * k < (96ll << 20)) return false;
+    return !(m <= 32 && n < 8192 && stream_supported(m, n, k));
 }
 
 template <int CD>
