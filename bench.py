@@ -292,9 +292,10 @@ def decode_roofline(dec: dict, ceil: dict) -> dict:
     best = max(dec, key=lambda k_: dec[k_]["hbm_frac"])
     geo = math.exp(sum(math.log(f) for f in fr) / len(fr))
     return {"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s", "cells": len(fr),
-            "kernels": ["fp8_gemm_skinny_kernel (M <= 16)", "fp8_gemm_stream_kernel (M = 32, 64)",
-                        "fp8_gemm_prefill / pingpong kernel, K sliced (M >= 9 on weights >= 96 MiB)",
-                        "skinny_single kernel (M = 3..16 on weights >= 96 MiB)"],
+            "kernels": ["fp8_gemm_skinny_kernel (M = 1, 2; up to 16 rows on short K or narrow N)",
+                        "fp8_gemm_stream_kernel (M = 3 .. 64; up to 32 rows on weights >= 96 MiB)",
+                        "fp8_gemm_grouped_skinny_kernel as one group (M = 3 .. 16 on weights >= 96 MiB)",
+                        "large-M kernel, K sliced (M = 33 .. 64 on weights >= 96 MiB)"],
             "bytes": "N*K + 4*ceil(N/128)*(K/128) + M*K + 4*M*K/128 + 2*M*N per launch",
             "frac_min": min(fr), "frac_min_cell": worst, "frac_max": max(fr), "frac_max_cell": best,
             "frac_geomean": round(geo, 3),
