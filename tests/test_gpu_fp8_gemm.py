@@ -59,6 +59,24 @@ def test_decode_shapes(K, kn, m):
     _check(K, x, w8, ws)
 
 
+@pytest.mark.parametrize("m,k,n", [
+    (3, 7168, 1536), (12, 7168, 1536), (16, 7168, 2112),   # one sub-tile, chunks of eight K blocks, 7 K slices
+    (5, 7168, 576),                                        # 9 groups: stays with the M <= 16 kernel
+    (12, 1536, 24576), (16, 1536, 24576),                  # K = 12 blocks: two sub-tiles, the second padding
+    (16, 512, 32768), (17, 512, 32768), (40, 512, 32768),  # K = 512: one ring round, 1 / 2 / 4 (for 3) sub-tiles
+    (17, 16384, 7168), (32, 16384, 7168),                  # a 117 MB weight of 7168 rows: four consumers, 2 K slices
+    (33, 16384, 7168),                                     # ... and the large-M kernel with K slices from 33 rows
+    (20, 1024, 8192 + 48), (64, 2048, 1000),               # ragged N on both consumer counts
+])
+def test_few_rows_on_every_streaming_plan(K, m, k, n):
+    """3 .. 64 rows: the activation-streaming kernel's plans (sub-tile counts, consumer counts, K slices with the
+    reduce pass, padded sub-tiles) and its neighbours in the dispatcher, each against the oracle."""
+    from dsv3fp8 import workloads
+    x = workloads.activations(m, k, seed=m + k % 11)
+    w8, ws = workloads.weight(n, k, seed=n % 89)
+    _check(K, x, w8, ws)
+
+
 @pytest.mark.parametrize("m", [65, 100, 128, 257, 300])
 def test_mid_m(K, m):
     from dsv3fp8 import workloads
