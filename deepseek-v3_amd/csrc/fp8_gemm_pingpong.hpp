@@ -16,15 +16,15 @@
 // work, and the matrix pipe sees an uninterrupted instruction stream from one wavefront at a time.
 //
 // LDS: two stages of [256 rows of A | 256 rows of B] x 128 bytes (the chunk permutation of fp8_gemm_prefill.hip)
-// and four slots of scales.  With block kb in stage kb % 2 and phases numbered from group 0's M1 of block 0:
-//     region                      last read in phase    refilled (block kb + 2) in phase    first read again
-//     A, B columns 0-63 of both   4 kb + 1              4 kb + 2 .. 4 kb + 4                4 kb + 8
-//     B columns 64-127 of both    4 kb + 3              4 kb + 5                            4 kb + 10
-// so every copy has at least one whole K block of time to land.  Group 0 requests, per block kb, the second half of
-// A of block kb + 1 in M1 and the first-columns part of B of block kb + 2 in M2; group 1 the last-columns part of B
-// of block kb + 1 in M1 and the first half of A of block kb + 2 in M2.  Copies retire in program order, so "the
-// copies the next readers need have landed" is a vmcnt(n) with n = the number of younger copies: 9 for group 1 at
-// the end of both M phases, 4 for group 0 at the end of C2.
+// and two slots of scales; block kb lives in stage kb % 2.  Which wavefront copies what, and when, is laid out at
+// the copy plan below: per block a wavefront requests two copies of block kb + 1 in M1 and six of block kb + 2 plus
+// the scales in M2, every region is refilled only after its last reader's phase has ended, and every copy has at
+// least one whole K block of time to land.  Copies retire in program order, so "the copies the next readers need have
+// landed" is a vmcnt(n) with n = the number of younger copies: 9, at the end of both M phases for group 1 and of
+// both C phases for group 0.
+//
+// Grouped mode (G): the tile is a slot of the grouped GEMM's tile table (a row range of one group, multiplied by that
+// group's weights, activation rows gathered through a row map) -- used for slots of more than 192 rows.
 #pragma once
 
 namespace pingpong {
@@ -76,17 +76,29 @@ constexpr int LDS_A = 0, LDS_B = 2 * STAGE, LDS_SC = 4 * STAGE;
 constexpr int SC_SLOT = 2048, SC_SLOTS = 2;
 constexpr int LDS_BYTES = LDS_SC + SC_SLOTS * SC_SLOT;  // 136 KiB
 
-template <int CD, bool P2>
+template <int CD, bool P2, bool G = false>
 __device__ __forceinline__ void tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
-        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, int wg) {
+        int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, int wg,
+        const GroupTable& g = GroupTable{}) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
-    // ---- workgroup -> tile: a contiguous run of tiles per XCD, walked in bands of GROUP_M tile rows
+    // ---- workgroup -> tile: a contiguous run of tiles per XCD, walked in bands of GROUP_M tile rows; in grouped
+    // mode the row tiles are dealt round-robin over the XCDs and the column tiles of a row tile stay on one XCD
+    // (the mapping of the grouped kernel, whose dispatch has already checked that the slot is in use)
     int m0, n0, rows_here;
-    {
+    if (G) {
+        const int x = wg % 8, idx = wg / 8;
+        const int tm = (idx / tiles_n) * 8 + x, tn = idx - (idx / tiles_n) * tiles_n;
+        const int expert = g.tile_group[tm];
+        m0 = g.tile_row0[tm];
+        rows_here = g.tile_rows[tm];
+        n0 = (tn_first + tn) * BN;
+        b += (size_t)expert * g.b_stride;
+        b_s += (size_t)expert * g.bs_stride;
+    } else {
         const int T = tiles_m * tiles_n;
         int pid = wg;
         {
@@ -102,7 +114,11 @@ __device__ __forceinline__ void tile(
         m0 = tm * TM; n0 = (tn_first + tn) * BN;
         rows_here = min(TM, M - m0);
     }
-    auto a_row = [&](int r) -> uint32_t { return (uint32_t)(((DSV3_PP_ABL & 16) ? 0 : m0) + min(r, rows_here - 1)); };
+    // row of a behind row r of the tile; rows past the tile's end repeat its last row (their results are dropped)
+    auto a_row = [&](int r) -> uint32_t {
+        const int rr = ((DSV3_PP_ABL & 16) ? 0 : m0) + min(r, rows_here - 1);
+        return (uint32_t)((G && g.a_rows) ? g.a_rows[rr] : rr);
+    };
     const int n0_ld = (DSV3_PP_ABL & 16) ? 0 : n0;
 
     const int tid = threadIdx.x, lane = tid & 63;

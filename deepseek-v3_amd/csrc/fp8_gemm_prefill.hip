@@ -605,7 +605,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 }
 
 // Grouped GEMM over a tile table with slots of up to 256 rows.  A slot with more than 192 rows runs the 256-row
-// configuration (the weights pass through LDS once for up to 256 rows), one with 129 .. 192 rows a 192-row
+// two-phase kernel (the weights pass through LDS once for up to 256 rows), one with 129 .. 192 rows a 192-row
 // configuration whose smaller activation stages leave room for a third weight stage (a group's weights come
 // straight from HBM, and a second block of prefetch is what hides that), one with fewer the 128-row
 // configuration with three stages of both.  The choice is uniform over the workgroup and needs no host knowledge of
@@ -619,8 +619,10 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
     const int idx = blockIdx.x / 8, tm = (idx / tiles_n) * 8 + blockIdx.x % 8;
     if (tm >= tiles_m) return;
     const int rows = g.tile_rows[tm];
-    if (rows > 192)
-        prefill_tile<CD, true, 256, 2, 2, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+    if (rows > 192) {
+        if (g.tile_group[tm] < 0) return;
+        pingpong::tile<CD, P2, true>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x, g);
+    }
     else if (rows > 128)
         prefill_tile<CD, true, 192, 2, 3, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
     else
@@ -890,7 +892,7 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
                                      b_stride, bs_stride, m < num_tiles ? m : num_tiles, stream);
     GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
     constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES;               // the largest of the three configurations
-    static_assert(LDS_BYTES >= Cfg<256, 2>::LDS_BYTES && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES, "LDS of the grouped kernel");
+    static_assert(LDS_BYTES >= pingpong::LDS_BYTES && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES, "LDS of the grouped kernel");
     const int64_t tn = (n + BN - 1) / BN;
     if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (num_tiles * tn == 0) return DSV3_OK;
