@@ -69,14 +69,22 @@ __device__ __forceinline__ void copy4(const void* base, uint32_t lane_off, uint3
                  :: "v"(lane_off), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
-constexpr int TM = 256;
-constexpr int SM = 4;                                   // 16-row sub-tiles per wavefront
-constexpr int STAGE = 256 * 128;                        // bytes of A (or of B) per K block
-constexpr int LDS_A = 0, LDS_B = 2 * STAGE, LDS_SC = 4 * STAGE;
+// SM: 16-row sub-tiles per wavefront.  4: the 256-row tile described above.  2: a 128-row tile (32 x 128 per
+// wavefront, eight MFMAs per C phase) for problems whose row count or tile count does not fill rounds of 256-row
+// tiles; its A stage is half as large and all of it is copied by group 1.
+template <int SM> struct Geo {
+    static_assert(SM == 2 || SM == 4, "128- or 256-row tiles");
+    static constexpr int WM = 16 * SM, TM = 4 * WM;
+    static constexpr int A_STAGE = TM * 128, B_STAGE = 256 * 128;       // bytes of A / of B per K block
+    static constexpr int LDS_A = 0, LDS_B = 2 * A_STAGE, LDS_SC = 2 * A_STAGE + 2 * B_STAGE;
+    static constexpr int NM2 = SM == 4 ? 6 : 4;                         // copies per wavefront in M2 (plus the scales)
+    static constexpr int WAIT = NM2 + 1 + 2;                            // copies younger than the ones a phase end waits for
+};
 constexpr int SC_SLOT = 2048, SC_SLOTS = 2;
-constexpr int LDS_BYTES = LDS_SC + SC_SLOTS * SC_SLOT;  // 136 KiB
+template <int SM> constexpr int lds_bytes() { return Geo<SM>::LDS_SC + SC_SLOTS * SC_SLOT; }
+constexpr int LDS_BYTES = lds_bytes<4>();               // 136 KiB (100 KiB for the 128-row tile)
 
-template <int CD, bool P2, bool G = false>
+template <int CD, bool P2, bool G = false, int SM = 4>
 __device__ __forceinline__ void tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -84,6 +92,10 @@ __device__ __forceinline__ void tile(
         int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, int wg,
         const GroupTable& g = GroupTable{}) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    using GEO = Geo<SM>;
+    constexpr int TM = GEO::TM, WM = GEO::WM, A_STAGE = GEO::A_STAGE, B_STAGE = GEO::B_STAGE;
+    constexpr int LDS_A = GEO::LDS_A, LDS_B = GEO::LDS_B, LDS_SC = GEO::LDS_SC, NM2 = GEO::NM2;
+    static_assert(!G || SM == 4, "grouped slots run the 256-row tile");
 
     // ---- workgroup -> tile: a contiguous run of tiles per XCD, walked in bands of GROUP_M tile rows; in grouped
     // mode the row tiles are dealt round-robin over the XCDs and the column tiles of a row tile stay on one XCD
@@ -131,16 +143,18 @@ __device__ __forceinline__ void tile(
     const int n_base = ldc == N ? 0 : tn_first * BN;
     a += (size_t)kb0 * 128u; b += (size_t)kb0 * 128u;
 
-    // ---- copy plan.  A K block is 32 + 32 wavefront-copies of 8 rows (1 KiB); copy q covers rows 8q .. 8q + 7.
+    // ---- copy plan.  A K block is TM / 8 + 32 wavefront-copies of 8 rows (1 KiB); copy q covers rows 8q .. 8q + 7.
     // The copies are requested in the M phases, interleaved with the LDS reads (the copy path takes one 1 KiB copy
     // per ~16 cycles and compute unit and holds the issuing wavefront meanwhile; a wavefront in a C phase that
     // issued them would leave gaps in its MFMA stream).  Per block kb a wavefront issues
     //   in M1  two copies of block kb + 1:  B rows 64-127 (group 0) / 192-255 (group 1), the last-columns part
-    //   in M2  six copies of block kb + 2:  group 0  B rows 0-63 and 128-191 (4) and A rows 0-63 (2)
-    //                                       group 1  A rows 64-255 (6)
-    uint32_t m1_src[2], m2_src[6];
-    int m1_dst[2], m2_dst[6];
-    const uint8_t* m2_base[6];
+    //   in M2  NM2 copies of block kb + 2:  256-row tile  group 0  B rows 0-63 and 128-191 (4) and A rows 0-63 (2)
+    //                                                     group 1  A rows 64-255 (6)
+    //                                       128-row tile  group 0  B rows 0-63 and 128-191 (4)
+    //                                                     group 1  A rows 0-127 (4)
+    uint32_t m1_src[2], m2_src[NM2];
+    int m1_dst[2], m2_dst[NM2];
+    const uint8_t* m2_base[NM2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         const int q = (grp == 0 ? 8 : 24) + wm * 2 + t;
@@ -149,21 +163,23 @@ __device__ __forceinline__ void tile(
         m1_dst[t] = LDS_B + q * 1024;
     }
 #pragma unroll
-    for (int t = 0; t < 6; ++t) {
+    for (int t = 0; t < NM2; ++t) {
         const bool from_b = grp == 0 && t < 4;
         int q;
         if (grp == 0) { const int idx = wm * 4 + t; q = t < 4 ? (idx < 8 ? idx : idx + 8) : wm * 2 + (t - 4); }
-        else q = 8 + wm * 6 + t;
+        else q = SM == 4 ? 8 + wm * 6 + t : wm * 4 + t;
         const int r = q * 8 + (lane >> 3), ch = (lane & 7) ^ swz(r);
         m2_src[t] = (from_b ? (uint32_t)min(n0_ld + r, N - 1) : a_row(r)) * (uint32_t)K + ch * 16;
         m2_dst[t] = (from_b ? LDS_B : LDS_A) + q * 1024;
         m2_base[t] = from_b ? b : a;
     }
+    // (a stage of the weight region and one of the activation region have different sizes in the 128-row tile)
     auto issue_m1 = [&](int t, int kb, int stage) {
-        copy16(b + (uint32_t)kb * 128u, m1_src[t], lds_addr_of(lds + m1_dst[t] + stage * STAGE));
+        copy16(b + (uint32_t)kb * 128u, m1_src[t], lds_addr_of(lds + m1_dst[t] + stage * B_STAGE));
     };
     auto issue_m2 = [&](int t, int kb, int stage) {
-        copy16(m2_base[t] + (uint32_t)kb * 128u, m2_src[t], lds_addr_of(lds + m2_dst[t] + stage * STAGE));
+        const bool from_b = grp == 0 && t < 4;
+        copy16(m2_base[t] + (uint32_t)kb * 128u, m2_src[t], lds_addr_of(lds + m2_dst[t] + stage * (from_b ? B_STAGE : A_STAGE)));
     };
     // scales of a K block: wavefronts 0-3 copy a_s[row, kb] of 64 tile rows each, wavefront 4 the b_s rows of the two
     // column halves (lanes 0 and 1; its other lanes and wavefronts 5-7 repeat an address already requested, so that
@@ -180,9 +196,9 @@ __device__ __forceinline__ void tile(
     const int fr = lane & 15, fq = lane >> 4;
     const int fx = swz(fr);
     const int c0 = ((2 * fq) ^ fx) * 16, c1 = ((2 * fq + 1) ^ fx) * 16;
-    const uint8_t* a_rd = lds + LDS_A + (wm * 64 + fr) * 128;           // + j * 2048 + stage * STAGE
-    const uint8_t* b_rd = lds + LDS_B + (grp * 128 + fr) * 128;         // + i * 2048 + stage * STAGE
-    const uint8_t* sa_rd = lds + LDS_SC + (wm * 64 + fr) * 4;           // + j * 64 + slot * SC_SLOT
+    const uint8_t* a_rd = lds + LDS_A + (wm * WM + fr) * 128;           // + j * 2048 + stage * A_STAGE
+    const uint8_t* b_rd = lds + LDS_B + (grp * 128 + fr) * 128;         // + i * 2048 + stage * B_STAGE
+    const uint8_t* sa_rd = lds + LDS_SC + (wm * WM + fr) * 4;           // + j * 64 + slot * SC_SLOT
     const uint8_t* sb_rd = lds + LDS_SC + (256 + grp) * 4;
 
     v4f acc[8][SM];
@@ -197,12 +213,12 @@ __device__ __forceinline__ void tile(
         constexpr bool LD = !(DSV3_PP_ABL & 2), RD = !(DSV3_PP_ABL & 4);
         // prologue: blocks 0 and 1 as far as the steady state expects them to have been requested
 #pragma unroll
-        for (int t = 0; t < 6; ++t) issue_m2(t, 0, 0);
+        for (int t = 0; t < NM2; ++t) issue_m2(t, 0, 0);
         issue_scales(0, 0);
 #pragma unroll
         for (int t = 0; t < 2; ++t) issue_m1(t, 0, 0);
 #pragma unroll
-        for (int t = 0; t < 6; ++t) issue_m2(t, min(1, KB - 1), 1);
+        for (int t = 0; t < NM2; ++t) issue_m2(t, min(1, KB - 1), 1);
         issue_scales(min(1, KB - 1), 1);
         __builtin_amdgcn_s_waitcnt(0x0f70);                         // vmcnt(0)
         wg_barrier();
@@ -215,12 +231,13 @@ __device__ __forceinline__ void tile(
 #pragma unroll
         for (int j = 0; j < SM; ++j) { sc[0][j] = sc[1][j] = 0.f; ea[j] = 0; }
 
-        // 16 MFMAs over column sub-tiles I0 .. I0 + 3 with the fold factors s; every MFMA is followed by the four
+        // 4 SM MFMAs over column sub-tiles I0 .. I0 + 3 with the fold factors s; every MFMA is followed by the four
         // FMAs of the MFMA issued two earlier -- the first two by those of the previous C phase's last two MFMAs
         // (column sub-tile IT, fold factors st), so that the M phases hold no vector ALU work: while the other
         // wavefront of the SIMD is in a C phase, the vector ALU issues this wavefront's instructions only in the gaps.
         auto compute = [&](auto i0_tag, auto it_tag, const float (&s)[SM], const float (&st)[SM]) {
             constexpr int I0 = decltype(i0_tag)::value, IT = decltype(it_tag)::value;
+            constexpr int NT = 4 * SM;
             __builtin_amdgcn_sched_barrier(0);
             if (DSV3_PP_ABL & 1) __builtin_amdgcn_s_setprio(1);
             if constexpr (P2) {
@@ -232,26 +249,26 @@ __device__ __forceinline__ void tile(
                             bf[ii], af[j], acc[I0 + ii][j], 0, 0, 0, eb, 0, ea[j]);
             } else {
                 const v4f z = {0.f, 0.f, 0.f, 0.f};
-                v4f p[16];
+                v4f p[NT];
 #pragma unroll
-                for (int t = 0; t < 16; ++t) {
-                    p[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[t / 4], af[t % 4], z, 0, 0, 0, 0, 0, 0);
+                for (int t = 0; t < NT; ++t) {
+                    p[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[t / SM], af[t % SM], z, 0, 0, 0, 0, 0, 0);
                     if (!(DSV3_PP_ABL & 8)) {
                         if (t < 2) {
                             const v4f q = t == 0 ? p14 : p15;
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) acc[IT][2 + t][e] = __builtin_fmaf(q[e], st[2 + t], acc[IT][2 + t][e]);
+                            for (int e = 0; e < 4; ++e) acc[IT][SM - 2 + t][e] = __builtin_fmaf(q[e], st[SM - 2 + t], acc[IT][SM - 2 + t][e]);
                         } else {
                             const int u = t - 2;
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                acc[I0 + u / 4][u % 4][e] = __builtin_fmaf(p[u][e], s[u % 4], acc[I0 + u / 4][u % 4][e]);
+                                acc[I0 + u / SM][u % SM][e] = __builtin_fmaf(p[u][e], s[u % SM], acc[I0 + u / SM][u % SM][e]);
                         }
                     }
                     DSV3_SGB(0x008, 1);
                     if (!(DSV3_PP_ABL & 8)) DSV3_SGB(0x002, 4);
                 }
-                p14 = p[14]; p15 = p[15];
+                p14 = p[NT - 2]; p15 = p[NT - 1];
             }
             if (DSV3_PP_ABL & 1) __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
@@ -265,11 +282,11 @@ __device__ __forceinline__ void tile(
             const int kb1 = min(kb + 1, KB - 1), kb2 = min(kb + 2, KB - 1);
             // ---- M1
             if (RD || kb == 0) {
-                const uint8_t* as_base = a_rd + ST * STAGE;
-                const uint8_t* bs_base = b_rd + ST * STAGE;
+                const uint8_t* as_base = a_rd + ST * A_STAGE;
+                const uint8_t* bs_base = b_rd + ST * B_STAGE;
 #pragma unroll
                 for (int j = 0; j < SM; ++j) {
-                    if (LD && j % 2 == 0) issue_m1(j / 2, kb1, ST ^ 1);
+                    if (LD && j % (SM / 2) == 0) issue_m1(j / (SM / 2), kb1, ST ^ 1);
                     af[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
                 }
 #pragma unroll
@@ -288,34 +305,38 @@ __device__ __forceinline__ void tile(
             }
             __builtin_amdgcn_sched_barrier(0);
             PP_PROF_MARK(0)
-            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | 9);
+            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT);
             wg_barrier();
             PP_PROF_MARK(1)
             // ---- C1 (its first two FMA groups belong to C2 of the previous block: zeros at kb = 0)
             compute(std::integral_constant<int, 0>{}, std::integral_constant<int, 7>{}, sc[ST], sc[ST ^ 1]);
             PP_PROF_MARK(2)
-            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | 9);
+            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT);
             wg_barrier();
             PP_PROF_MARK(3)
             // ---- M2
             {
-                const uint8_t* bs_base = b_rd + ST * STAGE + 4 * 2048;
+                const uint8_t* bs_base = b_rd + ST * B_STAGE + 4 * 2048;
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
                     if (LD) issue_m2(ii, kb2, ST);
                     if (RD) bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
                 }
-                if (LD) { issue_m2(4, kb2, ST); issue_m2(5, kb2, ST); issue_scales(kb2, ST); }
+                if (LD) {
+#pragma unroll
+                    for (int t = 4; t < NM2; ++t) issue_m2(t, kb2, ST);
+                    issue_scales(kb2, ST);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
             PP_PROF_MARK(4)
-            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | 9);
+            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT);
             wg_barrier();
             PP_PROF_MARK(5)
             // ---- C2
             compute(std::integral_constant<int, 4>{}, std::integral_constant<int, 3>{}, sc[ST], sc[ST]);
             PP_PROF_MARK(6)
-            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | 9);
+            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT);
             wg_barrier();
             PP_PROF_MARK(7)
         };
@@ -332,8 +353,8 @@ __device__ __forceinline__ void tile(
             const int last = (KB - 1) & 1;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                acc[7][2][e] = __builtin_fmaf(p14[e], last ? sc[1][2] : sc[0][2], acc[7][2][e]);
-                acc[7][3][e] = __builtin_fmaf(p15[e], last ? sc[1][3] : sc[0][3], acc[7][3][e]);
+                acc[7][SM - 2][e] = __builtin_fmaf(p14[e], last ? sc[1][SM - 2] : sc[0][SM - 2], acc[7][SM - 2][e]);
+                acc[7][SM - 1][e] = __builtin_fmaf(p15[e], last ? sc[1][SM - 1] : sc[0][SM - 1], acc[7][SM - 1][e]);
             }
         }
         if (GRP == 0) wg_barrier();                                 // group 1's last phase
@@ -346,7 +367,7 @@ __device__ __forceinline__ void tile(
 #undef DSV3_SGB
 
     // ---- epilogue: lane holds c[m][n .. n + 3] for every (i, j); see fp8_gemm_prefill.hip for the LDS route
-    constexpr int WM = 64, WN = 128, SN = 8;
+    constexpr int WN = 128, SN = 8;
     auto sub_row = [&](int j) { return wm * WM + j * 16; };
     const bool lds_epilogue = CD != DSV3_F32 && (N % 8) == 0 && ldc == N;
     const bool f32_lds_epilogue = CD == DSV3_F32 && (N % 4) == 0 && (ldc % 4) == 0;

@@ -585,14 +585,15 @@ __device__ __forceinline__ void prefill_tile(
 #include "fp8_gemm_pingpong.hpp"
 
 inline bool use_pingpong() { static const bool v = getenv("DSV3_PREFILL_NOPP") == nullptr; return v; }
+inline bool use_pingpong_short() { static const bool v = use_pingpong() && getenv("DSV3_PREFILL_NOPP128") == nullptr; return v; }
 
-template <int CD, bool P2 = false>
+template <int CD, bool P2 = false, int SM = 4>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_pingpong_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
         int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc) {
-    pingpong::tile<CD, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x);
+    pingpong::tile<CD, P2, false, SM>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x);
 }
 
 template <int CD, bool G, int TM, int S, bool P2 = false>
@@ -633,7 +634,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
 // tiles over the column tiles [0, tn_tall), the others 128-row tiles over [tn_tall, tn_tall + tn_short).  Workgroups
 // are handed out in index order, so the short tiles fill the compute units that the last, partly filled round of
 // tall tiles would leave idle.
-template <int CD, bool P2 = false, bool PP = true>
+template <int CD, bool P2 = false, bool PP = true, bool PPS = true>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_two_heights_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -644,9 +645,12 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_two_heights_kernel(
     if ((int)blockIdx.x < n_tall) {
         if constexpr (PP) pingpong::tile<CD, P2>(a, a_s, b, b_s, c, M, N, K, tm_tall, tn_tall, 0, K / 128, N, blockIdx.x);
         else prefill_tile<CD, false, 256, 2, 2, P2>(a, a_s, b, b_s, c, M, N, K, tm_tall, tn_tall, 0, K / 128, N, none, blockIdx.x);
-    } else if ((int)blockIdx.x >= short_first)
-        prefill_tile<CD, false, 128, 3, 3, P2>(a, a_s, b, b_s, c, M, N, K, (M + 127) / 128, tn_short, tn_tall, K / 128, N, none,
-                                        blockIdx.x - short_first);
+    } else if ((int)blockIdx.x >= short_first) {
+        if constexpr (PPS) pingpong::tile<CD, P2, false, 2>(a, a_s, b, b_s, c, M, N, K, (M + 127) / 128, tn_short, tn_tall, K / 128, N,
+                                                            blockIdx.x - short_first);
+        else prefill_tile<CD, false, 128, 3, 3, P2>(a, a_s, b, b_s, c, M, N, K, (M + 127) / 128, tn_short, tn_tall, K / 128, N, none,
+                                                    blockIdx.x - short_first);
+    }
 }
 
 }  // namespace prefill
@@ -666,14 +670,15 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
     constexpr int LDS_BYTES = Cfg<TM, S>::LDS_BYTES;
     if ((tm + 8) * tn_count > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (tm * tn_count == 0) return DSV3_OK;
-    if constexpr (!G && TM == 256) {
-        if (use_pingpong()) {
-            auto pp = fp8_gemm_pingpong_kernel<CD, P2>;
+    if constexpr (!G && (TM == 256 || TM == 128)) {
+        if (TM == 256 ? use_pingpong() : use_pingpong_short()) {
+            constexpr int SM = TM / 64, PP_LDS = pingpong::lds_bytes<SM>();
+            auto pp = fp8_gemm_pingpong_kernel<CD, P2, SM>;
             static LdsGrant pp_grant;
-            if (!pp_grant.ensure((const void*)pp, pingpong::LDS_BYTES)) return DSV3_ERR_LAUNCH;
+            if (!pp_grant.ensure((const void*)pp, PP_LDS)) return DSV3_ERR_LAUNCH;
             const int kbt = (int)(k / 128), per = (kbt + splits - 1) / splits;
             hipLaunchKernelGGL(pp, dim3((unsigned)(tm * tn_count), (unsigned)((kbt + per - 1) / per)), dim3(THREADS),
-                               pingpong::LDS_BYTES, stream, (const uint8_t*)a, a_s, (const uint8_t*)b, b_s,
+                               PP_LDS, stream, (const uint8_t*)a, a_s, (const uint8_t*)b, b_s,
                                (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)tm, (int)tn_count, (int)tn_first,
                                per, (int)(ldc ? ldc : n));
             return launch_status();
@@ -838,9 +843,10 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
         using namespace prefill;
         constexpr int LDS_OLD = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
         constexpr int LDS_BYTES = LDS_OLD > pingpong::LDS_BYTES ? LDS_OLD : pingpong::LDS_BYTES;
-        const bool pp = use_pingpong();
-        auto kern = pp ? fp8_gemm_two_heights_kernel<CD, P2, true> : fp8_gemm_two_heights_kernel<CD, P2, false>;
-        static LdsGrant grant[2];
+        const int pp = use_pingpong() ? (use_pingpong_short() ? 2 : 1) : 0;
+        auto kern = pp == 2 ? fp8_gemm_two_heights_kernel<CD, P2, true, true>
+                  : pp == 1 ? fp8_gemm_two_heights_kernel<CD, P2, true, false> : fp8_gemm_two_heights_kernel<CD, P2, false, false>;
+        static LdsGrant grant[3];
         if (!grant[pp].ensure((const void*)kern, LDS_BYTES)) return DSV3_ERR_LAUNCH;
         const int64_t n_tall = (m + 255) / 256 * p.tn_plain;
         const int64_t grid = (n_tall + 7) / 8 * 8 + (m + 127) / 128 * p.tn_short;
