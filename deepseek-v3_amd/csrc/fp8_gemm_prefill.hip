@@ -765,6 +765,8 @@ PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
     static const bool nosplit = getenv("DSV3_PREFILL_NOSPLIT") != nullptr;
     PrefillPlan best{128, (int)tn, 1, 0};
     int64_t best_cost = -1;
+    // a round of 128-row tiles against one of 256-row tiles (152): 0.60 on the two-phase kernel, 0.66 on the single-phase one
+    const int64_t short_unit = prefill::use_pingpong_short() ? 91 : 100;
     auto slices_for = [&](int64_t tiles) {       // K slices that keep `tiles` within one round
         int64_t s = tiles > 0 ? kCUs / tiles : 1;
         if (s > kb / 8) s = kb / 8;
@@ -776,7 +778,7 @@ PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
     auto slab_cost = [&](int64_t slabs, int64_t cols) { return 300 + slabs * m * cols * 12 / 100000; };
     for (int h : {128, 256}) {
         if (forced && forced != h) continue;
-        const int64_t unit = h == 128 ? 100 : (prefill::use_pingpong() ? 152 : 164), tm = (m + h - 1) / h, tiles = tm * tn;
+        const int64_t unit = h == 128 ? short_unit : (prefill::use_pingpong() ? 152 : 164), tm = (m + h - 1) / h, tiles = tm * tn;
         // plain or sliced over all columns
         {
             const int64_t s = slices_for(tiles), per = (kb + s - 1) / s, slabs = (kb + per - 1) / per;
@@ -805,14 +807,14 @@ PrefillPlan prefill_plan(int64_t m, int64_t n, int64_t k) {
         for (int64_t c = 1; c < tn && c <= 32; ++c) {
             const int64_t n_tall = tm_tall * (tn - c), n_short = tm_short * c;
             const int64_t q = n_tall / kCUs, r = n_tall % kCUs;
-            // kCUs - r units carry lo = q * tall, r units hi = lo + tall; the short tiles (100 each) go to whichever
+            // kCUs - r units carry lo = q * tall, r units hi = lo + tall; the short tiles (short_unit each) go to whichever
             // unit is free first, level by level
             const int64_t tall = prefill::use_pingpong() ? 152 : 164;
             const int64_t lo = q * tall, hi = lo + tall;
-            int64_t t = lo, t_lo = lo + 100, t_hi = hi + 100, done = 0;
+            int64_t t = lo, t_lo = lo + short_unit, t_hi = hi + short_unit, done = 0;
             while (done < n_short) {
-                if (r == 0 || t_lo <= t_hi) { t = t_lo; t_lo += 100; done += kCUs - r; }
-                else                        { t = t_hi; t_hi += 100; done += r; }
+                if (r == 0 || t_lo <= t_hi) { t = t_lo; t_lo += short_unit; done += kCUs - r; }
+                else                        { t = t_hi; t_hi += short_unit; done += r; }
             }
             const int64_t span = (r > 0 && hi > t) ? hi : t;
             const int64_t cost = span * kb + 100;                // (a little extra: prefer one height at equal cost)
