@@ -69,7 +69,23 @@ template <int CTRL> __device__ __forceinline__ float dpp_max(float v) {
     return fmaxf(v, __builtin_bit_cast(float, o));
 }
 
-template <int MT, int S, int NPF, bool QF>
+// 16-byte non-temporal load from (scalar base + 32-bit lane offset + immediate), and a wait until at most n vector
+// loads of the wavefront are outstanding with the ring slot threaded through it (so that the slot's consumers cannot
+// be scheduled ahead of the wait): the RING variant's weight loads and waits are written out, because the compiler's
+// own counting of outstanding loads falls back to "all of them" across a loop's back edge.
+#define DSV3_GLOAD(dst, voff, sbase, imm) \
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:" #imm " nt" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory")
+#define DSV3_WAIT(n, lo, hi) asm volatile("s_waitcnt vmcnt(" #n ")" : "+v"(lo), "+v"(hi) :: "memory")
+template <int N> struct WaitFor;
+#define DSV3_WAITFOR(N_) template <> struct WaitFor<N_> { static __device__ __forceinline__ void on(v4i& lo, v4i& hi) { DSV3_WAIT(N_, lo, hi); } };
+DSV3_WAITFOR(0) DSV3_WAITFOR(2) DSV3_WAITFOR(4) DSV3_WAITFOR(6) DSV3_WAITFOR(8) DSV3_WAITFOR(10) DSV3_WAITFOR(12) DSV3_WAITFOR(14)
+#undef DSV3_WAITFOR
+
+// RING (S == 1, every wavefront's K range a multiple of NPF blocks and at least two of them, n k < 2^32): a ring slot
+// is refilled as soon as its block has been multiplied, so a wavefront keeps NPF blocks of loads in flight until its
+// last NPF blocks.  Without it the range is worked through in batches -- issue NPF, use NPF, issue the next NPF --,
+// a wavefront has nothing in flight while it uses a batch, and all wavefronts of the chip reach that point together.
+template <int MT, int S, int NPF, bool QF, bool RING = false>
 __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 4))) void fp8_gemm_skinny_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -156,9 +172,20 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
             whi[p][s] = __builtin_nontemporal_load((const v4i*)(wsrc[s] + wrow8[s] + k * 128));    // rows 8..15
         }
     };
+    // RING: lane offsets of its two rows from b (< 2^32) and the wavefront-uniform address of its first K block
+    static_assert(!RING || (S == 1 && NPF == 8), "the ring variant is written for one strip and eight slots");
+    const uint32_t ring_lo = (uint32_t)min(n0 + (fr & 7), N - 1) * (uint32_t)K + (fr >> 3) * 64 + fq * 16;
+    const uint32_t ring_hi = (uint32_t)min(n0 + (fr & 7) + 8, N - 1) * (uint32_t)K + (fr >> 3) * 64 + fq * 16;
+    const uint8_t* ring_base = b + (size_t)kb0 * 128;
+#define DSV3_FETCH(P_, BASE_) { DSV3_GLOAD(wlo[P_][0], ring_lo, BASE_, P_ * 128); DSV3_GLOAD(whi[P_][0], ring_hi, BASE_, P_ * 128); }
+    if constexpr (RING) {
+        DSV3_FETCH(0, ring_base) DSV3_FETCH(1, ring_base) DSV3_FETCH(2, ring_base) DSV3_FETCH(3, ring_base)
+        DSV3_FETCH(4, ring_base) DSV3_FETCH(5, ring_base) DSV3_FETCH(6, ring_base) DSV3_FETCH(7, ring_base)
+    } else {
 #pragma unroll
-    for (int p = 0; p < NPF; ++p)
-        if (p < nkb) fetch(p, p);
+        for (int p = 0; p < NPF; ++p)
+            if (p < nkb) fetch(p, p);
+    }
     if (QF) {
         // the 8 lanes that hold the chunks of one (row, K block) are consecutive and aligned: amax by DPP
 #pragma unroll
@@ -224,42 +251,57 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
     // a lane's fragment: slab row (K block)*M + 16j + fr, logical chunks fq and 4 + fq of the K block
     const int row0 = (kb0 - wg_kb0) * M + fr;
 
-    // The wavefront works through its K blocks in batches of NPF: all weight loads of a batch are issued back to
-    // back, then consumed in order.  Memory-level parallelism across batches comes from the other wavefronts of
-    // the CU (up to 16), which are at different points of their own batches.
-    for (int kb = 0; kb < nkb; kb += NPF) {
-        if (kb > 0) {
+    // one K block k of the wavefront's range: ring slot p holds its weights
+    auto consume = [&](int p, int k) {
+        v8i af[MT], wf[S];
+        float sc[MT];
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            const int R = row0 + k * M + j * 16, fx = swz(R);
+            const uint8_t* r = act + R * 128;
+            af[j] = join(*(const v4i*)(r + ((fq ^ fx) * 16)), *(const v4i*)(r + (((4 + fq) ^ fx) * 16)));
+            sc[j] = act_s[R];
+        }
+#pragma unroll
+        for (int s = 0; s < S; ++s) wf[s] = untangle(wlo[p][s], whi[p][s]);
+#pragma unroll
+        for (int s = 0; s < S; ++s)
+#pragma unroll
+            for (int j = 0; j < MT; ++j) {
+                const v4f z = {0.f, 0.f, 0.f, 0.f};
+                const v4f p4 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[s], af[j], z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[s][j][e] = __builtin_fmaf(p4[e], sc[j], acc[s][j][e]);
+            }
+    };
+    if constexpr (RING) {
+        const int rounds = nkb / NPF;
+        int k = 0;
+        for (int r = 0; r + 1 < rounds; ++r) {              // steady state: every slot is refilled after use
+            const uint8_t* nbase = ring_base + (size_t)(r + 1) * NPF * 128;       // the K blocks one ring ahead
+#define DSV3_STEADY(P_) { WaitFor<2 * (NPF - 1)>::on(wlo[P_][0], whi[P_][0]); consume(P_, k); ++k; DSV3_FETCH(P_, nbase) }
+            DSV3_STEADY(0) DSV3_STEADY(1) DSV3_STEADY(2) DSV3_STEADY(3) DSV3_STEADY(4) DSV3_STEADY(5) DSV3_STEADY(6) DSV3_STEADY(7)
+#undef DSV3_STEADY
+        }
+#define DSV3_DRAIN(P_) { WaitFor<2 * (NPF - 1 - P_)>::on(wlo[P_][0], whi[P_][0]); consume(P_, k); ++k; }
+        DSV3_DRAIN(0) DSV3_DRAIN(1) DSV3_DRAIN(2) DSV3_DRAIN(3) DSV3_DRAIN(4) DSV3_DRAIN(5) DSV3_DRAIN(6) DSV3_DRAIN(7)
+#undef DSV3_DRAIN
+    } else {
+        // The wavefront works through its K blocks in batches of NPF: all weight loads of a batch are issued back
+        // to back, then consumed in order.  Memory-level parallelism across batches comes from the other wavefronts
+        // of the CU (up to 16), which are at different points of their own batches.
+        for (int kb = 0; kb < nkb; kb += NPF) {
+            if (kb > 0) {
+#pragma unroll
+                for (int p = 0; p < NPF; ++p)
+                    if (kb + p < nkb) fetch(p, kb + p);
+            }
 #pragma unroll
             for (int p = 0; p < NPF; ++p)
-                if (kb + p < nkb) fetch(p, kb + p);
-        }
-#pragma unroll
-        for (int p = 0; p < NPF; ++p) {
-            const int k = kb + p;
-            if (k < nkb) {                                    // wavefront-uniform
-                v8i af[MT], wf[S];
-                float sc[MT];
-#pragma unroll
-                for (int j = 0; j < MT; ++j) {
-                    const int R = row0 + k * M + j * 16, fx = swz(R);
-                    const uint8_t* r = act + R * 128;
-                    af[j] = join(*(const v4i*)(r + ((fq ^ fx) * 16)), *(const v4i*)(r + (((4 + fq) ^ fx) * 16)));
-                    sc[j] = act_s[R];
-                }
-#pragma unroll
-                for (int s = 0; s < S; ++s) wf[s] = untangle(wlo[p][s], whi[p][s]);
-#pragma unroll
-                for (int s = 0; s < S; ++s)
-#pragma unroll
-                    for (int j = 0; j < MT; ++j) {
-                        const v4f z = {0.f, 0.f, 0.f, 0.f};
-                        const v4f p4 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[s], af[j], z, 0, 0, 0, 0, 0, 0);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[s][j][e] = __builtin_fmaf(p4[e], sc[j], acc[s][j][e]);
-                    }
-            }
+                if (kb + p < nkb) consume(p, kb + p);             // wavefront-uniform
         }
     }
+#undef DSV3_FETCH
     __syncthreads();                                        // everyone is done with the activation slab
 
     // ---- add the wavefronts' partial sums in LDS (fixed order), then store
@@ -358,9 +400,20 @@ void launch_cfg(const Plan& p, const void* a, const float* a_s, const void* b, c
     const size_t red_bytes = (size_t)p.waves * S * MT * 64 * sizeof(v4f);
     const size_t slab_bytes = ((size_t)p.kb_per_wg * m + 16) * 128 + (size_t)p.kb_per_wg * m * 4;
     const size_t lds = red_bytes > slab_bytes ? red_bytes : slab_bytes;
+    const uint64_t m_magic = (uint64_t)(((1ull << 32) + (uint64_t)m - 1) / (uint64_t)m);
+    if constexpr (S == 1) {
+        // every wavefront's K range: the same whole number (>= 2) of ring rounds
+        const int kb = k / 128, per_wave = p.kb_per_wg / p.waves;
+        static const bool no_ring = getenv("DSV3_SKINNY_NORING") != nullptr;
+        if (!no_ring && kb % p.kb_per_wg == 0 && p.kb_per_wg % p.waves == 0 && per_wave % NPF == 0 && per_wave >= 2 * NPF &&
+            (int64_t)n * k < (1ll << 32)) {
+            hipLaunchKernelGGL((fp8_gemm_skinny_kernel<MT, S, NPF, QF, true>), dim3(groups, (unsigned)p.splits), dim3(p.waves * kWave), lds, st,
+                               (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, out_dtype, m, n, k, p.kb_per_wg, ue8m0, m_magic);
+            return;
+        }
+    }
     hipLaunchKernelGGL((fp8_gemm_skinny_kernel<MT, S, NPF, QF>), dim3(groups, (unsigned)p.splits), dim3(p.waves * kWave), lds, st,
-                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, out_dtype, m, n, k, p.kb_per_wg, ue8m0,
-                       (uint64_t)(((1ull << 32) + (uint64_t)m - 1) / (uint64_t)m));
+                       (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, out, out_dtype, m, n, k, p.kb_per_wg, ue8m0, m_magic);
 }
 
 }  // namespace skinny
