@@ -288,7 +288,10 @@ Plan make_plan(int64_t m, int64_t n, int64_t k) {
 // rows 25.5 against 30.4 us; 7168 -> 36864 at 8 rows 51 against 70 us).  One and two rows stay with the M <= 16
 // kernel, which quantises bf16 activations itself for linear() there (26.5 us fused against 25.5 + 3.5 us).
 bool single_group_stream(int64_t m, int64_t n, int64_t k) {
-    return m >= 3 && m <= 16 && n * k >= (96ll << 20) && skinny_single_supported(m, n, k);
+    if (m < 3 || m > 16 || n * k < (96ll << 20) || !skinny_single_supported(m, n, k)) return false;
+    // from 8 rows up the activation-streaming kernel is flat where this one grows with the rows (16384 -> 7168 at
+    // 8 / 12 / 16 rows: 26.2 / 26.3 / 26.5 against 26.7 / 28.3 / 29.6 us; at 3 / 4 rows 26.3 against 25.3 / 25.6)
+    return !(m >= 8 && n < 8192 && stream_supported(m, n, k));
 }
 
 // DSV3_GEMM_FORCE=tile|prefill pins the large-M kernel choice (tuning / debugging aid).
