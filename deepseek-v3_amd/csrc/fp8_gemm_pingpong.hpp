@@ -17,11 +17,11 @@
 //
 // LDS: two stages of [256 rows of A | 256 rows of B] x 128 bytes (the chunk permutation of fp8_gemm_prefill.hip)
 // and two slots of scales; block kb lives in stage kb % 2.  Which wavefront copies what, and when, is laid out at
-// the copy plan below: per block a wavefront requests two copies of block kb + 1 in M1 and six of block kb + 2 plus
-// the scales in M2, every region is refilled only after its last reader's phase has ended, and every copy has at
-// least one whole K block of time to land.  Copies retire in program order, so "the copies the next readers need have
-// landed" is a vmcnt(n) with n = the number of younger copies: 9, at the end of both M phases for group 1 and of
-// both C phases for group 0.
+// the copy plan below: per block a wavefront requests four copies of block kb + 1 in M1 and four of block kb + 2 plus
+// the scales in M2 (the same number in each of a block's four M phases), every region is refilled only after its
+// last reader's phase has ended, and every copy has at least one whole K block of time to land.  Copies retire in
+// program order, so "the copies the next readers need have landed" is a vmcnt(n) with n = the number of younger
+// copies: 9 at the end of both M phases for group 1, 5 at the end of C2 for group 0.
 //
 // Grouped mode (G): the tile is a slot of the grouped GEMM's tile table (a row range of one group, multiplied by that
 // group's weights, activation rows gathered through a row map) -- used for slots of more than 192 rows.
@@ -55,6 +55,13 @@ __device__ unsigned long long pp_clk[4];
 #define PP_PROF_FLUSH
 #define PP_CLK(i)
 #endif
+#ifdef DSV3_PP_TRACE
+__device__ unsigned long long pp_trace[8192 * 4];
+#define PP_TRACE(i) if (threadIdx.x == 0) { unsigned long long r_; \
+    asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r_) :: "memory"); pp_trace[(wg & 8191) * 4 + (i)] = r_; }
+#else
+#define PP_TRACE(i)
+#endif
 
 // One global -> LDS copy of 16 (or 4) bytes per lane: uniform 64-bit base in scalar registers, 32-bit lane offset,
 // uniform LDS address through M0 (lane l lands at lds_addr + 16 l).  Written out because the compiler otherwise
@@ -77,8 +84,10 @@ template <int SM> struct Geo {
     static constexpr int WM = 16 * SM, TM = 4 * WM;
     static constexpr int A_STAGE = TM * 128, B_STAGE = 256 * 128;       // bytes of A / of B per K block
     static constexpr int LDS_A = 0, LDS_B = 2 * A_STAGE, LDS_SC = 2 * A_STAGE + 2 * B_STAGE;
-    static constexpr int NM2 = SM == 4 ? 6 : 4;                         // copies per wavefront in M2 (plus the scales)
-    static constexpr int WAIT = NM2 + 1 + 2;                            // copies younger than the ones a phase end waits for
+    // copies per wavefront and K block: NM1_G0 / NM1_G1 in M1 (group 0 / 1), NM2 in M2 (plus the scales)
+    static constexpr int NM1_G0 = SM == 4 ? 4 : 2, NM1_G1 = 4, NM2 = SM == 4 ? 4 : 3;
+    // copies younger than the ones a phase end has to wait for: group 1 after both of its M phases, group 0 after C2
+    static constexpr int WAIT_G1 = NM1_G1 + NM2 + 1, WAIT_G0 = NM2 + 1;
 };
 constexpr int SC_SLOT = 2048, SC_SLOTS = 2;
 template <int SM> constexpr int lds_bytes() { return Geo<SM>::LDS_SC + SC_SLOTS * SC_SLOT; }
@@ -92,6 +101,7 @@ __device__ __forceinline__ void tile(
         int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, int wg,
         const GroupTable& g = GroupTable{}) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    PP_TRACE(0)
     using GEO = Geo<SM>;
     constexpr int TM = GEO::TM, WM = GEO::WM, A_STAGE = GEO::A_STAGE, B_STAGE = GEO::B_STAGE;
     constexpr int LDS_A = GEO::LDS_A, LDS_B = GEO::LDS_B, LDS_SC = GEO::LDS_SC, NM2 = GEO::NM2;
@@ -146,44 +156,62 @@ __device__ __forceinline__ void tile(
     // ---- copy plan.  A K block is TM / 8 + 32 wavefront-copies of 8 rows (1 KiB); copy q covers rows 8q .. 8q + 7.
     // The copies are requested in the M phases, interleaved with the LDS reads (the copy path takes one 1 KiB copy
     // per ~16 cycles and compute unit and holds the issuing wavefront meanwhile; a wavefront in a C phase that
-    // issued them would leave gaps in its MFMA stream).  Per block kb a wavefront issues
-    //   in M1  two copies of block kb + 1:  B rows 64-127 (group 0) / 192-255 (group 1), the last-columns part
-    //   in M2  NM2 copies of block kb + 2:  256-row tile  group 0  B rows 0-63 and 128-191 (4) and A rows 0-63 (2)
-    //                                                     group 1  A rows 64-255 (6)
-    //                                       128-row tile  group 0  B rows 0-63 and 128-191 (4)
-    //                                                     group 1  A rows 0-127 (4)
-    uint32_t m1_src[2], m2_src[NM2];
-    int m1_dst[2], m2_dst[NM2];
-    const uint8_t* m2_base[NM2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const int q = (grp == 0 ? 8 : 24) + wm * 2 + t;
+    // issued them would leave gaps in its MFMA stream), and spread evenly over the four M phases of a K block (two
+    // per group): with most of them in the M2 phases the second of the two found the memory pipeline still full of
+    // the first one's requests and took 140 cycles longer than the C phase beside it.
+    // What may be requested when: the part of a stage that M1 reads (all of A, B rows 0-63 and 128-191, the scales)
+    // is free once group 1 has left M1 of block kb and is read again by group 0 in M1 of block kb + 2 -- it is
+    // refilled in M2 of block kb by both groups and in M1 of block kb + 1 by group 0; the part that M2 reads (B
+    // rows 64-127 and 192-255) is free once group 1 has left M2 of block kb, and group 1 refills it in M1 of
+    // block kb + 1.  Per block kb a wavefront therefore issues
+    //   in M1  copies of block kb + 1:  group 1  B rows 64-127 and 192-255 (4 per wavefront)
+    //                                   group 0  the last 4 NM1_G0 entries of the list below
+    //   in M2  copies of block kb + 2:  group 0  entries 0 .. 4 NM2 - 1, group 1  entries 4 NM2 .. 8 NM2 - 1 of the list
+    //          [B rows 0-63, B rows 128-191, A rows 0 .. TM - 1] in groups of 8 rows, and the scales
+    // (256-row tile: 4 + 4 per wavefront and block, group 0 copies B's first halves and A rows 128-255, group 1 A rows
+    // 0-127; 128-row tile: 2 + 3 and 4 + 3).
+    constexpr int NM1_G0 = GEO::NM1_G0, NM1_G1 = GEO::NM1_G1, NM1 = NM1_G0 > NM1_G1 ? NM1_G0 : NM1_G1;
+    static_assert(8 * NM2 + 4 * NM1_G0 == 16 + TM / 8 && 4 * NM1_G1 == 16, "every 8-row group of a K block is copied once");
+    // per copy: the lane's source offset, the LDS address in stage 0 and in stage 1 (the two regions' stages differ in
+    // size in the 128-row tile), and whether it comes from b
+    uint32_t m1_src[NM1], m2_src[NM2];
+    uint32_t m1_dst[2][NM1], m2_dst[2][NM2];
+    bool m1_from_b[NM1], m2_from_b[NM2];
+    const uint32_t lds0 = lds_addr_of(lds);
+    auto plan = [&](bool from_b, int q, uint32_t& src, uint32_t& dst0, uint32_t& dst1) {
         const int r = q * 8 + (lane >> 3), ch = (lane & 7) ^ swz(r);
-        m1_src[t] = (uint32_t)min(n0_ld + r, N - 1) * (uint32_t)K + ch * 16;
-        m1_dst[t] = LDS_B + q * 1024;
+        src = (from_b ? (uint32_t)min(n0_ld + r, N - 1) : a_row(r)) * (uint32_t)K + ch * 16;
+        dst0 = lds0 + (from_b ? LDS_B : LDS_A) + q * 1024;
+        dst1 = dst0 + (from_b ? B_STAGE : A_STAGE);
+    };
+    // entry idx of the list [B rows 0-63, B rows 128-191, A rows 0 .. TM - 1]
+    auto plan_listed = [&](int idx, uint32_t& src, uint32_t& dst0, uint32_t& dst1, bool& from_b) {
+        from_b = idx < 16;
+        plan(from_b, from_b ? (idx < 8 ? idx : idx + 8) : idx - 16, src, dst0, dst1);
+    };
+#pragma unroll
+    for (int t = 0; t < NM1; ++t) {
+        const int listed = 8 * NM2 + wm * NM1_G0 + min(t, NM1_G0 - 1);
+        const bool fb = grp == 1 || listed < 16;
+        const int q = grp == 1 ? (t < 2 ? 8 : 24) + wm * 2 + (t & 1) : (listed < 16 ? (listed < 8 ? listed : listed + 8) : listed - 16);
+        m1_from_b[t] = fb;
+        plan(fb, q, m1_src[t], m1_dst[0][t], m1_dst[1][t]);
     }
 #pragma unroll
-    for (int t = 0; t < NM2; ++t) {
-        const bool from_b = grp == 0 && t < 4;
-        int q;
-        if (grp == 0) { const int idx = wm * 4 + t; q = t < 4 ? (idx < 8 ? idx : idx + 8) : wm * 2 + (t - 4); }
-        else q = SM == 4 ? 8 + wm * 6 + t : wm * 4 + t;
-        const int r = q * 8 + (lane >> 3), ch = (lane & 7) ^ swz(r);
-        m2_src[t] = (from_b ? (uint32_t)min(n0_ld + r, N - 1) : a_row(r)) * (uint32_t)K + ch * 16;
-        m2_dst[t] = (from_b ? LDS_B : LDS_A) + q * 1024;
-        m2_base[t] = from_b ? b : a;
-    }
-    // (a stage of the weight region and one of the activation region have different sizes in the 128-row tile)
+    for (int t = 0; t < NM2; ++t) plan_listed((grp * 4 + wm) * NM2 + t, m2_src[t], m2_dst[0][t], m2_dst[1][t], m2_from_b[t]);
     auto issue_m1 = [&](int t, int kb, int stage) {
-        copy16(b + (uint32_t)kb * 128u, m1_src[t], lds_addr_of(lds + m1_dst[t] + stage * B_STAGE));
+        copy16((m1_from_b[t] ? b : a) + (uint32_t)kb * 128u, m1_src[t], m1_dst[stage][t]);
     };
     auto issue_m2 = [&](int t, int kb, int stage) {
-        const bool from_b = grp == 0 && t < 4;
-        copy16(m2_base[t] + (uint32_t)kb * 128u, m2_src[t], lds_addr_of(lds + m2_dst[t] + stage * (from_b ? B_STAGE : A_STAGE)));
+        copy16((m2_from_b[t] ? b : a) + (uint32_t)kb * 128u, m2_src[t], m2_dst[stage][t]);
     };
     // scales of a K block: wavefronts 0-3 copy a_s[row, kb] of 64 tile rows each, wavefront 4 the b_s rows of the two
     // column halves (lanes 0 and 1; its other lanes and wavefronts 5-7 repeat an address already requested, so that
-    // every wavefront issues the same number of copies per block without asking the memory pipeline for more lines)
+    // every wavefront issues the same number of copies per block without asking the memory pipeline for more lines).
+    // a_s[row, kb] sits 4 KBT bytes from a_s[row + 1, kb]: the 64 scales of a copy are 64 memory lines, a third of all
+    // the lines a workgroup asks for, and they slow the phase after the one that requests them by 80-100 cycles (with
+    // one line per copy, results aside, a K block takes 2 % less).  Copying them for four K blocks at a time (16 bytes
+    // per row, a one-line copy in the other three blocks to keep the counts) was built and was not faster.
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
     const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT
@@ -216,12 +244,13 @@ __device__ __forceinline__ void tile(
         for (int t = 0; t < NM2; ++t) issue_m2(t, 0, 0);
         issue_scales(0, 0);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) issue_m1(t, 0, 0);
+        for (int t = 0; t < (GRP == 0 ? NM1_G0 : NM1_G1); ++t) issue_m1(t, 0, 0);
 #pragma unroll
         for (int t = 0; t < NM2; ++t) issue_m2(t, min(1, KB - 1), 1);
         issue_scales(min(1, KB - 1), 1);
         __builtin_amdgcn_s_waitcnt(0x0f70);                         // vmcnt(0)
         wg_barrier();
+        PP_TRACE(1)
         if (GRP == 1) wg_barrier();                                 // one phase behind group 0 from here on
 
         v8i af[SM], bf[4];
@@ -284,14 +313,22 @@ __device__ __forceinline__ void tile(
             if (RD || kb == 0) {
                 const uint8_t* as_base = a_rd + ST * A_STAGE;
                 const uint8_t* bs_base = b_rd + ST * B_STAGE;
+                // copy t goes in front of fragment read t (SM + 4) / n of the phase's SM + 4
+                constexpr int N1 = GRP == 0 ? NM1_G0 : NM1_G1;
 #pragma unroll
                 for (int j = 0; j < SM; ++j) {
-                    if (LD && j % (SM / 2) == 0) issue_m1(j / (SM / 2), kb1, ST ^ 1);
+#pragma unroll
+                    for (int t = 0; t < N1; ++t)
+                        if (LD && t * (SM + 4) / N1 == j) issue_m1(t, kb1, ST ^ 1);
                     af[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
                 }
 #pragma unroll
-                for (int ii = 0; ii < 4; ++ii)
+                for (int ii = 0; ii < 4; ++ii) {
+#pragma unroll
+                    for (int t = 0; t < N1; ++t)
+                        if (LD && t * (SM + 4) / N1 == SM + ii) issue_m1(t, kb1, ST ^ 1);
                     bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
+                }
             }
             {
                 const float bs = *(const float*)(sb_rd + ST * SC_SLOT);
@@ -305,38 +342,33 @@ __device__ __forceinline__ void tile(
             }
             __builtin_amdgcn_sched_barrier(0);
             PP_PROF_MARK(0)
-            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT);
+            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G1);
             wg_barrier();
             PP_PROF_MARK(1)
             // ---- C1 (its first two FMA groups belong to C2 of the previous block: zeros at kb = 0)
             compute(std::integral_constant<int, 0>{}, std::integral_constant<int, 7>{}, sc[ST], sc[ST ^ 1]);
             PP_PROF_MARK(2)
-            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT);
-            wg_barrier();
+            wg_barrier();                                           // (nothing group 0 has requested is read in the next phase)
             PP_PROF_MARK(3)
             // ---- M2
             {
                 const uint8_t* bs_base = b_rd + ST * B_STAGE + 4 * 2048;
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
-                    if (LD) issue_m2(ii, kb2, ST);
+                    if (LD && ii < NM2) issue_m2(ii, kb2, ST);
                     if (RD) bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
                 }
-                if (LD) {
-#pragma unroll
-                    for (int t = 4; t < NM2; ++t) issue_m2(t, kb2, ST);
-                    issue_scales(kb2, ST);
-                }
+                if (LD) issue_scales(kb2, ST);
             }
             __builtin_amdgcn_sched_barrier(0);
             PP_PROF_MARK(4)
-            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT);
+            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G1);
             wg_barrier();
             PP_PROF_MARK(5)
             // ---- C2
             compute(std::integral_constant<int, 4>{}, std::integral_constant<int, 3>{}, sc[ST], sc[ST]);
             PP_PROF_MARK(6)
-            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT);
+            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G0);
             wg_barrier();
             PP_PROF_MARK(7)
         };
@@ -364,6 +396,7 @@ __device__ __forceinline__ void tile(
     if (grp == 0) run(std::integral_constant<int, 0>{});
     else          run(std::integral_constant<int, 1>{});
     PP_CLK(2)
+    PP_TRACE(2)
 #undef DSV3_SGB
 
     // ---- epilogue: lane holds c[m][n .. n + 3] for every (i, j); see fp8_gemm_prefill.hip for the LDS route
@@ -395,6 +428,10 @@ __device__ __forceinline__ void tile(
             if (r < rows_here && n < N)
                 *(v4u*)(c + (size_t)(m0 + r) * N + n) = v;
         }
+#ifdef DSV3_PP_TRACE
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        PP_TRACE(3)
+#endif
         return;
     }
     if (f32_lds_epilogue) {
