@@ -33,8 +33,12 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     v2bf r = { (__bf16)lo, (__bf16)hi };
     return __builtin_bit_cast(uint32_t, r);
 }
-// Two binary32 -> packed fp16, round-to-nearest-even.
+// Two binary32 -> packed fp16, round-to-nearest-even.  The operands are made opaque first: where an FMA produces
+// one of them the compiler otherwise merges the two into v_fma_mix*_f16, which rounds the exact sum straight to
+// fp16 -- one rounding where every other path (and the binary32 result of the same product) has two, visible on
+// results that binary32 rounds onto an fp16 tie.
 __device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+    asm("" : "+v"(lo), "+v"(hi));
     __half2 r = __floats2half2_rn(lo, hi);
     return __builtin_bit_cast(uint32_t, r);
 }

@@ -58,7 +58,7 @@ __device__ unsigned long long pp_clk[4];
 #ifdef DSV3_PP_TRACE
 __device__ unsigned long long pp_trace[8192 * 4];
 #define PP_TRACE(i) if (threadIdx.x == 0) { unsigned long long r_; \
-    asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r_) :: "memory"); pp_trace[(wg & 8191) * 4 + (i)] = r_; }
+    asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r_) :: "memory"); pp_trace[(cur_w & 8191) * 4 + (i)] = r_; }
 #else
 #define PP_TRACE(i)
 #endif
@@ -93,23 +93,47 @@ constexpr int SC_SLOT = 2048, SC_SLOTS = 2;
 template <int SM> constexpr int lds_bytes() { return Geo<SM>::LDS_SC + SC_SLOTS * SC_SLOT; }
 constexpr int LDS_BYTES = lds_bytes<4>();               // 136 KiB (100 KiB for the 128-row tile)
 
-template <int CD, bool P2, bool G = false, int SM = 4>
+// PS (persistent): the workgroup computes tiles wg, wg + wg_stride, ... one after the other and treats their K blocks
+// as one stream -- the last two blocks of a tile request the first copies of the next tile where a single tile
+// repeats its last block, so the next tile starts without a prologue, and the finished tile's results leave through a
+// staging area of their own (2 KiB per wavefront behind the scales) while those copies are in flight.  Between two
+// tiles of a 7168-deep product this hides ~3 us of first-copy latency, ~0.7 us of workgroup dispatch and most of the
+// ~2.5 us a workgroup spends writing its results with nothing else resident on its compute unit.  For whole tiles
+// only (M a multiple of 256, the column tiles inside N), an even number (>= 4) of K blocks, one K slice and 16-bit
+// results; the caller sends everything else down the one-tile path.
+constexpr int PS_STAGING = 8 * 2048;
+
+template <int CD, bool P2, bool G = false, int SM = 4, bool PS = false>
 __device__ __forceinline__ void tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
         typename OutT<CD>::type* __restrict__ c,
         int M, int N, int K, int tiles_m, int tiles_n, int tn_first, int kb_per_split, int ldc, int wg,
-        const GroupTable& g = GroupTable{}) {
+        const GroupTable& g = GroupTable{}, int wg_stride = 0) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-    PP_TRACE(0)
     using GEO = Geo<SM>;
     constexpr int TM = GEO::TM, WM = GEO::WM, A_STAGE = GEO::A_STAGE, B_STAGE = GEO::B_STAGE;
     constexpr int LDS_A = GEO::LDS_A, LDS_B = GEO::LDS_B, LDS_SC = GEO::LDS_SC, NM2 = GEO::NM2;
     static_assert(!G || SM == 4, "grouped slots run the 256-row tile");
+    static_assert(!PS || (!G && SM == 4 && CD != DSV3_F32), "persistent mode: dense 256-row tiles with 16-bit results");
 
     // ---- workgroup -> tile: a contiguous run of tiles per XCD, walked in bands of GROUP_M tile rows; in grouped
     // mode the row tiles are dealt round-robin over the XCDs and the column tiles of a row tile stay on one XCD
     // (the mapping of the grouped kernel, whose dispatch has already checked that the slot is in use)
+    const int T = tiles_m * tiles_n;
+    auto dense_origin = [&](int w, int& m0_, int& n0_) {
+        int pid = w;
+        {
+            const int q = T / 8, r = T % 8, x = pid % 8;
+            pid = x * q + (x < r ? x : r) + pid / 8;
+        }
+        constexpr int GROUP_M = 4;
+        const int band = pid / (GROUP_M * tiles_n);
+        const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+        const int in_band = pid - band * GROUP_M * tiles_n;
+        m0_ = (band * GROUP_M + in_band % band_rows) * TM;
+        n0_ = (tn_first + in_band / band_rows) * BN;
+    };
     int m0, n0, rows_here;
     if (G) {
         const int x = wg % 8, idx = wg / 8;
@@ -121,27 +145,16 @@ __device__ __forceinline__ void tile(
         b += (size_t)expert * g.b_stride;
         b_s += (size_t)expert * g.bs_stride;
     } else {
-        const int T = tiles_m * tiles_n;
-        int pid = wg;
-        {
-            const int q = T / 8, r = T % 8, x = pid % 8;
-            pid = x * q + (x < r ? x : r) + pid / 8;
-        }
-        constexpr int GROUP_M = 4;
-        const int band = pid / (GROUP_M * tiles_n);
-        const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
-        const int in_band = pid - band * GROUP_M * tiles_n;
-        const int tm = band * GROUP_M + in_band % band_rows;
-        const int tn = in_band / band_rows;
-        m0 = tm * TM; n0 = (tn_first + tn) * BN;
+        dense_origin(wg, m0, n0);
         rows_here = min(TM, M - m0);
     }
-    // row of a behind row r of the tile; rows past the tile's end repeat its last row (their results are dropped)
+    // row of a behind row r of the tile; rows past the tile's end repeat its last row (their results are dropped).
+    // In persistent mode the tile's origin is part of the copies' scalar base address instead (cur / nxt below).
+    const int m0_ld = (PS || (DSV3_PP_ABL & 16)) ? 0 : m0, n0_ld = (PS || (DSV3_PP_ABL & 16)) ? 0 : n0;
     auto a_row = [&](int r) -> uint32_t {
-        const int rr = ((DSV3_PP_ABL & 16) ? 0 : m0) + min(r, rows_here - 1);
+        const int rr = m0_ld + min(r, rows_here - 1);
         return (uint32_t)((G && g.a_rows) ? g.a_rows[rr] : rr);
     };
-    const int n0_ld = (DSV3_PP_ABL & 16) ? 0 : n0;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -152,6 +165,18 @@ __device__ __forceinline__ void tile(
     c += (size_t)blockIdx.y * (size_t)M * (size_t)ldc;
     const int n_base = ldc == N ? 0 : tn_first * BN;
     a += (size_t)kb0 * 128u; b += (size_t)kb0 * 128u;
+    // persistent mode: the tile being computed and the one after it (the same once more behind the last one: its
+    // copies land in stages nobody reads any more)
+    struct Origin { const uint8_t* a; const uint8_t* b; const float* sc; };
+    auto origin_of = [&](int m0_, int n0_) {
+        return Origin{ a + (size_t)m0_ * (size_t)K, b + (size_t)n0_ * (size_t)K,
+                       wave < 4 ? a_s + (size_t)m0_ * (size_t)(K / 128) : b_s + (size_t)(n0_ / 128) * (size_t)(K / 128) };
+    };
+    int cur_w = wg, m0n = m0, n0n = n0;
+    bool has_next = PS && cur_w + wg_stride < T;
+    if (has_next) dense_origin(cur_w + wg_stride, m0n, n0n);
+    Origin cur = origin_of(m0, n0), nxt = origin_of(m0n, n0n);
+    PP_TRACE(0)
 
     // ---- copy plan.  A K block is TM / 8 + 32 wavefront-copies of 8 rows (1 KiB); copy q covers rows 8q .. 8q + 7.
     // The copies are requested in the M phases, interleaved with the LDS reads (the copy path takes one 1 KiB copy
@@ -199,11 +224,18 @@ __device__ __forceinline__ void tile(
     }
 #pragma unroll
     for (int t = 0; t < NM2; ++t) plan_listed((grp * 4 + wm) * NM2 + t, m2_src[t], m2_dst[0][t], m2_dst[1][t], m2_from_b[t]);
-    auto issue_m1 = [&](int t, int kb, int stage) {
-        copy16((m1_from_b[t] ? b : a) + (uint32_t)kb * 128u, m1_src[t], m1_dst[stage][t]);
+    // (persistent mode: block KB + i is block i of the next tile; only a tile's last two blocks -- `tail` -- get there)
+    auto issue_m1 = [&](int t, int kb, int stage, bool tail = true) {
+        if constexpr (PS) {
+            const bool nx = tail && kb >= KB;
+            copy16((m1_from_b[t] ? (nx ? nxt.b : cur.b) : (nx ? nxt.a : cur.a)) + (uint32_t)(nx ? kb - KB : kb) * 128u, m1_src[t], m1_dst[stage][t]);
+        } else copy16((m1_from_b[t] ? b : a) + (uint32_t)kb * 128u, m1_src[t], m1_dst[stage][t]);
     };
-    auto issue_m2 = [&](int t, int kb, int stage) {
-        copy16((m2_from_b[t] ? b : a) + (uint32_t)kb * 128u, m2_src[t], m2_dst[stage][t]);
+    auto issue_m2 = [&](int t, int kb, int stage, bool tail = true) {
+        if constexpr (PS) {
+            const bool nx = tail && kb >= KB;
+            copy16((m2_from_b[t] ? (nx ? nxt.b : cur.b) : (nx ? nxt.a : cur.a)) + (uint32_t)(nx ? kb - KB : kb) * 128u, m2_src[t], m2_dst[stage][t]);
+        } else copy16((m2_from_b[t] ? b : a) + (uint32_t)kb * 128u, m2_src[t], m2_dst[stage][t]);
     };
     // scales of a K block: wavefronts 0-3 copy a_s[row, kb] of 64 tile rows each, wavefront 4 the b_s rows of the two
     // column halves (lanes 0 and 1; its other lanes and wavefronts 5-7 repeat an address already requested, so that
@@ -215,9 +247,12 @@ __device__ __forceinline__ void tile(
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
     const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT
-                                      : (uint32_t)min(n0 / 128 + (wave == 4 ? min(lane, 1) : 0), nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
-    auto issue_scales = [&](int kb, int slot) {
-        copy4(sc_base + (uint32_t)kb, sc_off * 4u, lds_addr_of(lds + LDS_SC + slot * SC_SLOT + wave * 256));
+                                      : (uint32_t)min((PS ? 0 : n0 / 128) + (wave == 4 ? min(lane, 1) : 0), nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
+    auto issue_scales = [&](int kb, int slot, bool tail = true) {
+        if constexpr (PS) {
+            const bool nx = tail && kb >= KB;
+            copy4((nx ? nxt.sc : cur.sc) + (uint32_t)(nx ? kb - KB : kb), sc_off * 4u, lds_addr_of(lds + LDS_SC + slot * SC_SLOT + wave * 256));
+        } else copy4(sc_base + (uint32_t)kb, sc_off * 4u, lds_addr_of(lds + LDS_SC + slot * SC_SLOT + wave * 256));
     };
 
     // ---- fragment addresses: lane reads row (lane & 15) of a 16-row sub-tile, K bytes 32 (lane >> 4) .. + 31
@@ -234,6 +269,35 @@ __device__ __forceinline__ void tile(
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < SM; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // persistent mode: results of the current tile, one 16-row sub-tile and 64 columns at a time: four 16 x 16
+    // accumulator tiles go to the wavefront's staging area as 16 rows of 128 bytes (16-byte chunks permuted by the row so
+    // that neither the 8-byte writes nor the 16-byte reads collide) and leave as two stores of 8 rows x 128 bytes;
+    // the accumulators are cleared for the next tile on the way
+    auto ps_epilogue = [&]() {
+        uint8_t* stg = lds + LDS_SC + SC_SLOTS * SC_SLOT + wave * 2048;
+        const int rr = lane >> 3, ch = lane & 7;
+#pragma unroll
+        for (int j = 0; j < SM; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii) {
+                    v4f& v = acc[h * 4 + ii][j];
+                    v2u o;
+                    if (CD == DSV3_BF16) o = v2u{ pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]) };
+                    else o = v2u{ pack_f16(v[0], v[1]), pack_f16(v[2], v[3]) };
+                    *(v2u*)(stg + fr * 128 + (((ii * 2 + (fq >> 1)) ^ (fr & 7)) * 16) + (fq & 1) * 8) = o;
+                    v = (v4f){0.f, 0.f, 0.f, 0.f};
+                }
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    const int lr = p * 8 + rr;
+                    const v4u v = *(const v4u*)(stg + lr * 128 + ((ch ^ (lr & 7)) * 16));
+                    *(v4u*)(c + (size_t)(m0 + wm * WM + j * 16 + lr) * N + n0 + grp * 128 + h * 64 + ch * 8) = v;
+                }
+            }
+    };
 
 #define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
     auto run = [&](auto gtag) {
@@ -306,9 +370,15 @@ __device__ __forceinline__ void tile(
         PP_PROF_DECL
         // one K block whose LDS stage (and scale slot) ST is a compile-time constant: every LDS address of the loop is
         // a register plus an immediate
-        auto block = [&](int kb, auto st_tag) {
+        auto block = [&](int kb, auto st_tag, auto tail_tag) {
             constexpr int ST = decltype(st_tag)::value;
-            const int kb1 = min(kb + 1, KB - 1), kb2 = min(kb + 2, KB - 1);
+            constexpr bool TAIL = decltype(tail_tag)::value;     // persistent mode: one of the tile's last two blocks
+            // (the block numbers behind the copies' addresses are made opaque at the start of the phase that uses
+            // them: the scalar arithmetic that follows from them is otherwise moved up, in front of the barrier
+            // that ends the C phase before, where the matrix pipe waits for it)
+            int kb_m1 = kb;
+            asm volatile("" : "+s"(kb_m1));
+            const int kb1 = PS ? kb_m1 + 1 : min(kb_m1 + 1, KB - 1);
             // ---- M1
             if (RD || kb == 0) {
                 const uint8_t* as_base = a_rd + ST * A_STAGE;
@@ -319,14 +389,14 @@ __device__ __forceinline__ void tile(
                 for (int j = 0; j < SM; ++j) {
 #pragma unroll
                     for (int t = 0; t < N1; ++t)
-                        if (LD && t * (SM + 4) / N1 == j) issue_m1(t, kb1, ST ^ 1);
+                        if (LD && t * (SM + 4) / N1 == j) issue_m1(t, kb1, ST ^ 1, TAIL);
                     af[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
                 }
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
 #pragma unroll
                     for (int t = 0; t < N1; ++t)
-                        if (LD && t * (SM + 4) / N1 == SM + ii) issue_m1(t, kb1, ST ^ 1);
+                        if (LD && t * (SM + 4) / N1 == SM + ii) issue_m1(t, kb1, ST ^ 1, TAIL);
                     bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
                 }
             }
@@ -352,13 +422,16 @@ __device__ __forceinline__ void tile(
             PP_PROF_MARK(3)
             // ---- M2
             {
+                int kb_m2 = kb;
+                asm volatile("" : "+s"(kb_m2));
+                const int kb2 = PS ? kb_m2 + 2 : min(kb_m2 + 2, KB - 1);
                 const uint8_t* bs_base = b_rd + ST * B_STAGE + 4 * 2048;
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
-                    if (LD && ii < NM2) issue_m2(ii, kb2, ST);
+                    if (LD && ii < NM2) issue_m2(ii, kb2, ST, TAIL);
                     if (RD) bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
                 }
-                if (LD) issue_scales(kb2, ST);
+                if (LD) issue_scales(kb2, ST, TAIL);
             }
             __builtin_amdgcn_sched_barrier(0);
             PP_PROF_MARK(4)
@@ -373,22 +446,53 @@ __device__ __forceinline__ void tile(
             PP_PROF_MARK(7)
         };
 
-        int kb = 0;
-        for (; kb + 1 < KB; kb += 2) {
-            block(kb, std::integral_constant<int, 0>{});
-            block(kb + 1, std::integral_constant<int, 1>{});
-        }
-        if (kb < KB) block(kb, std::integral_constant<int, 0>{});
-        PP_PROF_FLUSH
-        // the FMAs of the last two MFMAs
-        if (!P2) {
-            const int last = (KB - 1) & 1;
+        for (;;) {                                                  // (one pass unless persistent)
+            constexpr std::integral_constant<int, 0> st0{};
+            constexpr std::integral_constant<int, 1> st1{};
+            int kb = 0;
+            if constexpr (PS) {                                     // (an even number of blocks, at least four)
+                for (; kb + 3 < KB; kb += 2) {
+                    block(kb, st0, std::false_type{});
+                    block(kb + 1, st1, std::false_type{});
+                }
+                block(kb, st0, std::true_type{});
+                block(kb + 1, st1, std::true_type{});
+            } else {
+                for (; kb + 1 < KB; kb += 2) {
+                    block(kb, st0, std::false_type{});
+                    block(kb + 1, st1, std::false_type{});
+                }
+                if (kb < KB) block(kb, st0, std::false_type{});
+            }
+            // the FMAs of the last two MFMAs
+            if (!P2) {
+                const int last = (KB - 1) & 1;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                acc[7][SM - 2][e] = __builtin_fmaf(p14[e], last ? sc[1][SM - 2] : sc[0][SM - 2], acc[7][SM - 2][e]);
-                acc[7][SM - 1][e] = __builtin_fmaf(p15[e], last ? sc[1][SM - 1] : sc[0][SM - 1], acc[7][SM - 1][e]);
+                for (int e = 0; e < 4; ++e) {
+                    acc[7][SM - 2][e] = __builtin_fmaf(p14[e], last ? sc[1][SM - 2] : sc[0][SM - 2], acc[7][SM - 2][e]);
+                    acc[7][SM - 1][e] = __builtin_fmaf(p15[e], last ? sc[1][SM - 1] : sc[0][SM - 1], acc[7][SM - 1][e]);
+                }
+            }
+            if constexpr (!PS) break;
+            else {
+                // the tile's results leave through this wavefront's own staging area (no barrier: the other group
+                // is one phase behind and meets this wavefront again at the next tile's first barrier); then the
+                // next tile, whose first two blocks have been requested by the blocks just finished
+                PP_TRACE(2)
+                ps_epilogue();
+                PP_TRACE(3)
+                if (!has_next) break;
+                cur_w += wg_stride;
+                m0 = m0n; n0 = n0n; cur = nxt;
+                has_next = cur_w + wg_stride < T;
+                if (has_next) { dense_origin(cur_w + wg_stride, m0n, n0n); nxt = origin_of(m0n, n0n); }
+                p14 = p15 = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < SM; ++j) sc[0][j] = sc[1][j] = 0.f;
+                PP_TRACE(0)
             }
         }
+        PP_PROF_FLUSH
         if (GRP == 0) wg_barrier();                                 // group 1's last phase
         __builtin_amdgcn_s_waitcnt(0x0f70);                         // the clamped refills of the last blocks
     };
@@ -396,8 +500,9 @@ __device__ __forceinline__ void tile(
     if (grp == 0) run(std::integral_constant<int, 0>{});
     else          run(std::integral_constant<int, 1>{});
     PP_CLK(2)
-    PP_TRACE(2)
 #undef DSV3_SGB
+    if constexpr (PS) return;
+    PP_TRACE(2)
 
     // ---- epilogue: lane holds c[m][n .. n + 3] for every (i, j); see fp8_gemm_prefill.hip for the LDS route
     constexpr int WN = 128, SN = 8;

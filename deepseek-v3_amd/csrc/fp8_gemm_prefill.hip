@@ -653,6 +653,22 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_two_heights_kernel(
     }
 }
 
+// Dense GEMM of whole 256-row tiles in which wg_tall (a multiple of 8) persistent workgroups walk the tall tiles
+// [0, tn_tall) x M / 256, wg_tall apart, with the copies of a tile's first K blocks requested by the last blocks of
+// the tile before it (pingpong::tile in persistent mode); the workgroups behind them compute the column tiles
+// [tn_tall, tn_tall + tn_short) as 128-row tiles, as in the kernel above.
+template <int CD, bool P2 = false>
+__global__ __launch_bounds__(THREADS, 1) void fp8_gemm_persistent_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c, int M, int N, int K, int tn_tall, int tn_short, int wg_tall) {
+    const GroupTable none{};
+    if ((int)blockIdx.x < wg_tall)
+        pingpong::tile<CD, P2, false, 4, true>(a, a_s, b, b_s, c, M, N, K, M / 256, tn_tall, 0, K / 128, N, blockIdx.x, none, wg_tall);
+    else
+        pingpong::tile<CD, P2, false, 2>(a, a_s, b, b_s, c, M, N, K, M / 128, tn_short, tn_tall, K / 128, N, blockIdx.x - wg_tall);
+}
+
 }  // namespace prefill
 
 // Usable when the row offsets fit 32 bits; the caller falls back to the generic tile kernel otherwise.
@@ -833,6 +849,36 @@ size_t prefill_workspace_bytes(int64_t m, int64_t n, int64_t k) {
     return (size_t)p.slabs * (size_t)m * (size_t)cols * sizeof(float);
 }
 
+// The persistent kernel takes a plan of 256-row tiles (and, behind them, 128-row tiles) when every tile is whole,
+// the K range is an even number of blocks between 4 and 32, the results are 16 bits wide and the tall tiles are more
+// than one round.  What it saves is ~3.5 us per tile after a workgroup's first; what it costs is that tiles are dealt
+// to the workgroups in advance instead of to whichever compute unit is free, and a per-block ~1 % from the longer
+// code.  M = 4096: 512 -> 32768 (8 tiles of 4 blocks per workgroup) 106 -> 91 us, 1536 -> 24576 148 -> 136 us,
+// 2048 -> 7168 59 -> 57.5 us, 4096 -> 7168 102.5 -> 101 us; at 56 blocks per tile (7168 -> 18432) the two are equal
+// and at 144 (18432 -> 7168, 448 tiles) the fixed deal loses 8 us of 408, hence the upper limit.
+// DSV3_PREFILL_NOPERSIST=1 switches it off (tuning aid).  Returns -1 when the plan is not for it.
+template <int CD, bool P2>
+int launch_persistent(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+                      int64_t m, int64_t n, int64_t k, int64_t tn_tall, int64_t tn_short, hipStream_t stream) {
+    using namespace prefill;
+    if constexpr (CD == DSV3_F32) return -1;
+    else {
+        static const bool off = getenv("DSV3_PREFILL_NOPERSIST") != nullptr;
+        const int64_t kb = k / 128, n_tall = m / 256 * tn_tall;
+        if (off || !use_pingpong_short() || m % 256 || n % 8 || (tn_tall + tn_short) * BN > n || kb < 4 || kb > 32 || kb % 2 || n_tall <= kCUs) return -1;
+        constexpr int LDS_BYTES = pingpong::LDS_BYTES + pingpong::PS_STAGING;
+        static_assert(LDS_BYTES <= 160 * 1024, "LDS of a compute unit");
+        auto kern = fp8_gemm_persistent_kernel<CD, P2>;
+        static LdsGrant grant;
+        if (!grant.ensure((const void*)kern, LDS_BYTES)) return DSV3_ERR_LAUNCH;
+        const int64_t grid = kCUs + m / 128 * tn_short;
+        if (grid > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
+                           (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)tn_tall, (int)tn_short, (int)kCUs);
+        return launch_status();
+    }
+}
+
 // ws must hold prefill_workspace_bytes(m, n, k) bytes
 template <int CD, bool P2>
 int launch_prefill(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
@@ -843,6 +889,8 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
     const prefill::GroupTable none{};
     if (p.tn_short > 0) {
         using namespace prefill;
+        const int rc_ps = launch_persistent<CD, P2>(a, a_s, b, b_s, c, m, n, k, p.tn_plain, p.tn_short, stream);
+        if (rc_ps >= 0) return rc_ps;
         constexpr int LDS_OLD = Cfg<256, 2>::LDS_BYTES > Cfg<128, 3>::LDS_BYTES ? Cfg<256, 2>::LDS_BYTES : Cfg<128, 3>::LDS_BYTES;
         constexpr int LDS_BYTES = LDS_OLD > pingpong::LDS_BYTES ? LDS_OLD : pingpong::LDS_BYTES;
         const int pp = use_pingpong() ? (use_pingpong_short() ? 2 : 1) : 0;
@@ -864,7 +912,8 @@ int launch_prefill(const void* a, const float* a_s, const void* b, const float* 
         return launch_kernel<OD, false, 256, 2, P2>(a, a_s, b, b_s, out, m, n, k, tm, tn_first, tn_count, none, stream, splits, ldc);
     };
     if (p.tn_plain > 0) {
-        const int rc = run(std::integral_constant<int, CD>{}, c, 0, p.tn_plain, 1, 0);
+        int rc = p.tile_rows == 256 ? launch_persistent<CD, P2>(a, a_s, b, b_s, c, m, n, k, p.tn_plain, 0, stream) : -1;
+        if (rc < 0) rc = run(std::integral_constant<int, CD>{}, c, 0, p.tn_plain, 1, 0);
         if (rc != DSV3_OK || p.slabs <= 1) return rc;
     }
     if (!ws) return DSV3_ERR_WORKSPACE;

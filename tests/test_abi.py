@@ -234,7 +234,7 @@ def test_linear_fp8_validation(L):
     assert not fused(4096, 1536, 7168)
     assert not fused(4, 1536, 7000) and not fused(0, 8, 128)
     #     x    dtype   b    b_s  c    cdtype  m  n     k     block fmt ws    ws_bytes stream
-    ok = [A16, L.BF16, A16, A16, A16, L.BF16, 4, 1536, 7168, 128,  0,  A16 * 16, 1 << 30, None]
+    ok = [A16, L.BF16, A16, A16, A16, L.BF16, 2, 1536, 7168, 128,  0,  A16 * 16, 1 << 30, None]
 
     def call(i=None, v=None):
         a = list(ok)

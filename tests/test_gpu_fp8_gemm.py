@@ -232,6 +232,38 @@ def test_prefill_w2_sampled(K):
     assert torch.equal(c16.view(torch.int16), c32.to(torch.bfloat16).view(torch.int16))
 
 
+@pytest.mark.parametrize("m,k,n", [
+    (4096, 512, 32768),     # 16 x 128 tiles of 4 K blocks: 8 tiles per workgroup, every block of a tile is one of its "last two"
+    (2048, 1536, 12288),    # 8 x 48 = 384 tiles of 12 blocks: half of the workgroups compute two tiles, the others one
+    (1280, 4096, 16384),    # 5 x 64 = 320 tiles of 32 blocks (the longest K range that takes this route)
+])
+def test_several_tiles_per_workgroup(K, m, k, n):
+    """Whole 256 x 256 tiles in more than one round with a short K range: the 16-bit product runs in workgroups that
+    compute their tiles one after the other (the last K blocks of a tile request the first copies of the next one), the
+    binary32 product of the same call one tile per workgroup; the oracle evaluates a sample, and the bf16 result
+    must be the rounding of the binary32 one bit for bit."""
+    from dsv3fp8 import workloads
+    x = workloads.activations(m, k, seed=m % 97, device="cuda")
+    w8, ws = workloads.weight(n, k, seed=n % 89, device="cuda")
+    a, a_s = K.act_quant(x)
+    c32, c16 = _gemm_both(K, a, a_s, w8, ws)
+    rows = torch.cat([torch.arange(5, m, 97), torch.tensor([0, 255, 256, m - 1])]).cuda()
+    nb = n // 128
+    ref, cols = _sampled_reference(a, a_s, w8, ws, rows, [0, 1, 2, nb // 2, nb - 2, nb - 1])
+    got = c32[rows][:, cols.cuda()].cpu()
+    rms = ref.pow(2).mean().sqrt().item()
+    assert (got - ref).abs().max().item() <= TOL * rms
+    assert torch.equal(c16.view(torch.int16), c32.to(torch.bfloat16).view(torch.int16))
+    # fp16 results take the same route
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float16)
+    try:
+        h16 = K.fp8_gemm(a, a_s, w8, ws)
+    finally:
+        torch.set_default_dtype(old)
+    assert torch.equal(h16.view(torch.int16), c32.to(torch.float16).view(torch.int16))
+
+
 def test_prefill_pow2_full_size_sampled(K):
     """fp8_gemm_pow2 at M=4096 on both prefill shapes: power-of-two activation scales (ue8m0) and weight block scales
     rounded up to powers of two; sampled against the oracle and held against the general kernel everywhere."""
@@ -345,6 +377,7 @@ def _pow2_problem(m, n, k, seed):
     (1030, 17000, 512),    # two tile heights in one launch, ragged N
     (130, 4096, 2048),     # K range cut into slices (binary32 slabs)
     (16, 1536, 7168),      # few rows: the same kernels as fp8_gemm
+    (2048, 12288, 512),    # 384 whole tall tiles of 4 K blocks: workgroups that compute two tiles in a row (16-bit results)
 ])
 def test_power_of_two_scales_in_the_matrix_instruction(K, m, n, k):
     a, a_s, w8, ws = _pow2_problem(m, n, k, seed=m)
