@@ -264,6 +264,39 @@ def test_several_tiles_per_workgroup(K, m, k, n):
     assert torch.equal(h16.view(torch.int16), c32.to(torch.float16).view(torch.int16))
 
 
+def test_every_kernel_family_replays_in_a_graph(K):
+    """act_quant + fp8_gemm over shapes that take every family of GEMM kernels (one- and two-row kernel with and
+    without K slices, activation-streaming kernel, one group of the grouped few-row kernel, K-sliced mid-M tiles,
+    two tile heights in one launch, several tiles per workgroup) captured in one HIP graph: three replays with
+    fresh activations and eager work between them, each compared with the eager result bit for bit."""
+    from dsv3fp8 import workloads
+    shapes = [(1, 7168, 1536), (2, 1536, 24576), (8, 7168, 2112), (32, 7168, 576), (64, 512, 32768),
+              (4, 16384, 7168), (130, 2048, 4096), (1030, 512, 17000), (2048, 512, 12288), (1280, 4096, 16384)]
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        weights = [workloads.weight(n, k, seed=i + 3, device="cuda") for i, (m, k, n) in enumerate(shapes)]
+        xs = [workloads.activations(m, k, seed=i, device="cuda") for i, (m, k, n) in enumerate(shapes)]
+
+        def run():
+            return [K.fp8_gemm(*K.act_quant(x), w8, ws) for x, (w8, ws) in zip(xs, weights)]
+        run()                                               # warm-up outside capture (attributes, workspaces)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = run()
+        for rep in range(3):
+            for i, x in enumerate(xs):
+                x.copy_(workloads.activations(x.size(0), x.size(1), seed=100 * rep + i, device="cuda"))
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = run()                                   # eager work between the replays
+            for i, (g, e) in enumerate(zip(outs, eager)):
+                assert torch.equal(g, e), (rep, shapes[i])
+    finally:
+        torch.set_default_dtype(old)
+
+
 def test_prefill_pow2_full_size_sampled(K):
     """fp8_gemm_pow2 at M=4096 on both prefill shapes: power-of-two activation scales (ue8m0) and weight block scales
     rounded up to powers of two; sampled against the oracle and held against the general kernel everywhere."""
