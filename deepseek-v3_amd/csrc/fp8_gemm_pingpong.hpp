@@ -4,16 +4,22 @@
 // Eight wavefronts, 4 along m x 2 along n, each owning 64 (m) x 128 (n) of the tile as 4 x 8 MFMA tiles of 16 x 16
 // (one v_mfma 16x16x128 = one 128-wide scale block of K, folded into binary32 accumulators by one FMA per element
 // with a_s[m, kb] * b_s[n / 128, kb]).  Wavefront w runs on SIMD w % 4, so the two wavefronts of a SIMD are the two
-// column halves ("groups") of one row quarter.  A K block is four phases per wavefront, separated by workgroup
-// barriers:
+// column halves ("groups") of one row quarter.  A K block is four phases per wavefront:
 //     M1  read the block's activation fragments (64 rows) and the weight fragments of its first 64 columns from LDS
 //         into registers, read the block's scales, request global -> LDS copies
 //     C1  16 MFMAs on those registers, each followed by the four FMAs of the MFMA issued two earlier
 //     M2  read the weight fragments of the other 64 columns, request copies
 //     C2  16 MFMAs
-// Group 1 takes one barrier more before its first block and therefore always runs one phase behind group 0: while
-// one wavefront of a SIMD issues nothing but MFMAs and their FMAs, the other does all of its LDS and global memory
-// work, and the matrix pipe sees an uninterrupted instruction stream from one wavefront at a time.
+// and two workgroup barriers: group 0 passes one after each C phase, group 1 after each M phase.  Between two
+// barriers group 0 therefore runs an M phase and then a C phase while group 1 runs a C phase (of the half block
+// before) and then an M phase: whenever a wavefront does its LDS and global memory work, the other wavefront of its
+// SIMD is in a C phase, and the matrix pipe always has a wavefront to take instructions from.  Group 1's C phases
+// run at raised priority (s_setprio): where the two C phases of a SIMD overlap, the arbiter otherwise serves group
+// 0's first, group 1's ends late, and its M phase is left with nothing beside it.  The two barriers are the ones
+// the data needs (every region of a stage is refilled only after all eight wavefronts have read it, and read only
+// after every wavefront has seen its copies land); a barrier after every phase, which also kept the two wavefronts of
+// a SIMD strictly apart, cost 11 % more cycles per block (and, the chip being power limited under this kernel,
+// 0.5 % more time).
 //
 // LDS: two stages of [256 rows of A | 256 rows of B] x 128 bytes (the chunk permutation of fp8_gemm_prefill.hip)
 // and two slots of scales; block kb lives in stage kb % 2.  Which wavefront copies what, and when, is laid out at
@@ -302,7 +308,7 @@ __device__ __forceinline__ void tile(
 #define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
     auto run = [&](auto gtag) {
         constexpr int GRP = decltype(gtag)::value;
-        constexpr bool LD = !(DSV3_PP_ABL & 2), RD = !(DSV3_PP_ABL & 4);
+        constexpr bool LD = !(DSV3_PP_ABL & 2), RD = !(DSV3_PP_ABL & 4), STRICT = (DSV3_PP_ABL & 256) != 0;
         // prologue: blocks 0 and 1 as far as the steady state expects them to have been requested
 #pragma unroll
         for (int t = 0; t < NM2; ++t) issue_m2(t, 0, 0);
@@ -315,7 +321,7 @@ __device__ __forceinline__ void tile(
         __builtin_amdgcn_s_waitcnt(0x0f70);                         // vmcnt(0)
         wg_barrier();
         PP_TRACE(1)
-        if (GRP == 1) wg_barrier();                                 // one phase behind group 0 from here on
+        if (STRICT && GRP == 1) wg_barrier();                       // one phase behind group 0 from here on
 
         v8i af[SM], bf[4];
         v4f p14 = {0.f, 0.f, 0.f, 0.f}, p15 = {0.f, 0.f, 0.f, 0.f}; // raw products of the last two MFMAs of a C phase
@@ -332,7 +338,7 @@ __device__ __forceinline__ void tile(
             constexpr int I0 = decltype(i0_tag)::value, IT = decltype(it_tag)::value;
             constexpr int NT = 4 * SM;
             __builtin_amdgcn_sched_barrier(0);
-            if (DSV3_PP_ABL & 1) __builtin_amdgcn_s_setprio(1);
+            if ((DSV3_PP_ABL & 1) || (!STRICT && GRP == 1)) __builtin_amdgcn_s_setprio(3);
             if constexpr (P2) {
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii)
@@ -363,7 +369,7 @@ __device__ __forceinline__ void tile(
                 }
                 p14 = p[NT - 2]; p15 = p[NT - 1];
             }
-            if (DSV3_PP_ABL & 1) __builtin_amdgcn_s_setprio(0);
+            if ((DSV3_PP_ABL & 1) || (!STRICT && GRP == 1)) __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
         };
 
@@ -413,12 +419,12 @@ __device__ __forceinline__ void tile(
             __builtin_amdgcn_sched_barrier(0);
             PP_PROF_MARK(0)
             if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G1);
-            wg_barrier();
+            if (STRICT || GRP == 1) wg_barrier();
             PP_PROF_MARK(1)
             // ---- C1 (its first two FMA groups belong to C2 of the previous block: zeros at kb = 0)
             compute(std::integral_constant<int, 0>{}, std::integral_constant<int, 7>{}, sc[ST], sc[ST ^ 1]);
             PP_PROF_MARK(2)
-            wg_barrier();                                           // (nothing group 0 has requested is read in the next phase)
+            if (STRICT || GRP == 0) wg_barrier();                   // (nothing group 0 has requested is read in the next phase)
             PP_PROF_MARK(3)
             // ---- M2
             {
@@ -436,13 +442,13 @@ __device__ __forceinline__ void tile(
             __builtin_amdgcn_sched_barrier(0);
             PP_PROF_MARK(4)
             if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G1);
-            wg_barrier();
+            if (STRICT || GRP == 1) wg_barrier();
             PP_PROF_MARK(5)
             // ---- C2
             compute(std::integral_constant<int, 4>{}, std::integral_constant<int, 3>{}, sc[ST], sc[ST]);
             PP_PROF_MARK(6)
             if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G0);
-            wg_barrier();
+            if (STRICT || GRP == 0) wg_barrier();
             PP_PROF_MARK(7)
         };
 
@@ -493,7 +499,7 @@ __device__ __forceinline__ void tile(
             }
         }
         PP_PROF_FLUSH
-        if (GRP == 0) wg_barrier();                                 // group 1's last phase
+        if (STRICT && GRP == 0) wg_barrier();                       // group 1's last phase
         __builtin_amdgcn_s_waitcnt(0x0f70);                         // the clamped refills of the last blocks
     };
     PP_CLK(0)
