@@ -118,6 +118,7 @@ class Probes:
                 "fp8_mfma_loop_TFLOPs": round(self.mfma_tflops(0), 1),
                 "fp8_mfma_loop_changing_operands_TFLOPs": round(self.mfma_tflops(1), 1),
                 "fp8_mfma_loop_with_fold_TFLOPs": round(self.mfma_tflops(2), 1),
+                "fp8_mfma_loop_with_fold_and_operand_traffic_TFLOPs": round(self.mfma_tflops(3), 1),
                 "empty_launch_us": round(nl, 2),
                 "note": "measured on this GPU in this run: 1 GiB read stream; 1 GiB copy (bytes read + written); streams "
                         "that read two bytes per byte written (the mix of act_quant and weight_quant) and one per two "
@@ -125,7 +126,11 @@ class Probes:
                         "CU: one operand pair for all instructions, 4 x 4 fragments of random bytes accumulated in the "
                         "matrix core (what power-of-two scales allow), and the same with every product folded into "
                         "its accumulator by four FMAs (what binary32 block scales need) -- the chip is power limited, "
-                        "so the rate falls as operands toggle and as vector work is added; empty kernel in a graph"}
+                        "so the rate falls as operands toggle and as vector work is added; that last loop inside the data movement "
+                        "of a 256 x 256 x 128 GEMM step and nothing else (per 16 products a wavefront copies 4 KiB from "
+                        "L2 into LDS and reads six 2 KiB fragments from LDS into the operand registers; no barrier, the "
+                        "copied bytes are not consumed): what the chip sustains for the GEMM's instruction mix and "
+                        "traffic when every overlap is perfect; empty kernel in a graph"}
 
 
 def _events(n):
@@ -532,7 +537,9 @@ def main():
                      "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4), "traffic": measured_traffic(),
                      "launch_us": round(gemm_ms * 1e3, 2), "flops_per_launch": flops,
                      "frac_of_measured_mfma_loop": round(achieved / ceil["fp8_mfma_loop_TFLOPs"], 4),
-                     "frac_of_measured_mfma_loop_with_fold": round(achieved / ceil["fp8_mfma_loop_with_fold_TFLOPs"], 4)},
+                     "frac_of_measured_mfma_loop_with_fold": round(achieved / ceil["fp8_mfma_loop_with_fold_TFLOPs"], 4),
+                     "frac_of_measured_mfma_loop_with_fold_and_operand_traffic":
+                         round(achieved / ceil["fp8_mfma_loop_with_fold_and_operand_traffic_TFLOPs"], 4)},
         "ceilings": ceil,
     }
     if not args.no_cpu:

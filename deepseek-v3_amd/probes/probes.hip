@@ -1,8 +1,10 @@
 // Measurement probes for the benchmark (libdsv3probe.so): kernels of known traffic / arithmetic that give the
-// ceilings this GPU sustains -- a read stream, a copy, read/write mixes, fp8 MFMA loops and an empty launch.  They are not part of
-// libdsv3fp8.so and nothing in the product path calls them.
+// ceilings this GPU sustains -- a read stream, a copy, read/write mixes, fp8 MFMA loops (registers only, and with a
+// GEMM step's operand traffic) and an empty launch.  They are not part of libdsv3fp8.so and nothing in the product
+// path calls them.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -113,6 +115,73 @@ __global__ __launch_bounds__(512, 1) void mfma_kernel(int iters, const int* __re
     if (r == 12345.678f) sink[blockIdx.x] = r;
 }
 
+// MODE 2's loop inside the operand traffic of a 256 x 256 x 128 GEMM step, with no synchronisation at all: per 16
+// products every wavefront copies 4 KiB of an L2-resident 2 MiB window into LDS with the direct-to-LDS load (32 KiB
+// per compute unit and 128 products, as a 256 x 256 tile moves) and reads six 2 KiB fragments (two of A, four of
+// B) from LDS into the operand registers (12 KiB, as a 64 x 128 wavefront tile reads), one step ahead of the
+// products that use them.  Nothing waits on a barrier and the copied bytes are never consumed, so this is what the
+// chip sustains for the GEMM's mix of matrix instructions, fold and data movement when every overlap is perfect.
+__global__ __launch_bounds__(512, 1) void mfma_traffic_kernel(int iters, const int* __restrict__ rnd, float* sink) {
+    extern __shared__ __align__(16) unsigned char lds[];               // 64 KiB of fragments | 64 KiB landing area
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    v4i* frag = (v4i*)lds;
+    for (int i = 0; i < 8; ++i) {
+        const unsigned idx = ((blockIdx.x * 4096 + threadIdx.x * 8 + i) * 4) & 0xffffc;
+        v4i v = *(const v4i*)(rnd + idx);
+        for (int e = 0; e < 4; ++e) v[e] &= 0x7b7b7b7b;                // no NaN codes
+        frag[threadIdx.x * 8 + i] = v;
+    }
+    __syncthreads();
+    auto load = [&](int f) {                                           // fragment f of 32: lane l's two 16-byte halves
+        const v4i lo = frag[(f & 31) * 128 + lane], hi = frag[(f & 31) * 128 + 64 + lane];
+        return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    // Two register sets of A and of B fragments: a step multiplies out of one while the reads for the next step
+    // land in the other (B: four new fragments per step; A: two per step, a new set of four every second step).
+    v8i a[2][4], b[2][4];
+    for (int f = 0; f < 4; ++f) { a[0][f] = load(wave + f); a[1][f] = load(wave + 8 + f); b[0][f] = load(wave + 4 + f); }
+    v4f acc[4][4];
+    for (int i = 0; i < 4; ++i) for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    const float sc = 1.0f + lane * 1e-7f;
+    v4f prev = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t land = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds + 65536u + wave * 4096u;
+    auto step = [&](int it, auto phase) {
+        constexpr int P = decltype(phase)::value, BC = P & 1, AC = P >> 1;
+        const unsigned char* src = (const unsigned char*)rnd + (size_t)(((it * 8 + wave + blockIdx.x * 3) * 4) & 2047) * 1024;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(lane * 16u), "s"(src + c * 1024), "s"(land + BC * 32768u + c * 1024u) : "memory", "m0");
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[BC ^ 1][j] = load(it * 6 + wave + j);
+        a[AC ^ 1][BC * 2] = load(it * 6 + wave + 4);
+        a[AC ^ 1][BC * 2 + 1] = load(it * 6 + wave + 5);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v4f z = {0.f, 0.f, 0.f, 0.f};
+                const v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[AC][i], b[BC][j], z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(prev[e], sc, acc[i][j][e]);
+                prev = p;
+            }
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");               // at most two steps of copies in flight
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int it = 0; it < iters; it += 4) {                            // iters is a multiple of four
+        step(it, std::integral_constant<int, 0>{});
+        step(it + 1, std::integral_constant<int, 1>{});
+        step(it + 2, std::integral_constant<int, 2>{});
+        step(it + 3, std::integral_constant<int, 3>{});
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    float r = prev[0];
+    for (int i = 0; i < 4; ++i) for (int j = 0; j < 4; ++j) r += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+    if (r == 12345.678f) sink[blockIdx.x] = r;
+}
+
 __global__ void null_kernel() {}
 
 int status() { return hipGetLastError() == hipSuccess ? 0 : 1; }
@@ -157,12 +226,21 @@ int dsv3_probe_mix(const void* src, void* dst, size_t bytes_read, int rd, int wr
 }
 
 // flops of one launch: 256 workgroups x 8 wavefronts x iters x 16 x 65536.  rnd: 4 MiB of random bytes.
-// mode 0: constant operands, 1: changing random operands, 2: changing random operands + the fold's four FMAs
+// mode 0: constant operands, 1: changing random operands, 2: changing random operands + the fold's four FMAs,
+// 3: mode 2 with a GEMM step's copies into LDS and fragment reads from LDS around it
 int dsv3_probe_mfma(int iters, int mode, const void* rnd, float* sink, void* stream) {
-    if (!sink || !rnd || iters <= 0 || mode < 0 || mode > 2) return 2;
+    if (!sink || !rnd || iters <= 0 || mode < 0 || mode > 3 || (mode == 3 && iters % 4)) return 2;
     if (mode == 0) hipLaunchKernelGGL(mfma_kernel<0>, dim3(256), dim3(512), 0, (hipStream_t)stream, iters, (const int*)rnd, sink);
     if (mode == 1) hipLaunchKernelGGL(mfma_kernel<1>, dim3(256), dim3(512), 0, (hipStream_t)stream, iters, (const int*)rnd, sink);
     if (mode == 2) hipLaunchKernelGGL(mfma_kernel<2>, dim3(256), dim3(512), 0, (hipStream_t)stream, iters, (const int*)rnd, sink);
+    if (mode == 3) {
+        static bool lds_set = false;                                    // 128 KiB of dynamic LDS needs the attribute once
+        if (!lds_set) {
+            if (hipFuncSetAttribute((const void*)mfma_traffic_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) return 1;
+            lds_set = true;
+        }
+        hipLaunchKernelGGL(mfma_traffic_kernel, dim3(256), dim3(512), 131072, (hipStream_t)stream, iters, (const int*)rnd, sink);
+    }
     return status();
 }
 double dsv3_probe_mfma_flops(int iters) { return 256.0 * 8.0 * iters * 16.0 * 65536.0; }
