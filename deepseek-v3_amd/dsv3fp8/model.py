@@ -365,13 +365,15 @@ class MLP(nn.Module):
         self._w13 = w
         return True
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, quantised: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+        """``quantised``: ``act_quant(x, block_size)`` (no scale format) where the caller already holds it; the
+        stacked projection then starts from it instead of quantising ``x`` once more."""
         if (self.stacked and gemm_impl == "fp8" and world_size == 1 and x.is_cuda and x.dtype == torch.bfloat16
                 and x.is_contiguous() and torch.get_default_dtype() == torch.bfloat16 and block_size == 128
                 and self.w2.bias is None and self.w1.bias is None and self.w3.bias is None and self.stack_13()):
             # one GEMM for both projections, SwiGLU fused with the re-quantisation of w2's input: the same
             # arithmetic and roundings as the three linears and two tensor ops below
-            h = linear(x, self._w13)
+            h = linear(x, self._w13) if quantised is None else fp8_gemm(quantised[0], quantised[1], self._w13, self._w13.scale)
             gq, gs = torch.ops.dsv3fp8.swiglu_quant(h.view(-1, h.size(-1)), block_size, ops._lib.SCALE_FMT_NONE)
             y = fp8_gemm(gq, gs, self.w2.weight, self.w2.weight.scale)
             return y.view(*x.size()[:-1], y.size(-1))
@@ -543,7 +545,9 @@ class MoE(nn.Module):
         h = gemm(xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, code)
         gq, gs = torch.ops.dsv3fp8.swiglu_quant(h, block_size, fmt)
         out = gemm(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code)
-        z = None if fold else self.shared_experts(x).contiguous()
+        # (the shared expert's linears quantise x with no scale format, model.py:233: xq serves them when the routed
+        # experts use none either)
+        z = None if fold else self.shared_experts(x, (xq, xs) if Linear.scale_fmt is None else None).contiguous()
         return torch.ops.dsv3fp8.moe_combine(out, rows, w_sorted, z)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
