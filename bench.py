@@ -439,7 +439,7 @@ def moe_stages(moe, x, Mdl):
     h = t("grouped_w1w3", lambda: g(xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, code))
     gq, gs = t("swiglu_quant", lambda: torch.ops.dsv3fp8.swiglu_quant(h, bs, 0))
     out = t("grouped_w2", lambda: g(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code))
-    z = t("shared_expert", lambda: moe.shared_experts(x).contiguous())
+    z = t("shared_expert", lambda: moe.shared_experts(x, (xq, xs)).contiguous())
     t("moe_combine", lambda: torch.ops.dsv3fp8.moe_combine(out, rows, w_sorted, z))
     st["sum"] = round(sum(st.values()), 1)
     return st
