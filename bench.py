@@ -45,9 +45,13 @@ class Probes:
 
     def __init__(self):
         import ctypes as C
-        path = ROOT / "deepseek-v3_amd" / "lib" / "libdsv3probe.so"
-        if not path.exists():
-            sys.exit(f"bench.py: {path} is missing; run `python deepseek-v3_amd/build.py`.")
+        path = ROOT / "bench" / "probes" / "libdsv3probe.so"
+        if not path.exists():                                  # built by __graft_entry__.build(); only if nothing is there
+            import importlib.util
+            spec = importlib.util.spec_from_file_location("dsv3_probe_build", path.parent / "build.py")
+            mod = importlib.util.module_from_spec(spec)
+            spec.loader.exec_module(mod)
+            mod.build_probes(verbose=False)
         L = self.lib = C.CDLL(str(path))
         L.dsv3_probe_read_stream.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
         L.dsv3_probe_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
@@ -118,7 +122,12 @@ class Probes:
                 "fp8_mfma_loop_TFLOPs": round(self.mfma_tflops(0), 1),
                 "fp8_mfma_loop_changing_operands_TFLOPs": round(self.mfma_tflops(1), 1),
                 "fp8_mfma_loop_with_fold_TFLOPs": round(self.mfma_tflops(2), 1),
+                "fp8_mfma_loop_with_fold_no_shared_operand_TFLOPs": round(self.mfma_tflops(8), 1),
                 "fp8_mfma_loop_with_fold_and_operand_traffic_TFLOPs": round(self.mfma_tflops(3), 1),
+                "fp8_mfma_loop_with_operand_traffic_no_fold_TFLOPs": round(self.mfma_tflops(4), 1),
+                "fp8_mfma_32x32x64_loop_changing_operands_TFLOPs": round(self.mfma_tflops(5), 1),
+                "fp8_mfma_32x32x64_loop_with_fold_TFLOPs": round(self.mfma_tflops(6), 1),
+                "fp8_mfma_32x32x64_loop_with_fold_and_operand_traffic_TFLOPs": round(self.mfma_tflops(7), 1),
                 "empty_launch_us": round(nl, 2),
                 "note": "measured on this GPU in this run: 1 GiB read stream; 1 GiB copy (bytes read + written); streams "
                         "that read two bytes per byte written (the mix of act_quant and weight_quant) and one per two "
@@ -126,11 +135,16 @@ class Probes:
                         "CU: one operand pair for all instructions, 4 x 4 fragments of random bytes accumulated in the "
                         "matrix core (what power-of-two scales allow), and the same with every product folded into "
                         "its accumulator by four FMAs (what binary32 block scales need) -- the chip is power limited, "
-                        "so the rate falls as operands toggle and as vector work is added; that last loop inside the data movement "
+                        "so the rate falls as operands toggle and as vector work is added (no_shared_operand: an issue "
+                        "order in which consecutive instructions share neither operand, where the others share one); "
+                        "the fold loop inside the data movement "
                         "of a 256 x 256 x 128 GEMM step and nothing else (per 16 products a wavefront copies 4 KiB from "
                         "L2 into LDS and reads six 2 KiB fragments from LDS into the operand registers; no barrier, the "
                         "copied bytes are not consumed): what the chip sustains for the GEMM's instruction mix and "
-                        "traffic when every overlap is perfect; empty kernel in a graph"}
+                        "traffic when every overlap is perfect, and the same without the fold (the ceiling of "
+                        "power-of-two scales); the three loops again on v_mfma_f32_32x32x64_f8f6f4, two chained "
+                        "instructions per 128-wide scale block (half the operand-register reads per flop, 16 fold FMAs "
+                        "per 32 x 32 x 128 product); empty kernel in a graph"}
 
 
 def _events(n):
@@ -445,11 +459,39 @@ def moe_stages(moe, x, Mdl):
     return st
 
 
+CPU_THREADS_CAP = 16      # a one-GPU box gives a job 16 host cores, whatever os.cpu_count() shows there
+
+
+def _host() -> dict:
+    model = "unknown"
+    try:
+        for ln in open("/proc/cpuinfo"):
+            if ln.startswith("model name"):
+                model = ln.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"os_cpu_count": os.cpu_count(), "torch_num_threads": torch.get_num_threads(), "cpu_model": model,
+            "threads_cap": CPU_THREADS_CAP}
+
+
+def _cpu_time(fn, budget_s: float, max_passes: int = 8):
+    """Seconds per pass of fn on the host: one untimed pass, then whole passes until budget_s has gone by."""
+    fn()
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or passes >= max_passes:
+            return dt / passes, passes
+
+
 def cpu_baseline(W, rows: int = 1024):
     """The torch-CPU oracle (a port of the reference arithmetic) on the first `rows` tokens of
-    the same workload, all host threads."""
+    the same workload, on the host's threads (at most CPU_THREADS_CAP)."""
     from oracle import oracle
-    torch.set_num_threads(max(1, min(os.cpu_count() or 1, 16)))
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, CPU_THREADS_CAP)))
     x = W.activations(rows, 7168, 0, "cpu")
     w8, ws = W.weight(18432, 7168, 1, "cpu")
     oracle.linear(x[:64], w8, scale=ws)                      # warm-up
@@ -463,7 +505,53 @@ def cpu_baseline(W, rows: int = 1024):
     return {"value": round(2 * rows * passes * 18432 * 7168 / dt / 1e12, 4), "unit": "TFLOP/s",
             "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"oracle.linear() (act_quant + fp8_gemm, fp32 torch-CPU), {passes} passes over {rows} of 4096 rows, "
-                      f"K=7168 -> N=18432, {dt:.2f} s"}
+                      f"K=7168 -> N=18432, {dt:.2f} s", "host": _host()}
+
+
+def cpu_baselines_other_configs(W) -> dict:
+    """The oracle timed on the host for the configurations beside the headline one (the headline's figure is
+    `cpu_baseline`): config 1 whole, config 2 whole (act_quant, weight_dequant), config 3 all cells (fp8_gemm at 1, 8,
+    32, 64 rows over the five projections), config 5 on 16 routed experts and 256 tokens (every token still selects 8
+    experts in 4 of 8 groups; flops 1/16 of the full layer's, stated beside the figure).  About 40 s in all."""
+    from oracle import oracle
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, CPU_THREADS_CAP)))
+    out = {"host": _host()}
+    x, w8, ws = W.cfg1_cpu_plumbing()
+    sec, n = _cpu_time(lambda: oracle.linear(x, w8, scale=ws), 1.0)
+    out["cfg1_linear_16x7168_to_1536"] = {"ms": round(sec * 1e3, 2), "GFLOPs": round(2 * 16 * 1536 * 7168 / sec / 1e9, 1), "passes": n}
+    xa = W.activations(4096, 7168, 0, "cpu", outliers=True)
+    sec, n = _cpu_time(lambda: oracle.act_quant(xa), 2.0, 4)
+    out["cfg2_act_quant_4096x7168"] = {"ms": round(sec * 1e3, 1), "GBps": round(88.998e6 / sec / 1e9, 2), "passes": n}
+    del xa
+    wq, wsc = W.random_fp8_weight(18432, 7168, 2, "cpu")
+    sec, n = _cpu_time(lambda: oracle.weight_dequant(wq, wsc), 3.0, 3)
+    out["cfg2_weight_dequant_18432x7168"] = {"ms": round(sec * 1e3, 1), "GBps": round(396.394e6 / sec / 1e9, 2), "passes": n}
+    del wq, wsc
+    dec = {}
+    for name, (k, nn) in W.DECODE_SHAPES.items():
+        w8, ws = W.weight(nn, k, 1, "cpu")
+        for m in W.DECODE_M:
+            a, a_s = oracle.act_quant(W.activations(m, k, m, "cpu"))
+            sec, n = _cpu_time(lambda: oracle.fp8_gemm(a, a_s, w8, ws), 0.6, 2)
+            dec[f"{name}_{k}to{nn}_M{m}"] = {"ms": round(sec * 1e3, 1), "GBps": round(decode_bytes(m, nn, k) / sec / 1e9, 2)}
+        del w8, ws
+    out["cfg3_decode_fp8_gemm"] = dec
+    # config 5, reduced: 16 routed experts (2 per group), 256 tokens, the same router rule and expert shapes
+    experts_n, tokens, dim, inter = 16, 256, 7168, 2048
+    g = torch.Generator().manual_seed(5)
+    protos = [W.weight(inter, dim, 40, "cpu"), W.weight(dim, inter, 41, "cpu")]
+    ex = (protos[0][0], protos[0][1], protos[1][0], protos[1][1], protos[0][0], protos[0][1])
+    xm = W.activations(tokens, dim, 6, "cpu")
+    scores = (torch.randn(tokens, experts_n, generator=g) * 1.7).bfloat16()
+    wts, idx = oracle.gate_route(scores, torch.randn(experts_n, generator=g) * 0.1, 8, 8, 4, 2.5)
+    wts = wts.type_as(xm)
+    sec, n = _cpu_time(lambda: oracle.moe(xm, wts, idx, [ex] * experts_n, ex), 4.0, 2)
+    flops = 2.0 * 3 * dim * inter * (tokens * 8 + tokens)
+    out["cfg5_moe_16_experts_256_tokens"] = {
+        "ms": round(sec * 1e3, 1), "TFLOPs": round(flops / sec / 1e12, 4), "passes": n,
+        "scaling": "1/16 of the full layer's tokens and routed experts (flops 1/16); at this rate the full layer "
+                   f"(3.247e12 flop) would take {3.247e12 / (flops / sec):.1f} s"}
+    return out
 
 
 def main():
@@ -547,6 +635,8 @@ def main():
     if not args.no_extras:
         line["extras"] = run_extras(K, W, probes, ceil)
         line["roofline_decode"] = decode_roofline(line["extras"]["decode"], ceil)
+        if not args.no_cpu:
+            line["extras"]["cpu_oracle_other_configs"] = cpu_baselines_other_configs(W)
     print(json.dumps(line), flush=True)
 
 

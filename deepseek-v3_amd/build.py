@@ -63,26 +63,7 @@ def build_library(verbose: bool = True) -> Path:
     os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"[build] linked {LIB_PATH}", flush=True)
-    build_probes(verbose)
     return LIB_PATH
-
-
-PROBE_SRC = HERE / "probes" / "probes.hip"
-PROBE_PATH = LIB_DIR / "libdsv3probe.so"
-
-
-def build_probes(verbose: bool = True) -> Path:
-    """libdsv3probe.so: the benchmark's ceiling probes (read stream, copy, MFMA loop, empty launch)."""
-    LIB_DIR.mkdir(exist_ok=True)
-    tmp = PROBE_PATH.with_suffix(".so.tmp")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", str(PROBE_SRC), "-o", str(tmp)]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed on {PROBE_SRC.name}:\n{r.stdout}\n{r.stderr}")
-    os.replace(tmp, PROBE_PATH)
-    if verbose:
-        print(f"[build] linked {PROBE_PATH}", flush=True)
-    return PROBE_PATH
 
 
 if __name__ == "__main__":

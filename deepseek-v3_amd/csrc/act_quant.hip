@@ -50,23 +50,14 @@ template <> struct In<DSV3_F32> {
     }
 };
 
-// The block maximum is taken over the bit patterns of |x| as unsigned integers: for finite values and infinity that
-// is the order of the values, and a NaN (exponent all ones, mantissa non-zero) is larger than everything, so it
-// reaches the scale the way torch's amax and the reference's tl.max let it (v_max_f32 would drop it).
-__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
-template <int CTRL> __device__ __forceinline__ uint32_t dpp_max(uint32_t v) {
-    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
-    return umax(v, o);
-}
-
-// max over the LPB lanes that share a block; every lane ends with the result.
+// max over the LPB lanes that share a block (bit patterns of |x|, see block_scale); every lane ends with the result.
 template <int LPB> __device__ __forceinline__ uint32_t group_max(uint32_t v) {
-    if (LPB >= 2) v = dpp_max<0xB1>(v);    // quad_perm [1,0,3,2]
-    if (LPB >= 4) v = dpp_max<0x4E>(v);    // quad_perm [2,3,0,1]
-    if (LPB >= 8) v = dpp_max<0x141>(v);   // row_half_mirror
-    if (LPB >= 16) v = dpp_max<0x140>(v);  // row_mirror
-    if (LPB >= 32) v = umax(v, (uint32_t)__shfl_xor((int)v, 16));
-    if (LPB >= 64) v = umax(v, (uint32_t)__shfl_xor((int)v, 32));
+    if (LPB >= 2) v = dpp_umax<0xB1>(v);    // quad_perm [1,0,3,2]
+    if (LPB >= 4) v = dpp_umax<0x4E>(v);    // quad_perm [2,3,0,1]
+    if (LPB >= 8) v = dpp_umax<0x141>(v);   // row_half_mirror
+    if (LPB >= 16) v = dpp_umax<0x140>(v);  // row_mirror
+    if (LPB >= 32) v = umax_u32(v, (uint32_t)__shfl_xor((int)v, 16));
+    if (LPB >= 64) v = umax_u32(v, (uint32_t)__shfl_xor((int)v, 32));
     return v;
 }
 
@@ -90,29 +81,20 @@ __global__ __launch_bounds__(kThreads) void act_quant_kernel(
         const int64_t c = base + (int64_t)u * kThreads;
         uint32_t abits = 0u;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) abits = umax(abits, f32_as_u32(f[u][i]) & 0x7fffffffu);
+        for (int i = 0; i < 8; ++i) abits = umax_u32(abits, abs_bits(f[u][i]));
         abits = group_max<LPB>(abits);
-        const bool finite = abits < 0x7f800000u;                 // the same for all lanes of the block
         // infinity gives s = inf (finite elements quantise to 0, infinite ones to NaN), NaN gives s = NaN and a block
-        // of NaN codes: what the IEEE evaluation of the formula gives
-        float sc = abits > 0x7f800000u ? u32_as_f32(0x7fc00000u) : fmaxf(u32_as_f32(abits), 1e-4f) / 448.f;
-        if (UE8M0) {
-            uint32_t b = f32_as_u32(sc);
-            b = ((b >> 23) + ((b & 0x7fffffu) ? 1u : 0u)) << 23;
-            sc = u32_as_f32(b);
-        }
+        // of NaN codes, in both scale formats: what the IEEE evaluation of the formula gives
+        const float sc = block_scale(abits, UE8M0);
+        const bool fast = XD == DSV3_BF16 && block_is_finite(abits);     // the same for all lanes of the block
         float q[8];
-        if (XD == DSV3_BF16 && finite) {
+        if (fast) {
             const float r = 1.0f / sc;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float q0 = f[u][i] * r;
-                const float e = __builtin_fmaf(-q0, sc, f[u][i]);
-                q[i] = __builtin_copysignf(__builtin_fmaf(e, r, q0), f[u][i]);
-            }
+            for (int i = 0; i < 8; ++i) q[i] = block_quotient(f[u][i], sc, r, true);
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) q[i] = f[u][i] / sc;
+            for (int i = 0; i < 8; ++i) q[i] = block_quotient(f[u][i], sc, 0.f, false);
         }
         if (c < n_chunks) {
             v2u o;
@@ -139,6 +121,42 @@ int launch2(const void* x, void* y, float* s, int64_t numel, int scale_fmt, hipS
     return launch_status();
 }
 
+// Any other block size (the reference's wrapper takes every block size that divides the last dimension,
+// inference/kernel.py:38,52): one wavefront per block, the block read twice (maximum, then quotients), one element
+// per lane and step.  Same arithmetic as above with the IEEE division throughout.
+template <int XD> __device__ __forceinline__ float load_elem(const void* x, int64_t i) {
+    if (XD == DSV3_F32) return ((const float*)x)[i];
+    if (XD == DSV3_F16) return (float)((const _Float16*)x)[i];
+    return u32_as_f32((uint32_t)((const uint16_t*)x)[i] << 16);
+}
+template <int XD>
+__global__ __launch_bounds__(kThreads) void act_quant_any_block_kernel(
+        const void* __restrict__ x, uint8_t* __restrict__ y, float* __restrict__ s, int64_t n_blocks, int block, int ue8m0) {
+    const int lane = threadIdx.x & 63;
+    const int64_t blk = (int64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (blk >= n_blocks) return;                             // (wavefront-uniform)
+    const int64_t base = blk * block;
+    uint32_t abits = 0u;
+    for (int i = lane; i < block; i += 64) abits = umax_u32(abits, abs_bits(load_elem<XD>(x, base + i)));
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) abits = umax_u32(abits, (uint32_t)__shfl_xor((int)abits, d));
+    const float sc = block_scale(abits, ue8m0 != 0);
+    for (int i = lane; i < block; i += 64) {
+        const float q = load_elem<XD>(x, base + i) / sc;
+        y[base + i] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(q, q, 0, false) & 0xff);
+    }
+    if (lane == 0) s[blk] = sc;
+}
+
+template <int XD>
+int launch_any_block(const void* x, void* y, float* s, int64_t numel, int block, int fmt, hipStream_t st) {
+    const int64_t n_blocks = numel / block, grid = (n_blocks + kThreads / 64 - 1) / (kThreads / 64);
+    if (grid > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL((act_quant_any_block_kernel<XD>), dim3((unsigned)grid), dim3(kThreads), 0, st,
+                       x, (uint8_t*)y, s, n_blocks, block, fmt == DSV3_SCALE_FMT_UE8M0 ? 1 : 0);
+    return launch_status();
+}
+
 template <int XD>
 int launch1(const void* x, void* y, float* s, int64_t numel, int block, int fmt, hipStream_t st) {
     switch (block) {
@@ -147,7 +165,7 @@ int launch1(const void* x, void* y, float* s, int64_t numel, int block, int fmt,
         case 128: return launch2<XD, 16>(x, y, s, numel, fmt, st);
         case 256: return launch2<XD, 32>(x, y, s, numel, fmt, st);
         case 512: return launch2<XD, 64>(x, y, s, numel, fmt, st);
-        default:  return DSV3_ERR_BAD_BLOCK;
+        default:  return launch_any_block<XD>(x, y, s, numel, block, fmt, st);
     }
 }
 

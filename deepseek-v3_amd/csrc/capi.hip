@@ -59,8 +59,7 @@ int dsv3_act_quant(const void* x, int x_dtype, void* y, float* s,
                    int scale_fmt, void* stream) {
     if (!valid_dtype(x_dtype)) return DSV3_ERR_BAD_DTYPE;
     if (scale_fmt != DSV3_SCALE_FMT_NONE && scale_fmt != DSV3_SCALE_FMT_UE8M0) return DSV3_ERR_BAD_DTYPE;
-    if (block_size != 32 && block_size != 64 && block_size != 128 && block_size != 256 && block_size != 512)
-        return DSV3_ERR_BAD_BLOCK;
+    if (block_size < 1) return DSV3_ERR_BAD_BLOCK;
     if (numel < 0 || last_dim < 0) return DSV3_ERR_BAD_SHAPE;
     if (last_dim % block_size != 0) return DSV3_ERR_BAD_SHAPE;
     if (numel == 0) return DSV3_OK;
@@ -101,7 +100,7 @@ size_t dsv3_fp8_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
 // Host-side checks of the fp8_gemm entry points (no GPU call).  DSV3_OK with m == 0 or n == 0 means "nothing to do".
 static int fp8_gemm_validate(const void* a, const float* a_s, const void* b, const float* b_s,
                              void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
-                             void* workspace, size_t workspace_bytes) {
+                             void* workspace, size_t workspace_bytes, bool check_workspace = true) {
     if (!valid_dtype(c_dtype)) return DSV3_ERR_BAD_DTYPE;
     if (m < 0 || n < 0 || k < 0) return DSV3_ERR_BAD_SHAPE;
     if (k % 128 != 0) return DSV3_ERR_BAD_SHAPE;
@@ -112,6 +111,7 @@ static int fp8_gemm_validate(const void* a, const float* a_s, const void* b, con
     if (!aligned(a, 16) || !aligned(b, 16) || !aligned(a_s, 4) || !aligned(b_s, 4) ||
         !aligned(c, c_dtype == DSV3_F32 ? 16 : 8))
         return DSV3_ERR_MISALIGNED;
+    if (!check_workspace) return DSV3_OK;
     const size_t need = dsv3_fp8_gemm_workspace_bytes(m, n, k);
     if (need > 0 && (!workspace || workspace_bytes < need || !aligned(workspace, 256))) return DSV3_ERR_WORKSPACE;
     return DSV3_OK;
@@ -142,12 +142,12 @@ size_t dsv3_fp8_gemm_static_max_bytes(void) { return DSV3_STATIC_SCRATCH_BYTES; 
 
 int dsv3_fp8_gemm_static(const void* a, const float* a_s, const void* b, const float* b_s,
                          void* c, int c_dtype, int64_t m, int64_t n, int64_t k, void* stream) {
-    const size_t need = dsv3_fp8_gemm_workspace_bytes(m, n, k);          // 0 for shapes the checks below refuse
-    if (need > DSV3_STATIC_SCRATCH_BYTES) return DSV3_ERR_TOO_LARGE;     // refused before anything is launched
-    // the argument checks of dsv3_fp8_gemm, with a stand-in for the workspace: no GPU call on an error path
-    alignas(256) static unsigned char stand_in;
-    const int rc = fp8_gemm_validate(a, a_s, b, b_s, c, c_dtype, m, n, k, need ? &stand_in : nullptr, need);
+    // the argument checks of dsv3_fp8_gemm first (no GPU call on an error path), then the size of the scratch: a
+    // malformed call reports what is wrong with it, not DSV3_ERR_TOO_LARGE
+    const int rc = fp8_gemm_validate(a, a_s, b, b_s, c, c_dtype, m, n, k, nullptr, 0, false);
     if (rc != DSV3_OK || m == 0 || n == 0) return rc;
+    const size_t need = dsv3_fp8_gemm_workspace_bytes(m, n, k);
+    if (need > DSV3_STATIC_SCRATCH_BYTES) return DSV3_ERR_TOO_LARGE;     // refused before anything is launched
     void* ws = nullptr;
     if (need) {
         ws = static_scratch();

@@ -54,6 +54,36 @@ __device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float 
 __device__ __forceinline__ v2f fp8x2_lo_to_f32(uint32_t p) { return __builtin_amdgcn_cvt_pk_f32_fp8((int)p, false); }
 __device__ __forceinline__ v2f fp8x2_hi_to_f32(uint32_t p) { return __builtin_amdgcn_cvt_pk_f32_fp8((int)p, true); }
 
+// Scale of a quantisation block (inference/kernel.py:26-31) from the largest bit pattern of |x| among its
+// elements.  As unsigned integers the patterns of finite values and infinity are ordered like the values, and a NaN
+// (exponent all ones, mantissa non-zero) is larger than all of them, so it reaches the scale as it does through
+// torch's amax (v_max_f32 would drop it): NaN -> s = NaN, infinity -> s = inf, otherwise max(amax, 1e-4) / 448,
+// rounded up to a power of two for the ue8m0 format (non-finite scales pass through unchanged).
+__device__ __forceinline__ uint32_t umax_u32(uint32_t a, uint32_t b) { return a > b ? a : b; }
+__device__ __forceinline__ uint32_t abs_bits(float f) { return f32_as_u32(f) & 0x7fffffffu; }
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_umax(uint32_t v) {
+    return umax_u32(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ bool block_is_finite(uint32_t abits) { return abits < 0x7f800000u; }
+__device__ __forceinline__ float block_scale(uint32_t abits, bool ue8m0) {
+    float sc = abits > 0x7f800000u ? u32_as_f32(0x7fc00000u) : fmaxf(u32_as_f32(abits), 1e-4f) / 448.f;
+    if (ue8m0 && block_is_finite(abits)) {
+        const uint32_t b = f32_as_u32(sc);
+        sc = u32_as_f32(((b >> 23) + ((b & 0x7fffffu) ? 1u : 0u)) << 23);
+    }
+    return sc;
+}
+// x / sc for a block element.  FAST (bf16 x of a finite block, |x| <= amax): a reciprocal and one correction step,
+// equal to the correctly rounded quotient wherever the e4m3 rounding can tell (oracle/check_fast_division.c
+// enumerates it); otherwise the IEEE division.
+__device__ __forceinline__ float block_quotient(float x, float sc, float r, bool fast) {
+    if (fast) {
+        const float q0 = x * r;
+        return __builtin_copysignf(__builtin_fmaf(__builtin_fmaf(-q0, sc, x), r, q0), x);
+    }
+    return x / sc;
+}
+
 // Output element writers: one binary32 -> C element of dsv3_dtype T.
 template <int DT> struct OutT;
 template <> struct OutT<DSV3_BF16> { typedef uint16_t type; static constexpr int bytes = 2; };

@@ -35,40 +35,6 @@
 
 namespace pingpong {
 
-// Development aid (never defined in the library build): per-phase time stamps of every wavefront.
-#ifndef DSV3_PP_ABL
-#define DSV3_PP_ABL 0
-#endif
-#ifdef DSV3_PP_PROF
-__device__ unsigned long long pp_prof[8 * 8];
-#ifdef PP_NO_STAMPS
-#define PP_PROF_DECL
-#define PP_PROF_MARK(slot)
-#define PP_PROF_FLUSH
-#else
-#define PP_PROF_DECL unsigned long long prof_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, prof_t; \
-    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(prof_t) :: "memory");
-#define PP_PROF_MARK(slot) { unsigned long long t_; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_) :: "memory"); \
-    prof_acc[slot] += t_ - prof_t; prof_t = t_; }
-#define PP_PROF_FLUSH if (lane == 0) { for (int i_ = 0; i_ < 8; ++i_) atomicAdd(&pp_prof[wave * 8 + i_], prof_acc[i_]); }
-#endif
-__device__ unsigned long long pp_clk[4];
-#define PP_CLK(i) if (wg == 0 && threadIdx.x == 0) { unsigned long long c_, r_; \
-    asm volatile("s_memtime %0\n\ts_memrealtime %1\n\ts_waitcnt lgkmcnt(0)" : "=s"(c_), "=s"(r_) :: "memory"); pp_clk[i] = c_; pp_clk[i + 1] = r_; }
-#else
-#define PP_PROF_DECL
-#define PP_PROF_MARK(slot)
-#define PP_PROF_FLUSH
-#define PP_CLK(i)
-#endif
-#ifdef DSV3_PP_TRACE
-__device__ unsigned long long pp_trace[8192 * 4];
-#define PP_TRACE(i) if (threadIdx.x == 0) { unsigned long long r_; \
-    asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r_) :: "memory"); pp_trace[(cur_w & 8191) * 4 + (i)] = r_; }
-#else
-#define PP_TRACE(i)
-#endif
-
 // One global -> LDS copy of 16 (or 4) bytes per lane: uniform 64-bit base in scalar registers, 32-bit lane offset,
 // uniform LDS address through M0 (lane l lands at lds_addr + 16 l).  Written out because the compiler otherwise
 // forms a 64-bit address per lane with vector ALU instructions in front of every copy.
@@ -156,7 +122,7 @@ __device__ __forceinline__ void tile(
     }
     // row of a behind row r of the tile; rows past the tile's end repeat its last row (their results are dropped).
     // In persistent mode the tile's origin is part of the copies' scalar base address instead (cur / nxt below).
-    const int m0_ld = (PS || (DSV3_PP_ABL & 16)) ? 0 : m0, n0_ld = (PS || (DSV3_PP_ABL & 16)) ? 0 : n0;
+    const int m0_ld = PS ? 0 : m0, n0_ld = PS ? 0 : n0;
     auto a_row = [&](int r) -> uint32_t {
         const int rr = m0_ld + min(r, rows_here - 1);
         return (uint32_t)((G && g.a_rows) ? g.a_rows[rr] : rr);
@@ -182,7 +148,6 @@ __device__ __forceinline__ void tile(
     bool has_next = PS && cur_w + wg_stride < T;
     if (has_next) dense_origin(cur_w + wg_stride, m0n, n0n);
     Origin cur = origin_of(m0, n0), nxt = origin_of(m0n, n0n);
-    PP_TRACE(0)
 
     // ---- copy plan.  A K block is TM / 8 + 32 wavefront-copies of 8 rows (1 KiB); copy q covers rows 8q .. 8q + 7.
     // The copies are requested in the M phases, interleaved with the LDS reads (the copy path takes one 1 KiB copy
@@ -308,7 +273,6 @@ __device__ __forceinline__ void tile(
 #define DSV3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
     auto run = [&](auto gtag) {
         constexpr int GRP = decltype(gtag)::value;
-        constexpr bool LD = !(DSV3_PP_ABL & 2), RD = !(DSV3_PP_ABL & 4), STRICT = (DSV3_PP_ABL & 256) != 0;
         // prologue: blocks 0 and 1 as far as the steady state expects them to have been requested
 #pragma unroll
         for (int t = 0; t < NM2; ++t) issue_m2(t, 0, 0);
@@ -320,8 +284,6 @@ __device__ __forceinline__ void tile(
         issue_scales(min(1, KB - 1), 1);
         __builtin_amdgcn_s_waitcnt(0x0f70);                         // vmcnt(0)
         wg_barrier();
-        PP_TRACE(1)
-        if (STRICT && GRP == 1) wg_barrier();                       // one phase behind group 0 from here on
 
         v8i af[SM], bf[4];
         v4f p14 = {0.f, 0.f, 0.f, 0.f}, p15 = {0.f, 0.f, 0.f, 0.f}; // raw products of the last two MFMAs of a C phase
@@ -337,8 +299,11 @@ __device__ __forceinline__ void tile(
         auto compute = [&](auto i0_tag, auto it_tag, const float (&s)[SM], const float (&st)[SM]) {
             constexpr int I0 = decltype(i0_tag)::value, IT = decltype(it_tag)::value;
             constexpr int NT = 4 * SM;
+            // activation sub-tile of MFMA t: the SM sub-tiles are walked forwards for even weight fragments and
+            // backwards for odd ones, so that consecutive instructions always share one operand (measured 0.5 %)
+            auto SJ = [](int t) { return ((t / SM) & 1) ? SM - 1 - (t % SM) : (t % SM); };
             __builtin_amdgcn_sched_barrier(0);
-            if ((DSV3_PP_ABL & 1) || (!STRICT && GRP == 1)) __builtin_amdgcn_s_setprio(3);
+            if (GRP == 1) __builtin_amdgcn_s_setprio(3);
             if constexpr (P2) {
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii)
@@ -351,29 +316,26 @@ __device__ __forceinline__ void tile(
                 v4f p[NT];
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    p[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[t / SM], af[t % SM], z, 0, 0, 0, 0, 0, 0);
-                    if (!(DSV3_PP_ABL & 8)) {
-                        if (t < 2) {
-                            const v4f q = t == 0 ? p14 : p15;
+                    p[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[t / SM], af[SJ(t)], z, 0, 0, 0, 0, 0, 0);
+                    if (t < 2) {
+                        const v4f q = t == 0 ? p14 : p15;
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) acc[IT][SM - 2 + t][e] = __builtin_fmaf(q[e], st[SM - 2 + t], acc[IT][SM - 2 + t][e]);
-                        } else {
-                            const int u = t - 2;
+                        for (int e = 0; e < 4; ++e) acc[IT][SJ(NT - 2 + t)][e] = __builtin_fmaf(q[e], st[SJ(NT - 2 + t)], acc[IT][SJ(NT - 2 + t)][e]);
+                    } else {
+                        const int u = t - 2;
 #pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                acc[I0 + u / SM][u % SM][e] = __builtin_fmaf(p[u][e], s[u % SM], acc[I0 + u / SM][u % SM][e]);
-                        }
+                        for (int e = 0; e < 4; ++e)
+                            acc[I0 + u / SM][SJ(u)][e] = __builtin_fmaf(p[u][e], s[SJ(u)], acc[I0 + u / SM][SJ(u)][e]);
                     }
                     DSV3_SGB(0x008, 1);
-                    if (!(DSV3_PP_ABL & 8)) DSV3_SGB(0x002, 4);
+                    DSV3_SGB(0x002, 4);
                 }
                 p14 = p[NT - 2]; p15 = p[NT - 1];
             }
-            if ((DSV3_PP_ABL & 1) || (!STRICT && GRP == 1)) __builtin_amdgcn_s_setprio(0);
+            if (GRP == 1) __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
         };
 
-        PP_PROF_DECL
         // one K block whose LDS stage (and scale slot) ST is a compile-time constant: every LDS address of the loop is
         // a register plus an immediate
         auto block = [&](int kb, auto st_tag, auto tail_tag) {
@@ -386,7 +348,7 @@ __device__ __forceinline__ void tile(
             asm volatile("" : "+s"(kb_m1));
             const int kb1 = PS ? kb_m1 + 1 : min(kb_m1 + 1, KB - 1);
             // ---- M1
-            if (RD || kb == 0) {
+            {
                 const uint8_t* as_base = a_rd + ST * A_STAGE;
                 const uint8_t* bs_base = b_rd + ST * B_STAGE;
                 // copy t goes in front of fragment read t (SM + 4) / n of the phase's SM + 4
@@ -395,14 +357,14 @@ __device__ __forceinline__ void tile(
                 for (int j = 0; j < SM; ++j) {
 #pragma unroll
                     for (int t = 0; t < N1; ++t)
-                        if (LD && t * (SM + 4) / N1 == j) issue_m1(t, kb1, ST ^ 1, TAIL);
+                        if (t * (SM + 4) / N1 == j) issue_m1(t, kb1, ST ^ 1, TAIL);
                     af[j] = join(*(const v4i*)(as_base + j * 2048 + c0), *(const v4i*)(as_base + j * 2048 + c1));
                 }
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
 #pragma unroll
                     for (int t = 0; t < N1; ++t)
-                        if (LD && t * (SM + 4) / N1 == SM + ii) issue_m1(t, kb1, ST ^ 1, TAIL);
+                        if (t * (SM + 4) / N1 == SM + ii) issue_m1(t, kb1, ST ^ 1, TAIL);
                     bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
                 }
             }
@@ -417,15 +379,11 @@ __device__ __forceinline__ void tile(
                 if (P2) eb = (int)(f32_as_u32(bs) >> 23);
             }
             __builtin_amdgcn_sched_barrier(0);
-            PP_PROF_MARK(0)
-            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G1);
-            if (STRICT || GRP == 1) wg_barrier();
-            PP_PROF_MARK(1)
+            if (GRP == 1) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G1);
+            if (GRP == 1) wg_barrier();
             // ---- C1 (its first two FMA groups belong to C2 of the previous block: zeros at kb = 0)
             compute(std::integral_constant<int, 0>{}, std::integral_constant<int, 7>{}, sc[ST], sc[ST ^ 1]);
-            PP_PROF_MARK(2)
-            if (STRICT || GRP == 0) wg_barrier();                   // (nothing group 0 has requested is read in the next phase)
-            PP_PROF_MARK(3)
+            if (GRP == 0) wg_barrier();                   // (nothing group 0 has requested is read in the next phase)
             // ---- M2
             {
                 int kb_m2 = kb;
@@ -434,22 +392,18 @@ __device__ __forceinline__ void tile(
                 const uint8_t* bs_base = b_rd + ST * B_STAGE + 4 * 2048;
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
-                    if (LD && ii < NM2) issue_m2(ii, kb2, ST, TAIL);
-                    if (RD) bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
+                    if (ii < NM2) issue_m2(ii, kb2, ST, TAIL);
+                    bf[ii] = join(*(const v4i*)(bs_base + ii * 2048 + c0), *(const v4i*)(bs_base + ii * 2048 + c1));
                 }
-                if (LD) issue_scales(kb2, ST, TAIL);
+                issue_scales(kb2, ST, TAIL);
             }
             __builtin_amdgcn_sched_barrier(0);
-            PP_PROF_MARK(4)
-            if (GRP == 1 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G1);
-            if (STRICT || GRP == 1) wg_barrier();
-            PP_PROF_MARK(5)
+            if (GRP == 1) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G1);
+            if (GRP == 1) wg_barrier();
             // ---- C2
             compute(std::integral_constant<int, 4>{}, std::integral_constant<int, 3>{}, sc[ST], sc[ST]);
-            PP_PROF_MARK(6)
-            if (GRP == 0 && !(DSV3_PP_ABL & 32)) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G0);
-            if (STRICT || GRP == 0) wg_barrier();
-            PP_PROF_MARK(7)
+            if (GRP == 0) __builtin_amdgcn_s_waitcnt(0x0f70 | GEO::WAIT_G0);
+            if (GRP == 0) wg_barrier();
         };
 
         for (;;) {                                                  // (one pass unless persistent)
@@ -475,8 +429,8 @@ __device__ __forceinline__ void tile(
                 const int last = (KB - 1) & 1;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    acc[7][SM - 2][e] = __builtin_fmaf(p14[e], last ? sc[1][SM - 2] : sc[0][SM - 2], acc[7][SM - 2][e]);
-                    acc[7][SM - 1][e] = __builtin_fmaf(p15[e], last ? sc[1][SM - 1] : sc[0][SM - 1], acc[7][SM - 1][e]);
+                    acc[7][1][e] = __builtin_fmaf(p14[e], last ? sc[1][1] : sc[0][1], acc[7][1][e]);
+                    acc[7][0][e] = __builtin_fmaf(p15[e], last ? sc[1][0] : sc[0][0], acc[7][0][e]);
                 }
             }
             if constexpr (!PS) break;
@@ -484,9 +438,7 @@ __device__ __forceinline__ void tile(
                 // the tile's results leave through this wavefront's own staging area (no barrier: the other group
                 // is one phase behind and meets this wavefront again at the next tile's first barrier); then the
                 // next tile, whose first two blocks have been requested by the blocks just finished
-                PP_TRACE(2)
                 ps_epilogue();
-                PP_TRACE(3)
                 if (!has_next) break;
                 cur_w += wg_stride;
                 m0 = m0n; n0 = n0n; cur = nxt;
@@ -495,20 +447,14 @@ __device__ __forceinline__ void tile(
                 p14 = p15 = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int j = 0; j < SM; ++j) sc[0][j] = sc[1][j] = 0.f;
-                PP_TRACE(0)
             }
         }
-        PP_PROF_FLUSH
-        if (STRICT && GRP == 0) wg_barrier();                       // group 1's last phase
         __builtin_amdgcn_s_waitcnt(0x0f70);                         // the clamped refills of the last blocks
     };
-    PP_CLK(0)
     if (grp == 0) run(std::integral_constant<int, 0>{});
     else          run(std::integral_constant<int, 1>{});
-    PP_CLK(2)
 #undef DSV3_SGB
     if constexpr (PS) return;
-    PP_TRACE(2)
 
     // ---- epilogue: lane holds c[m][n .. n + 3] for every (i, j); see fp8_gemm_prefill.hip for the LDS route
     constexpr int WN = 128, SN = 8;
@@ -539,10 +485,6 @@ __device__ __forceinline__ void tile(
             if (r < rows_here && n < N)
                 *(v4u*)(c + (size_t)(m0 + r) * N + n) = v;
         }
-#ifdef DSV3_PP_TRACE
-        __builtin_amdgcn_s_waitcnt(0x0f70);
-        PP_TRACE(3)
-#endif
         return;
     }
     if (f32_lds_epilogue) {

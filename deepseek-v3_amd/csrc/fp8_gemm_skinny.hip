@@ -64,11 +64,6 @@ constexpr int kSlabChunks = 4;             // 16-byte activation chunks a thread
 // workgroup quantises its K range of them on the way into LDS exactly as act_quant would (amax over the 128
 // block, clamp at 1e-4, / 448, optional power-of-two rounding of the scale, correctly rounded quotient, OCP e4m3),
 // so the result equals act_quant followed by this kernel bit for bit and the separate launch disappears.
-template <int CTRL> __device__ __forceinline__ float dpp_max(float v) {
-    int o = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
-    return fmaxf(v, __builtin_bit_cast(float, o));
-}
-
 // 16-byte non-temporal load from (scalar base + 32-bit lane offset + immediate), and a wait until at most n vector
 // loads of the wavefront are outstanding with the ring slot threaded through it (so that the slot's consumers cannot
 // be scheduled ahead of the wait): the RING variant's weight loads and waits are written out, because the compiler's
@@ -198,26 +193,21 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
                     f[8 * h + 2 * e] = bf16lo_to_f32(raw[i][h][e]);
                     f[8 * h + 2 * e + 1] = bf16hi_to_f32(raw[i][h][e]);
                 }
-            float amax = 0.f;
+            uint32_t abits = 0u;                 // non-finite values reach the scale as in act_quant
 #pragma unroll
-            for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(f[e]));
-            amax = dpp_max<0xB1>(amax);      // quad_perm [1,0,3,2]
-            amax = dpp_max<0x4E>(amax);      // quad_perm [2,3,0,1]
-            amax = dpp_max<0x141>(amax);     // row_half_mirror
-            amax = fmaxf(amax, 1e-4f);
-            float sc = amax / 448.f;
-            if (ue8m0) {
-                uint32_t bits = f32_as_u32(sc);
-                bits = ((bits >> 23) + ((bits & 0x7fffffu) ? 1u : 0u)) << 23;
-                sc = u32_as_f32(bits);
-            }
-            const float r = 1.0f / sc;
+            for (int e = 0; e < 16; ++e) abits = umax_u32(abits, abs_bits(f[e]));
+            abits = dpp_umax<0xB1>(abits);       // quad_perm [1,0,3,2]
+            abits = dpp_umax<0x4E>(abits);       // quad_perm [2,3,0,1]
+            abits = dpp_umax<0x141>(abits);      // row_half_mirror
+            const float sc = block_scale(abits, ue8m0 != 0);
             float q[16];
+            if (block_is_finite(abits)) {        // x / sc, correctly rounded for bf16 x with |x| <= amax (as act_quant)
+                const float r = 1.0f / sc;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {       // x / sc, correctly rounded for bf16 x with |x| <= amax (as act_quant)
-                const float q0 = f[e] * r;
-                const float er = __builtin_fmaf(-q0, sc, f[e]);
-                q[e] = __builtin_copysignf(__builtin_fmaf(er, r, q0), f[e]);
+                for (int e = 0; e < 16; ++e) q[e] = block_quotient(f[e], sc, r, true);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) q[e] = block_quotient(f[e], sc, 0.f, false);
             }
             const int c = tid + i * (int)blockDim.x;
             if (c < chunks) {

@@ -18,11 +18,6 @@ constexpr int kThreads = 256;
 
 __device__ __forceinline__ float round_bf16(float v) { return bf16lo_to_f32(pack_bf16(v, 0.f) & 0xffffu); }
 
-template <int CTRL> __device__ __forceinline__ float dpp_max(float v) {
-    int o = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
-    return fmaxf(v, __builtin_bit_cast(float, o));
-}
-
 // h: [rows, 2*inter] bf16 (h1 | h3 side by side), y: [rows, inter] e4m3, s: [rows, inter/128].
 // A lane owns 8 consecutive output columns; the 16 lanes of a DPP row own one 128-wide scale block.
 template <bool UE8M0>
@@ -65,28 +60,23 @@ __global__ __launch_bounds__(kThreads) void swiglu_quant_kernel(
             g[i] = live ? round_bf16(sl * x3[i]) : 0.f;
         }
     }
-    float amax = 0.f;
+    uint32_t abits = 0u;             // non-finite values reach the scale as in act_quant
 #pragma unroll
-    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(g[i]));
-    amax = dpp_max<0xB1>(amax);    // quad_perm [1,0,3,2]
-    amax = dpp_max<0x4E>(amax);    // quad_perm [2,3,0,1]
-    amax = dpp_max<0x141>(amax);   // row_half_mirror
-    amax = dpp_max<0x140>(amax);   // row_mirror
-    amax = fmaxf(amax, 1e-4f);
-    float sc = amax / 448.f;
-    if (UE8M0) {
-        uint32_t bits = f32_as_u32(sc);
-        bits = ((bits >> 23) + ((bits & 0x7fffffu) ? 1u : 0u)) << 23;
-        sc = u32_as_f32(bits);
-    }
+    for (int i = 0; i < 8; ++i) abits = umax_u32(abits, abs_bits(g[i]));
+    abits = dpp_umax<0xB1>(abits);   // quad_perm [1,0,3,2]
+    abits = dpp_umax<0x4E>(abits);   // quad_perm [2,3,0,1]
+    abits = dpp_umax<0x141>(abits);  // row_half_mirror
+    abits = dpp_umax<0x140>(abits);  // row_mirror
+    const float sc = block_scale(abits, UE8M0);
     // correctly rounded g / sc for bf16 g with |g| <= amax (same evaluation as act_quant)
-    const float r = 1.0f / sc;
     float q[8];
+    if (block_is_finite(abits)) {
+        const float r = 1.0f / sc;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float q0 = g[i] * r;
-        const float e = __builtin_fmaf(-q0, sc, g[i]);
-        q[i] = __builtin_copysignf(__builtin_fmaf(e, r, q0), g[i]);
+        for (int i = 0; i < 8; ++i) q[i] = block_quotient(g[i], sc, r, true);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = block_quotient(g[i], sc, 0.f, false);
     }
     if (live) {
         v2u o;

@@ -17,6 +17,7 @@
 //
 // w / s for bf16 w uses the same reciprocal-and-correction sequence as act_quant (see act_quant.hip: exact wherever
 // the e4m3 rounding can see a difference, for |w| <= amax); wider inputs use the IEEE division.
+#include <type_traits>
 #include "common.hpp"
 
 namespace dsv3 {
@@ -56,17 +57,12 @@ template <int XD> __device__ __forceinline__ void load8(const void* p, int64_t i
     }
 }
 
-template <int CTRL> __device__ __forceinline__ float dpp_max(float v) {
-    int o = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
-    return fmaxf(v, __builtin_bit_cast(float, o));
-}
-
 // VEC: n % 8 == 0 and 16-byte aligned bases, so an 8-element chunk is loaded and stored whole and lies entirely
 // inside or outside the matrix; otherwise every element is guarded on its own.
 template <int XD, bool VEC>
 __global__ __launch_bounds__(kThreads) void weight_quant_kernel(
         const void* __restrict__ w, uint8_t* __restrict__ y, float* __restrict__ s, int m, int n, int nb, int ue8m0) {
-    __shared__ float wave_max[kThreads / kWave];
+    __shared__ uint32_t wave_max[kThreads / kWave];
     const int t = threadIdx.x;
     const int col = blockIdx.x * 128 + (t & 15) * 8;           // first of the thread's 8 columns
     const int row0 = blockIdx.y * 128 + (t >> 4);              // its rows: row0 + 16 i
@@ -89,54 +85,48 @@ __global__ __launch_bounds__(kThreads) void weight_quant_kernel(
         }
     }
 
-    float amax = 0.f;
+    uint32_t abits = 0u;                       // non-finite values reach the scale as in act_quant
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(f[i][e]));
-    amax = dpp_max<0xB1>(amax);      // quad_perm [1,0,3,2]
-    amax = dpp_max<0x4E>(amax);      // quad_perm [2,3,0,1]
-    amax = dpp_max<0x141>(amax);     // row_half_mirror
-    amax = dpp_max<0x140>(amax);     // row_mirror: the 16 lanes of a DPP row agree
-    amax = fmaxf(amax, __shfl_xor(amax, 16));
-    amax = fmaxf(amax, __shfl_xor(amax, 32));
-    if ((t & 63) == 0) wave_max[t >> 6] = amax;
+        for (int e = 0; e < 8; ++e) abits = umax_u32(abits, abs_bits(f[i][e]));
+    abits = dpp_umax<0xB1>(abits);             // quad_perm [1,0,3,2]
+    abits = dpp_umax<0x4E>(abits);             // quad_perm [2,3,0,1]
+    abits = dpp_umax<0x141>(abits);            // row_half_mirror
+    abits = dpp_umax<0x140>(abits);            // row_mirror: the 16 lanes of a DPP row agree
+    abits = umax_u32(abits, (uint32_t)__shfl_xor((int)abits, 16));
+    abits = umax_u32(abits, (uint32_t)__shfl_xor((int)abits, 32));
+    if ((t & 63) == 0) wave_max[t >> 6] = abits;
     __syncthreads();
-    amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
-    amax = fmaxf(amax, 1e-4f);
-    float sc = amax / 448.f;
-    if (ue8m0) {                                // round the scale up to a power of two, as act_quant does (kernel.py:29-31)
-        uint32_t bits = f32_as_u32(sc);
-        bits = ((bits >> 23) + ((bits & 0x7fffffu) ? 1u : 0u)) << 23;
-        sc = u32_as_f32(bits);
-    }
+    abits = umax_u32(umax_u32(wave_max[0], wave_max[1]), umax_u32(wave_max[2], wave_max[3]));
+    // (ue8m0: the scale rounded up to a power of two, as act_quant does, kernel.py:29-31)
+    const float sc = block_scale(abits, ue8m0 != 0);
+    const bool fast = XD == DSV3_BF16 && block_is_finite(abits);
     if (t == 0) s[(int64_t)blockIdx.y * nb + blockIdx.x] = sc;
 
-    const float r = 1.0f / sc;
+    // (a workgroup-uniform branch around the whole write-out: one of the two division sequences is executed)
+    auto write_out = [&](auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+        const float r = FAST ? 1.0f / sc : 0.f;
 #pragma unroll
-    for (int i = 0; i < kRowsPerThread; ++i) {
-        const int row = row0 + 16 * i;
-        float q[8];
+        for (int i = 0; i < kRowsPerThread; ++i) {
+            const int row = row0 + 16 * i;
+            float q[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            if (XD == DSV3_BF16) {
-                const float q0 = f[i][e] * r;
-                const float er = __builtin_fmaf(-q0, sc, f[i][e]);
-                q[e] = __builtin_copysignf(__builtin_fmaf(er, r, q0), f[i][e]);
-            } else {
-                q[e] = f[i][e] / sc;
+            for (int e = 0; e < 8; ++e) q[e] = block_quotient(f[i][e], sc, r, FAST);
+            const v2u o = { pack_fp8x4(q[0], q[1], q[2], q[3]), pack_fp8x4(q[4], q[5], q[6], q[7]) };
+            const int64_t at = (int64_t)row * n + col;
+            if (VEC) {
+                if (row < m && col < n) __builtin_nontemporal_store(o, (v2u*)(y + at));
+            } else if (row < m) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (col + e < n) y[at + e] = (uint8_t)((o[e >> 2] >> (8 * (e & 3))) & 0xffu);
             }
         }
-        const v2u o = { pack_fp8x4(q[0], q[1], q[2], q[3]), pack_fp8x4(q[4], q[5], q[6], q[7]) };
-        const int64_t at = (int64_t)row * n + col;
-        if (VEC) {
-            if (row < m && col < n) __builtin_nontemporal_store(o, (v2u*)(y + at));
-        } else if (row < m) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (col + e < n) y[at + e] = (uint8_t)((o[e >> 2] >> (8 * (e & 3))) & 0xffu);
-        }
-    }
+    };
+    if (fast) write_out(std::true_type{});
+    else      write_out(std::false_type{});
 }
 
 template <int XD>

@@ -213,12 +213,16 @@ def apply_rotary_emb(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
 class MLA(nn.Module):
     """Host of the two ``wkv_b`` products of the absorbed multi-head latent attention (model.py:395-497).
 
-    Only the reference's default cache layout (``attn_impl == "absorb"``) is hosted: the compressed latent
+    In the reference's default cache layout (``attn_impl == "absorb"``) the compressed latent
     (``kv_cache`` [b, t, kv_lora_rank]) and the shared rotary key (``pe_cache``) are cached and the up-projection
     ``wkv_b`` is folded into the query (``q_nope @ wkv_b[:, :nope]``, before the scores) and into the output
     (``@ wkv_b[:, -v:]^T``, after the weighted sum).  With ``wkv_b`` in FP8 the reference dequantises the whole
     weight on every call (model.py:481); here the two products read the FP8 weight and its block scales in place
     (``torch.ops.dsv3fp8.wkv_b_absorb``) with the same bf16 rounding of every dequantised weight.
+    ``attn_impl == "naive"`` (model.py:443-445, 470-479, 488-490) caches per-head keys and values instead
+    (``k_cache`` [b, t, h, nope + rope], ``v_cache`` [b, t, h, v]): ``wkv_b`` is then an ordinary linear layer on
+    the new positions' latents (an FP8 GEMM through ``linear()``), and the scores and the weighted sum are plain
+    per-head einsums.
     ``MLA.fused = False`` selects the dequantise-then-einsum sequence instead.  Everything between the two products
     (scores, softmax, weighted sum) is bf16 torch arithmetic that never touches FP8 data; it is here so that the
     products can be tested in place.  Parameter names are the checkpoint's.
@@ -234,8 +238,9 @@ class MLA(nn.Module):
 
     def __init__(self, args: ModelArgs):
         super().__init__()
-        if attn_impl != "absorb":
-            raise NotImplementedError("only the absorbed cache layout (the reference's default) is hosted")
+        if attn_impl not in ("absorb", "naive"):
+            raise ValueError(f"attn_impl must be 'absorb' or 'naive', not {attn_impl!r}")
+        self.attn_impl = attn_impl
         nope, rope, v = args.qk_nope_head_dim, args.qk_rope_head_dim, args.v_head_dim
         self.dim, self.n_heads, self.n_local_heads = args.dim, args.n_heads, args.n_heads // world_size
         self.q_lora_rank, self.kv_lora_rank = args.q_lora_rank, args.kv_lora_rank
@@ -255,8 +260,12 @@ class MLA(nn.Module):
         # 1/sqrt(d), times the YaRN magnitude correction squared when the window is extended (model.py:438-441)
         yarn = 0.1 * args.mscale * math.log(args.rope_factor) + 1.0 if args.max_seq_len > args.original_seq_len else 1.0
         self.softmax_scale = self.qk_head_dim ** -0.5 * yarn * yarn
-        for name, width in (("kv_cache", self.kv_lora_rank), ("pe_cache", rope)):
-            self.register_buffer(name, torch.zeros(args.max_batch_size, args.max_seq_len, width), persistent=False)
+        if self.attn_impl == "naive":
+            caches = (("k_cache", (self.n_local_heads, self.qk_head_dim)), ("v_cache", (self.n_local_heads, v)))
+        else:
+            caches = (("kv_cache", (self.kv_lora_rank,)), ("pe_cache", (rope,)))
+        for name, width in caches:
+            self.register_buffer(name, torch.zeros(args.max_batch_size, args.max_seq_len, *width), persistent=False)
 
     def stack_a(self) -> bool:
         """wq_a over wkv_a in one buffer (scales likewise); returns whether the layers qualify.  Idempotent; the
@@ -310,6 +319,8 @@ class MLA(nn.Module):
         b, s = x.size(0), x.size(1)
         t = start_pos + s
         q, kva = self._project(x)
+        if self.attn_impl == "naive":
+            return self._forward_naive(x, q, kva, start_pos, freqs_cis, mask)
         wkv_b = self._dequantised_wkv_b(x)
         # this step's rows of the two caches
         self.kv_cache[:b, start_pos:t] = self.kv_norm(kva[..., :self.kv_lora_rank])
@@ -325,6 +336,24 @@ class MLA(nn.Module):
         probs = scores.softmax(dim=-1, dtype=torch.float32).type_as(x)
         out = self._absorb(torch.einsum("bsht,btc->bshc", probs, latent), ops._lib.ABSORB_V, wkv_b)
         return self.wo(out.flatten(2))
+
+
+    def _forward_naive(self, x, q, kva, start_pos: int, freqs_cis, mask):
+        """Per-head key / value caches (model.py:470-479, 488-490): the new positions' latents go through wkv_b as a
+        linear layer, keys are [nope part | the shared rotary key], scores and weighted sum are per-head einsums."""
+        b, s = x.size(0), x.size(1)
+        t = start_pos + s
+        nope = self.qk_nope_head_dim
+        q = torch.cat([q[..., :nope], apply_rotary_emb(q[..., nope:], freqs_cis)], dim=-1)
+        rope_key = apply_rotary_emb(kva[..., self.kv_lora_rank:].unsqueeze(2), freqs_cis)
+        kv = self.wkv_b(self.kv_norm(kva[..., :self.kv_lora_rank])).unflatten(-1, (self.n_local_heads, nope + self.v_head_dim))
+        self.k_cache[:b, start_pos:t] = torch.cat([kv[..., :nope], rope_key.expand(-1, -1, self.n_local_heads, -1)], dim=-1)
+        self.v_cache[:b, start_pos:t] = kv[..., nope:]
+        scores = torch.einsum("bshd,bthd->bsht", q, self.k_cache[:b, :t]) * self.softmax_scale
+        if mask is not None:
+            scores = scores + mask.unsqueeze(1)
+        probs = scores.softmax(dim=-1, dtype=torch.float32).type_as(x)
+        return self.wo(torch.einsum("bsht,bthd->bshd", probs, self.v_cache[:b, :t]).flatten(2))
 
 
 class MLP(nn.Module):

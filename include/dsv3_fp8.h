@@ -88,12 +88,16 @@ const char* dsv3_status_string(int status);
  * x: [numel] of x_dtype, y: [numel] bytes, s: [numel / block_size] binary32.
  * `last_dim` is x.size(-1); it must be a multiple of block_size (the reference's
  * assert at inference/kernel.py:52) and numel a multiple of last_dim.
- * block_size in {32, 64, 128, 256, 512}.  x must be 16-byte aligned, y 8-byte, s 4-byte.
+ * Any block_size >= 1 (32, 64, 128, 256 and 512 take the vectorised kernel, every other
+ * size one wavefront per block).  x must be 16-byte aligned, y 8-byte, s 4-byte.
  * numel == 0 is a no-op.  The result is bit-identical to the IEEE evaluation of
- * the formula above.  Non-finite inputs follow that evaluation too (torch's amax and
- * tl.max propagate NaN): a block that holds a NaN gets s = NaN and NaN codes throughout,
- * a block that holds an infinity (and no NaN) gets s = inf, zeros for its finite elements
- * and NaN codes for the infinite ones.
+ * the formula above.  Non-finite inputs follow that evaluation as torch's CPU operators
+ * carry it out (amax propagates NaN), in both scale formats: a block that holds a NaN gets
+ * s = NaN and NaN codes throughout, a block that holds an infinity (and no NaN) gets
+ * s = inf, zeros for its finite elements and NaN codes for the infinite ones.  (Whether
+ * the reference's tl.max propagates or drops a NaN depends on the Triton version; this
+ * behaviour is pinned against the torch evaluation only.)  The quantisers fused into
+ * dsv3_linear_fp8, dsv3_swiglu_quant and dsv3_weight_quant form their scales the same way.
  */
 int dsv3_act_quant(const void* x, int x_dtype, void* y, float* s,
                    int64_t numel, int64_t last_dim, int block_size,

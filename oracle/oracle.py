@@ -37,16 +37,17 @@ BLOCK = 128
 
 
 def ue8m0_round_up(s: torch.Tensor) -> torch.Tensor:
-    """s -> 2^ceil(log2 s) for positive normal binary32 (kernel.py:29-31).
+    """s -> 2^ceil(log2 s) for positive binary32 (kernel.py:29-31).
 
     Defined on the bits so that it does not depend on a libm: a power of two is
-    kept, any other value moves up to the next power of two.
+    kept, any other value moves up to the next power of two.  Infinity and NaN
+    pass through, as they do through exp2(ceil(log2(s))).
     """
     bits = s.contiguous().view(torch.int32)
     exp = bits >> 23
     mant = bits & 0x7FFFFF
     exp = exp + (mant != 0).to(torch.int32)
-    return (exp << 23).view(torch.float32)
+    return torch.where(torch.isfinite(s), (exp << 23).view(torch.float32), s)
 
 
 def act_quant(x: torch.Tensor, block_size: int = BLOCK,
@@ -232,8 +233,11 @@ def _bf16_einsum(eq: str, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 
 def mla(x, start_pos: int, freqs_cis, mask, p: dict, kv_cache, pe_cache, n_heads: int, nope_dim: int,
-        rope_dim: int, v_dim: int, kv_rank: int, softmax_scale: float, scale_fmt=None) -> torch.Tensor:
-    """model.py:456-497, the "absorb" branch with a low-rank query (q_lora_rank > 0), at world_size 1.
+        rope_dim: int, v_dim: int, kv_rank: int, softmax_scale: float, scale_fmt=None,
+        attn_impl: str = "absorb") -> torch.Tensor:
+    """model.py:456-497 with a low-rank query (q_lora_rank > 0), at world_size 1: the "absorb" branch, or the
+    "naive" one (model.py:470-479, 488-490), for which ``kv_cache`` / ``pe_cache`` are the per-head
+    k_cache [b, t, h, nope + rope] / v_cache [b, t, h, v].
     ``p`` maps a layer name to (weight, scale) for the five linears and to the weight for the two norms;
     the caches are updated in place like the reference's buffers.  Every einsum is a bf16 matmul: binary32
     accumulation, one rounding."""
@@ -247,6 +251,18 @@ def mla(x, start_pos: int, freqs_cis, mask, p: dict, kv_cache, pe_cache, n_heads
     q_pe = rotary(q_pe, freqs_cis)
     kv, k_pe = torch.split(lin("wkv_a", x, scale_fmt), [kv_rank, rope_dim], dim=-1)
     k_pe = rotary(k_pe.unsqueeze(2), freqs_cis)
+    if attn_impl == "naive":
+        k_cache, v_cache = kv_cache, pe_cache
+        q = torch.cat([q_nope, q_pe], dim=-1)
+        kv = lin("wkv_b", rms_norm(kv, p["kv_norm"])).view(bsz, seqlen, n_heads, nope_dim + v_dim)
+        k_nope, v = torch.split(kv, [nope_dim, v_dim], dim=-1)
+        k_cache[:bsz, start_pos:end_pos] = torch.cat([k_nope, k_pe.expand(-1, -1, n_heads, -1)], dim=-1)
+        v_cache[:bsz, start_pos:end_pos] = v
+        scores = _bf16_einsum("bshd,bthd->bsht", q, k_cache[:bsz, :end_pos]) * softmax_scale
+        if mask is not None:
+            scores = scores + mask.unsqueeze(1)
+        scores = scores.softmax(dim=-1, dtype=torch.float32).type_as(x)
+        return lin("wo", _bf16_einsum("bsht,bthd->bshd", scores, v_cache[:bsz, :end_pos]).flatten(2))
     q_nope = wkv_b_absorb(q_nope, p["wkv_b"][0], p["wkv_b"][1], "q", nope_dim, v_dim)
     kv_cache[:bsz, start_pos:end_pos] = rms_norm(kv, p["kv_norm"])
     pe_cache[:bsz, start_pos:end_pos] = k_pe.squeeze(2)

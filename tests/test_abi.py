@@ -43,7 +43,9 @@ def test_act_quant_validation(L):
     assert f(A16, L.BF16, A16, A16, 100, 100, 128, 0, None) == 2        # last dim % block (kernel.py:52)
     assert f(A16, L.BF16, A16, A16, -128, 128, 128, 0, None) == 2
     assert f(A16, L.BF16, A16, A16, 384, 256, 128, 0, None) == 2        # numel not a multiple of last dim
-    assert f(A16, L.BF16, A16, A16, 128, 128, 100, 0, None) == 3
+    assert f(A16, L.BF16, A16, A16, 128, 128, 100, 0, None) == 2        # any block size, but it must divide the last dim
+    assert f(A16, L.BF16, A16, A16, 128, 128, 0, 0, None) == 3
+    assert f(A16, L.BF16, A16, A16, 128, 128, -128, 0, None) == 3
     assert f(A16 + 2, L.BF16, A16, A16, 128, 128, 128, 0, None) == 4
     assert f(A16, 9, A16, A16, 128, 128, 128, 0, None) == 5
     assert f(A16, L.BF16, A16, A16, 128, 128, 128, 7, None) == 5
@@ -92,6 +94,21 @@ def test_fp8_gemm_validation(L, entry):
     assert f(A16, A16, A16, A16, A16, L.BF16, 8, 1536, 7168, None, 0, None) == 6
     assert f(A16, A16, A16, A16, A16, L.BF16, 8, 1536, 7168, A16, need - 1, None) == 6
     assert f(A16, A16, A16, A16, A16, L.BF16, 8, 1536, 7168, A16 + 16, need, None) == 6
+
+
+def test_fp8_gemm_static_reports_argument_errors_before_the_size_limit(L):
+    """The entry point that allocates nothing checks its arguments like dsv3_fp8_gemm and only then the size of its
+    scratch array: a malformed call on a large shape reports what is wrong with it, not DSV3_ERR_TOO_LARGE."""
+    f = L.lib.dsv3_fp8_gemm_static
+    big = (9, 129280, 7168)                                               # 84 MiB of partial sums: beyond the array
+    assert L.lib.dsv3_fp8_gemm_workspace_bytes(*big) > L.lib.dsv3_fp8_gemm_static_max_bytes()
+    assert f(A16, A16, A16, A16, A16, L.BF16, *big, None) == 8            # well-formed: refused for its size
+    assert f(A16, A16, A16, A16, A16, 3, *big, None) == 5                 # bad dtype code
+    assert f(None, A16, A16, A16, A16, L.BF16, *big, None) == 1
+    assert f(A16 + 8, A16, A16, A16, A16, L.BF16, *big, None) == 4
+    assert f(A16, A16, A16, A16, A16, L.BF16, 9, 129280, 7168 + 64, None) == 2   # K % 128
+    assert f(A16, A16, A16, A16, A16, L.BF16, -9, 129280, 7168, None) == 2
+    assert f(None, None, None, None, None, L.BF16, 0, 129280, 7168, None) == 0   # nothing to do
 
 
 def test_ops_shape_inference_and_no_cpu_fallback():

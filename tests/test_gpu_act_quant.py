@@ -92,6 +92,20 @@ def test_other_block_sizes(K, block):
     _check(K, x, block)
 
 
+@pytest.mark.parametrize("block", [1, 2, 8, 16, 24, 100, 1024, 2048, 4096])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_any_block_size_that_divides_the_last_dimension(K, block, dtype):
+    """The reference's wrapper takes every block size that divides the last dimension (inference/kernel.py:38,52);
+    sizes other than 32 ... 512 run one wavefront per block."""
+    torch.manual_seed(block)
+    cols = block * (3 if block >= 1024 else 5)
+    x = (torch.randn(9, cols) * torch.rand(9, 1) * 10).to(dtype)
+    x[0, :block] = 0
+    x[1, 0] = 3e4
+    _check(K, x, block)
+    _check(K, x, block, "ue8m0")
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_other_input_dtypes(K, dtype):
     torch.manual_seed(11)
@@ -133,11 +147,7 @@ def test_full_size_properties(K):
     assert bool((mag.amax(-1) == 0x7E).all())
 
 
-def test_non_finite_inputs_follow_the_ieee_evaluation(K):
-    """NaN and infinity in the activations (inference/kernel.py:26-33 with tl.max / torch.amax, which propagate NaN):
-    a block with a NaN gets s = NaN and NaN codes everywhere, a block with an infinity s = inf, zeros for the finite
-    elements and NaN codes for the infinite ones; blocks beside them are untouched.  Held against oracle.act_quant
-    (NaN codes are compared as "is a NaN code": 0x7f and 0xff differ only in the sign of the NaN)."""
+def _non_finite_rows():
     g = torch.Generator().manual_seed(12)
     x = torch.randn(6, 512, generator=g).bfloat16()
     x[0, 5] = float("nan")                      # block (0, 0)
@@ -145,6 +155,43 @@ def test_non_finite_inputs_follow_the_ieee_evaluation(K):
     x[2, 300] = float("-inf"); x[2, 301] = 7.0  # block (2, 2)
     x[3, 10] = float("nan"); x[3, 11] = float("inf")   # NaN wins over infinity
     x[4, 384:512] = 0                           # an all-zero block beside normal ones
+    return x
+
+
+def _same_up_to_nan_sign(y, s, yr, sr):
+    """Scales: NaN where the oracle has NaN, inf where it has inf, equal elsewhere; bytes: NaN codes where the oracle
+    has NaN codes (0x7f and 0xff differ only in the sign of the NaN), equal elsewhere.  Returns the NaN-code mask."""
+    y, yr = y.cpu().view(torch.uint8), yr.view(torch.uint8)
+    s = s.cpu()
+    assert torch.equal(torch.isnan(s), torch.isnan(sr)) and torch.equal(torch.isinf(s), torch.isinf(sr))
+    ok = torch.isfinite(sr)
+    assert torch.equal(s[ok], sr[ok])
+    nan_ref, nan_got = (yr & 0x7F) == 0x7F, (y & 0x7F) == 0x7F
+    assert torch.equal(nan_ref, nan_got)
+    assert torch.equal(y[~nan_ref], yr[~nan_ref])
+    return nan_got
+
+
+@pytest.mark.parametrize("fmt", [None, "ue8m0"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("block", [128, 16])
+def test_non_finite_inputs_every_variant(K, fmt, dtype, block):
+    """Both scale formats (the power-of-two rounding must leave s = NaN / inf alone), the reciprocal and the IEEE
+    division paths, the vectorised and the one-wavefront-per-block kernels."""
+    x = _non_finite_rows().to(dtype)
+    yr, sr = oracle.act_quant(x, block, fmt)
+    y, s = K.act_quant(x.cuda(), block, fmt)
+    nan_got = _same_up_to_nan_sign(y, s, yr, sr)
+    assert bool(torch.isnan(s[0, 0])) and bool(nan_got[0, :block].all())
+    assert bool(torch.isinf(s[1, 130 // block])) and s[1, 130 // block] > 0
+
+
+def test_non_finite_inputs_follow_the_ieee_evaluation(K):
+    """NaN and infinity in the activations (inference/kernel.py:26-33 evaluated with torch's CPU operators, whose amax
+    propagates NaN): a block with a NaN gets s = NaN and NaN codes everywhere, a block with an infinity s = inf, zeros
+    for the finite elements and NaN codes for the infinite ones; blocks beside them are untouched.  Held against
+    oracle.act_quant (NaN codes are compared as "is a NaN code": 0x7f and 0xff differ only in the sign of the NaN)."""
+    x = _non_finite_rows()
     yr, sr = oracle.act_quant(x)
     y, s = K.act_quant(x.cuda())
     y, s = y.cpu().view(torch.uint8), s.cpu()

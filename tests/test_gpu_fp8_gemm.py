@@ -46,7 +46,8 @@ def _check(K, x, w8, ws, fmt=None):
     return err / rms
 
 
-DECODE = [(7168, 1536), (1536, 24576), (7168, 576), (512, 32768), (16384, 7168)]
+# the five attention projections (inference/model.py:427-433) and wq_a | wkv_a stacked into one 7168 -> 2112 weight
+DECODE = [(7168, 1536), (1536, 24576), (7168, 576), (512, 32768), (16384, 7168), (7168, 2112)]
 
 
 @pytest.mark.parametrize("kn", DECODE)
@@ -471,3 +472,25 @@ def test_seeded_shape_sweep(K):
         w8, ws = workloads.weight(n, k, seed=200 + i)
         worst = max(worst, _check(K, x, w8, ws))
     assert worst <= TOL
+
+
+@pytest.mark.parametrize("fmt", [None, "ue8m0"])
+def test_fused_linear_non_finite_activations(K, fmt):
+    """The quantiser inside dsv3_linear_fp8 forms its scales as act_quant does (a NaN or an infinity in a block reaches
+    the scale): rows that hold one come out as NaN in the one call and in the two calls alike, the other rows bit-equal."""
+    from dsv3fp8 import workloads, ops, _lib
+    code_fmt = _lib.SCALE_FMT_UE8M0 if fmt == "ue8m0" else _lib.SCALE_FMT_NONE
+    k, n = 7168, 576
+    x = workloads.activations(4, k, seed=9)
+    x[0, 100] = float("nan")
+    x[1, 3000] = float("inf")
+    x[2, 7000] = float("-inf"); x[2, 5] = float("nan")
+    assert ops.linear_fp8_fused(4, n, k)
+    w8, ws = workloads.weight(n, k, seed=3)
+    xc, w8, ws = x.cuda(), w8.cuda(), ws.cuda()
+    a, a_s = K.act_quant(xc, 128, fmt)
+    two = torch.ops.dsv3fp8.fp8_gemm(a, a_s, w8, ws, _lib.F32)
+    one = torch.ops.dsv3fp8.linear_fp8(xc, w8, ws, code_fmt, _lib.F32)
+    assert bool(torch.isnan(two[:3]).all()) and bool(torch.isfinite(two[3]).all())
+    assert torch.equal(torch.isnan(one), torch.isnan(two))
+    assert torch.equal(one[3], two[3])

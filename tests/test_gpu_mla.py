@@ -236,3 +236,41 @@ def test_mla_prefill_then_decode_vs_oracle(M):
         z1 = layer(x1.cuda(), 7, freqs[7:8].cuda(), None)
         _close(y0, z0.cpu(), 2e-2)
         _close(y1, z1.cpu(), 2e-2)
+
+
+def test_mla_naive_cache_layout_vs_oracle(M):
+    """attn_impl = "naive" (model.py:443-445, 470-479, 488-490): per-head key / value caches, wkv_b as an FP8 linear
+    layer.  Prefill then one decode step against oracle.mla(..., attn_impl="naive"), and against the absorbed layout."""
+    dim, heads, q_rank, kv_rank, nope, rope, v = 256, 4, 128, 128, 64, 32, 64
+    p = small_mla_params(dim, heads, q_rank, kv_rank, nope, rope, v, 22)
+    absorbed = _build(M, p, dim, heads, q_rank, kv_rank, nope, rope, v)
+    M.attn_impl = "naive"
+    layer = _build(M, p, dim, heads, q_rank, kv_rank, nope, rope, v)
+    M.attn_impl = "absorb"
+    assert layer.k_cache.shape == (2, 16, heads, nope + rope) and layer.v_cache.shape == (2, 16, heads, v)
+    assert not hasattr(layer, "kv_cache")
+    freqs = _freqs(rope, 16)
+    g = torch.Generator().manual_seed(23)
+    x0 = torch.randn(2, 7, dim, generator=g).bfloat16()
+    x1 = torch.randn(2, 1, dim, generator=g).bfloat16()
+    mask = torch.full((7, 7), float("-inf")).triu_(1)
+    k_c = torch.zeros(2, 16, heads, nope + rope, dtype=torch.bfloat16)
+    v_c = torch.zeros(2, 16, heads, v, dtype=torch.bfloat16)
+    scale = (nope + rope) ** -0.5
+    ref0 = oracle.mla(x0, 0, freqs[:7], mask, p, k_c, v_c, heads, nope, rope, v, kv_rank, scale, attn_impl="naive")
+    ref1 = oracle.mla(x1, 7, freqs[7:8], None, p, k_c, v_c, heads, nope, rope, v, kv_rank, scale, attn_impl="naive")
+    with torch.inference_mode():
+        y0 = layer(x0.cuda(), 0, freqs[:7].cuda(), mask.cuda())
+        y1 = layer(x1.cuda(), 7, freqs[7:8].cuda(), None)
+        _close(y0, ref0, 2e-2)
+        _close(y1, ref1, 2e-2)
+        _close(layer.k_cache, k_c, 2e-2)
+        _close(layer.v_cache, v_c, 2e-2)
+        a0 = absorbed(x0.cuda(), 0, freqs[:7].cuda(), mask.cuda())
+        a1 = absorbed(x1.cuda(), 7, freqs[7:8].cuda(), None)
+        for yn, ya in ((y0, a0), (y1, a1)):     # the two layouts differ by one FP8 quantisation of the latent
+            rel = (yn.float() - ya.float()).pow(2).mean().sqrt() / ya.float().pow(2).mean().sqrt()
+            assert rel.item() < 0.08, rel.item()
+    with pytest.raises(ValueError):
+        M.attn_impl = "other"
+        M.MLA(M.ModelArgs(dim=dim, n_heads=heads, q_lora_rank=q_rank, kv_lora_rank=kv_rank))

@@ -193,6 +193,29 @@ def test_swiglu_quant_every_bf16_value(K):
     assert torch.equal(s[finite], sd[finite]) and torch.equal(y.view(torch.uint8)[finite], yd.view(torch.uint8)[finite])
 
 
+@pytest.mark.parametrize("fmt", [None, "ue8m0"])
+def test_swiglu_quant_non_finite(K, fmt):
+    """A NaN or an infinity in silu(h1) * h3 reaches the block's scale as it does through act_quant."""
+    from dsv3fp8 import _lib
+    g = torch.Generator().manual_seed(8)
+    h = torch.randn(5, 512, generator=g).bfloat16()
+    h[0, 3] = float("nan")                      # h1 of block (0, 0)
+    h[1, 256 + 130] = float("inf")              # h3 of block (1, 1)
+    h[2, 200] = float("inf")                    # silu(inf) = inf, block (2, 1)
+    h[3, 7] = float("-inf")                     # silu(-inf) = -0 / NaN as F.silu gives it
+    hc = h.cuda()
+    y, s = torch.ops.dsv3fp8.swiglu_quant(hc, 128, _lib.SCALE_FMT_UE8M0 if fmt else _lib.SCALE_FMT_NONE)
+    gd = (F.silu(hc[:, :256]) * hc[:, 256:]).contiguous()
+    yd, sd = K.act_quant(gd, 128, fmt)
+    assert bool(torch.isnan(sd[0, 0])) and bool(torch.isinf(sd[1, 1]))
+    assert torch.equal(torch.isnan(s), torch.isnan(sd)) and torch.equal(torch.isinf(s), torch.isinf(sd))
+    ok = torch.isfinite(sd)
+    assert torch.equal(s[ok], sd[ok])
+    yb, ydb = y.view(torch.uint8), yd.view(torch.uint8)
+    nan_a, nan_b = (yb & 0x7F) == 0x7F, (ydb & 0x7F) == 0x7F
+    assert torch.equal(nan_a, nan_b) and torch.equal(yb[~nan_a], ydb[~nan_a])
+
+
 @pytest.mark.parametrize("with_shared", [True, False])
 def test_moe_combine_bit_exact(K, with_shared):
     g = torch.Generator().manual_seed(4)
@@ -485,17 +508,54 @@ def test_moe_layer_full_configuration(K):
         assert torch.equal(y_perm.view(torch.int16), y[perm].view(torch.int16))
         counts = torch.bincount(idx.flatten(), minlength=args.n_routed_experts)
         assert int(counts.sum()) == tokens * 8 and int((counts > 0).sum()) > 200
-        sample = torch.tensor([0, 1777, 4095])
+        # sampled tokens, chosen greedily so that together they select many different experts: every new token adds
+        # as many experts not seen so far as possible
+        idx_cpu = idx.cpu()
+        sample, hit = [0, 1777, 4095], set(idx_cpu[[0, 1777, 4095]].flatten().tolist())
+        cand = torch.randperm(tokens, generator=torch.Generator().manual_seed(7))[:600].tolist()
+        while len(sample) < 24:
+            best = max(cand, key=lambda t: len(set(idx_cpu[t].tolist()) - hit))
+            cand.remove(best)
+            sample.append(best)
+            hit |= set(idx_cpu[best].tolist())
+        assert len(hit) >= 64, len(hit)
+        sample = torch.tensor(sample)
 
         def cpu(ex):
             return tuple(t.data.cpu() for lin in (ex.w1, ex.w2, ex.w3) for t in (lin.weight, lin.scale))
-        hit = set(idx[sample.cuda()].flatten().tolist())
         experts = [cpu(ex) if e in hit else None for e, ex in enumerate(moe.experts)]
-        ref = oracle.moe(x[sample.cuda()].cpu(), wts[sample.cuda()].cpu(), idx[sample.cuda()].cpu(), experts,
+        ref = oracle.moe(x[sample.cuda()].cpu(), wts[sample.cuda()].cpu(), idx_cpu[sample], experts,
                          cpu(moe.shared_experts))
         rms = ref.float().pow(2).mean().sqrt().item()
         err = (y[sample.cuda()].float().cpu() - ref.float()).abs().max().item()
         assert err <= 5e-2 * rms + 2 ** -8 * ref.abs().max().item(), (err, rms)
+
+        # the first grouped GEMM by itself, expert by expert: the rows of a sampled expert against the oracle's
+        # fp8_gemm with THAT expert's w1 | w3 (and scales), on the expert's own token list
+        from dsv3fp8 import ops
+        with torch.inference_mode():
+            route = torch.ops.dsv3fp8.moe_route(idx.contiguous(), wts.contiguous(), args.n_routed_experts, False)
+            _, a_rows, rows, _, tile_group, tile_row0, tile_rows = route
+            xq, xs = K.act_quant(x)
+            w13, s13 = (t[:args.n_routed_experts] for t in moe._stacked[:2])
+            h = torch.ops.dsv3fp8.fp8_gemm_grouped(xq, xs, a_rows, w13, s13, rows.numel(), tile_group, tile_row0,
+                                                   tile_rows, ops.dtype_code(torch.float32))
+        starts = torch.cumsum(counts, 0) - counts
+        inter = args.moe_inter_dim
+        checked = 0
+        for e in sorted(hit)[::3]:                               # every third of the sampled experts (>= 21 of them)
+            c, r0 = int(counts[e]), int(starts[e])
+            pick = torch.unique(torch.tensor([0, c // 2, c - 1])) + r0
+            toks = a_rows[pick.cuda()].long()
+            assert bool((idx[toks] == e).any(dim=1).all())       # the list holds tokens that selected expert e
+            w1, s1, _, _, w3, s3 = experts[e]
+            for half, (w8, sc) in enumerate(((w1, s1), (w3, s3))):
+                ref_h = oracle.fp8_gemm_f32(xq[toks].cpu(), xs[toks].cpu(), w8[:256], sc[:2])
+                got_h = h[pick.cuda()][:, half * inter: half * inter + 256].cpu()
+                err_h = (got_h - ref_h).abs().max().item()
+                assert err_h <= 1e-2 * ref_h.pow(2).mean().sqrt().item(), (e, half, err_h)
+            checked += 1
+        assert checked >= 21
     finally:
         M.gemm_impl, M.Linear.dtype = old[0], old[2]
         torch.set_default_dtype(old[1])

@@ -152,3 +152,24 @@ def test_quantise_then_multiply_with_power_of_two_scales(K):
     ra, ras = oracle.act_quant(x, 128, "ue8m0")
     ref = oracle.fp8_gemm_f32(ra, ras, r8, rs)
     assert (c.cpu() - ref).abs().max().item() <= 1e-2 * ref.pow(2).mean().sqrt().item()
+
+
+@pytest.mark.parametrize("fmt", [None, "ue8m0"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_non_finite_weights(K, fmt, dtype):
+    """A NaN or an infinity in a 128 x 128 block reaches that block's scale (NaN / inf) as through act_quant; the other
+    blocks are untouched.  Against the oracle: scales NaN / inf in the same places, bytes NaN codes in the same places."""
+    g = torch.Generator().manual_seed(21)
+    w = (torch.randn(256, 384, generator=g) * 0.02).to(dtype)
+    w[3, 5] = float("nan")               # block (0, 0)
+    w[130, 200] = float("inf")           # block (1, 1)
+    w[200, 300] = float("-inf"); w[201, 301] = float("nan")     # block (1, 2): NaN wins
+    ref8, refs = oracle.block_quant_weight(w, scale_fmt=fmt)
+    q8, qs = K.weight_quant(w.cuda(), scale_fmt=fmt)
+    qs, q8, ref8 = qs.cpu(), q8.cpu().view(torch.uint8), ref8.view(torch.uint8)
+    assert bool(torch.isnan(refs[0, 0])) and bool(torch.isinf(refs[1, 1])) and bool(torch.isnan(refs[1, 2]))
+    assert torch.equal(torch.isnan(qs), torch.isnan(refs)) and torch.equal(torch.isinf(qs), torch.isinf(refs))
+    ok = torch.isfinite(refs)
+    assert torch.equal(qs[ok], refs[ok])
+    nan_a, nan_b = (q8 & 0x7F) == 0x7F, (ref8 & 0x7F) == 0x7F
+    assert torch.equal(nan_a, nan_b) and torch.equal(q8[~nan_a], ref8[~nan_a])

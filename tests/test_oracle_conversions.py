@@ -115,3 +115,9 @@ def test_ue8m0_round_up(coracle):
     up = oracle.ue8m0_round_up(s)
     assert bool((up >= s).all()) and bool((up < 2 * s).all())
     assert bool(((up.view(torch.int32) & 0x7FFFFF) == 0).all())
+    # non-finite scales (a block that holds an infinity or a NaN): exp2(ceil(log2(s))) returns them unchanged
+    odd = torch.tensor([float("inf"), float("nan")])
+    want = torch.exp2(torch.ceil(torch.log2(odd)))
+    got = oracle.ue8m0_round_up(odd)
+    assert bool(torch.isinf(got[0])) and got[0] > 0 and bool(torch.isnan(got[1]))
+    assert torch.equal(torch.isnan(got), torch.isnan(want)) and torch.equal(torch.isinf(got), torch.isinf(want))

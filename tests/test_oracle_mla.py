@@ -127,6 +127,17 @@ def test_mla_absorbed_equals_textbook_attention():
     # the caches hold the normalised latent and the rotated shared key of the positions just written
     assert (kv_cache[:, :seqlen].double() - lat).abs().max() < 0.1 and kv_cache[:, seqlen:].abs().max() == 0
     assert (pe_cache[:, :seqlen].double() - k_pe.squeeze(2)).abs().max() < 0.1
+    # the "naive" branch (per-head key / value caches, model.py:470-479, 488-490) against the same textbook result,
+    # its caches against the explicit keys and values, and against the absorbed branch
+    k_cache = torch.zeros(bsz, 16, heads, nope + rope, dtype=torch.bfloat16)
+    v_cache = torch.zeros(bsz, 16, heads, v, dtype=torch.bfloat16)
+    naive = oracle.mla(x, 0, freqs, mask, p, k_cache, v_cache, heads, nope, rope, v, kv_rank, scale,
+                       attn_impl="naive").double()
+    err_n = (naive - ref).pow(2).mean().sqrt() / ref.pow(2).mean().sqrt()
+    assert err_n < 0.08, err_n                   # (one more FP8 activation quantisation: the latent in front of wkv_b)
+    assert (naive - got).pow(2).mean().sqrt() / ref.pow(2).mean().sqrt() < 0.08
+    assert (k_cache[:, :seqlen].double() - k).abs().max() < 0.3 and k_cache[:, seqlen:].abs().max() == 0
+    assert (v_cache[:, :seqlen].double() - kvh[..., nope:]).abs().max() < 0.3 and v_cache[:, seqlen:].abs().max() == 0
 
 
 def test_rotary_table_equals_the_reference_expressions_bit_for_bit():
