@@ -312,6 +312,28 @@ def run_extras(K, W, probes, ceil):
     return out
 
 
+def decode_trace(K, W, launches_per_cell: int = 60):
+    """For `rocprofv3 --kernel-trace`: every cell of the decode sweep as plain launches (no graph) over rotating
+    weight copies, cell after cell in a fixed order, with a device synchronisation between cells.  Prints one JSON
+    line naming the cells in launch order and the launches per cell, so that the kernel rows of the trace (sorted by
+    start time) can be cut into cells: a launch is one GEMM kernel, followed by the kernel that adds its K slices
+    when the plan has any."""
+    order = []
+    for name, (k, n) in W.DECODE_SWEEP.items():
+        wq, wsc = W.weight(n, k, 1, "cuda")
+        copies = max(2, min(160, -(-640_000_000 // (n * k))))
+        wqs = [wq.clone() for _ in range(copies)]
+        for m in W.DECODE_M:
+            a, a_s = K.act_quant(W.activations(m, k, m, "cuda"))
+            torch.cuda.synchronize()
+            for i in range(launches_per_cell):
+                K.fp8_gemm(a, a_s, wqs[i % copies], wsc)
+            torch.cuda.synchronize()
+            order.append({"cell": f"{name}_{k}to{n}_M{m}", "bytes": decode_bytes(m, n, k)})
+        del wqs
+    print(json.dumps({"decode_trace": {"launches_per_cell": launches_per_cell, "cells": order}}), flush=True)
+
+
 def decode_roofline(dec: dict, ceil: dict) -> dict:
     """The metric's second half in one block: the decode sweep (M = 1, 8, 32, 64 over the MLA projections) as HBM
     fractions of its algorithmic bytes, against the 8 TB/s peak and against this GPU's measured read stream."""
@@ -563,6 +585,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only-absorb", type=int, default=0, metavar="TOKENS",
                     help="profiling aid: run only the wkv_b_absorb leg at this token count and print its JSON")
+    ap.add_argument("--decode-trace", action="store_true",
+                    help="profiling aid: run only the decode sweep as plain launches (see decode_trace) and print "
+                         "the cell order")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known HBM traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled")
@@ -577,6 +602,9 @@ def main():
     from dsv3fp8 import workloads as W
     torch.set_default_dtype(torch.bfloat16)  # as the reference's caller does (generate.py:109)
     torch.cuda.set_device(0)
+    if args.decode_trace:
+        decode_trace(K, W)
+        return
     if args.only_absorb:
         if args.copy_calibration:
             src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")

@@ -283,41 +283,42 @@ Plan make_plan(int64_t m, int64_t n, int64_t k) {
     return p;
 }
 
-// 3 to 16 rows on a weight of 96 MiB or more: the dense GEMM runs as one group of the grouped weight-streaming
-// kernel -- 32-row strips of such a weight fill the chip, one launch, no partial sums in memory (16384 -> 7168 at 4
-// rows 25.5 against 30.4 us; 7168 -> 36864 at 8 rows 51 against 70 us).  One and two rows stay with the M <= 16
-// kernel, which quantises bf16 activations itself for linear() there (26.5 us fused against 25.5 + 3.5 us).
+// 3 to 16 rows on a weight of 96 MiB or more with 8192 rows or more: the dense GEMM runs as one group of the grouped
+// weight-streaming kernel -- 32-row strips of such a weight fill the chip, one launch, no partial sums in memory
+// (7168 -> 36864 at 8 rows 51 against 70 us).  One and two rows stay with the M <= 16 kernel, which quantises bf16
+// activations itself for linear() there.
 bool single_group_stream(int64_t m, int64_t n, int64_t k) {
     if (m < 3 || m > 16 || n * k < (96ll << 20) || !skinny_single_supported(m, n, k)) return false;
-    // from 8 rows up the activation-streaming kernel is flat where this one grows with the rows (16384 -> 7168 at
-    // 8 / 12 / 16 rows: 26.2 / 26.3 / 26.5 against 26.7 / 28.3 / 29.6 us; at 3 / 4 rows 26.3 against 25.3 / 25.6)
-    return !(m >= 8 && n < 8192 && stream_supported(m, n, k));
+    // weights of fewer than 8192 rows: the activation-streaming kernel with two workgroups per compute unit
+    // (16384 -> 7168 at 4 / 8 / 16 rows: 22.4 / 22.7 / 23.8 against 25.6 / 26.7 / 29.6 us)
+    return !(n < 8192 && stream_supported(m, n, k));
 }
 
-// DSV3_GEMM_FORCE=tile|prefill pins the large-M kernel choice (tuning / debugging aid).
+// DSV3_GEMM_FORCE=tile|prefill|stream|skinny pins the kernel choice where the named kernel supports the shape (tuning /
+// debugging aid).
 int forced_kernel() {
     static const int v = [] {
         const char* e = std::getenv("DSV3_GEMM_FORCE");
         if (!e) return 0;
         if (!std::strcmp(e, "tile")) return 1;
         if (!std::strcmp(e, "prefill")) return 2;
+        if (!std::strcmp(e, "stream")) return 3;
+        if (!std::strcmp(e, "skinny")) return 4;
         return 0;
     }();
     return v;
 }
 
 // Which problems go to the large-M kernel (K range cut into slices when the tiles do not fill the chip): every M
-// above 64, and M = 9 .. 64 when the weight is large (>= 96 MiB).  There it runs at a flat 32-34 us per 117-132 MB
-// from 9 to 64 rows, while the M <= 16 streaming kernel grows with M (its K splits multiply with the rows it has
-// to stage: 31 us at 8 rows, 42-50 us at 16).  Exception: up to 32 rows on a large weight of fewer than 8192 rows go
-// to the activation-streaming kernel in its four-consumer form, two K slices (16384 -> 7168 at 17 / 32 rows 27.3 /
-// 29.1 against 33.3 / 31.6 us, 18432 -> 7168 28.6 / 29.2 against 36.4 / 32.7; at 48-64 rows and on wider weights the
-// large-M kernel is equal or faster).  For the smaller decode weights the streaming and tile kernels are faster.
+// above 64, and M = 9 .. 64 when the weight is large (>= 96 MiB) and has 8192 rows or more.  There it runs at a flat
+// 32-34 us per 117-132 MB from 9 to 64 rows.  Large weights of fewer rows go to the activation-streaming kernel
+// (16384 -> 7168 at 16 / 32 / 64 rows 23.8 / 27.3 / 32.7 against 33 / 31.6 / 34.6 us); for the smaller decode weights
+// the streaming and tile kernels are faster anyway.
 bool to_large_m_kernel(int64_t m, int64_t n, int64_t k) {
     if (!prefill_supported(m, n, k)) return false;
     if (m > 64) return true;
     if (m <= 8 || n * k < (96ll << 20)) return false;
-    return !(m <= 32 && n < 8192 && stream_supported(m, n, k));
+    return !(n < 8192 && stream_supported(m, n, k));
 }
 
 template <int CD>
@@ -332,8 +333,8 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
     const int force = forced_kernel();
     if (force == 0 && single_group_stream(m, n, k))
         return launch_skinny_single(a, a_s, b, b_s, c, CD, m, n, k, st);
-    const bool to_prefill = force != 1 && to_large_m_kernel(m, n, k);
-    const bool use_stream = force != 1 && !to_prefill && stream_supported(m, n, k);
+    const bool to_prefill = force != 1 && !(force == 3 && stream_supported(m, n, k)) && to_large_m_kernel(m, n, k);
+    const bool use_stream = force != 1 && !to_prefill && !(force == 4 && skinny_supported(m, n, k)) && stream_supported(m, n, k);
     if (use_stream || (force != 1 && !to_prefill && skinny_supported(m, n, k))) {          // decode shapes: weight-streaming kernels
         int splits = 1;
         const int rc = use_stream ? launch_stream(a, a_s, b, b_s, c, CD, m, n, k, ws, &splits, st)
@@ -372,7 +373,8 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
 // fused, so that the one call and the two calls always give the same bits.
 bool linear_fp8_supported(int64_t m, int64_t n, int64_t k) {
     return forced_kernel() != 1 && k % 128 == 0 && skinny_supported(m, n, k) && !to_large_m_kernel(m, n, k) &&
-           !(forced_kernel() == 0 && single_group_stream(m, n, k)) && !stream_supported(m, n, k) && m * k <= 131072;
+           !(forced_kernel() == 0 && single_group_stream(m, n, k)) && (m <= 2 || !stream_supported(m, n, k)) &&
+           m * k <= 131072;
 }
 
 int launch_linear_fp8(const void* x, const void* b, const float* b_s, void* c, int c_dtype, int64_t m, int64_t n,

@@ -247,7 +247,10 @@ def test_gate_route_validation(L):
 def test_linear_fp8_validation(L):
     f, fused = L.lib.dsv3_linear_fp8, L.lib.dsv3_linear_fp8_fused
     assert fused(1, 1536, 7168) and fused(2, 7168, 16384) and not fused(16, 7168, 16384) and not fused(17, 1536, 7168)
-    assert fused(8, 24576, 1536) and not fused(8, 7168, 16384)   # 3+ rows on a weight of 96 MiB or more: two calls
+    # 3+ rows: two calls wherever fp8_gemm takes the activation-streaming kernel (K of 512 and more); one and two rows
+    # are always one call
+    assert fused(8, 4096, 256) and not fused(8, 24576, 1536) and not fused(8, 7168, 16384)
+    assert fused(1, 24576, 1536) and fused(2, 576, 7168) and fused(1, 32768, 512)
     assert not fused(4096, 1536, 7168)
     assert not fused(4, 1536, 7000) and not fused(0, 8, 128)
     #     x    dtype   b    b_s  c    cdtype  m  n     k     block fmt ws    ws_bytes stream

@@ -339,20 +339,19 @@ def test_asserts_match_reference(K):
 @pytest.mark.parametrize("m", [1, 3, 8, 16])
 def test_fused_linear_equals_act_quant_then_gemm(K, m, fmt):
     """dsv3_linear_fp8 (activation quantisation inside the M <= 16 weight-streaming kernel) against the two separate
-    calls, bit for bit, on every decode shape; and the two-step result against the oracle as everywhere else."""
+    calls on every decode shape: bit for bit wherever fp8_gemm runs the same kernel -- from three rows up the one call
+    is only offered there --, and up to the order of the binary32 sums at one and two rows where fp8_gemm streams the
+    activations through LDS instead (the quantised bytes and scales are the same; both sides meet the oracle's bar)."""
     from dsv3fp8 import workloads, ops, _lib
     code_fmt = _lib.SCALE_FMT_UE8M0 if fmt == "ue8m0" else _lib.SCALE_FMT_NONE
     for name, (k, n) in workloads.DECODE_SHAPES.items():
-        # fused up to 131072 activation elements where fp8_gemm takes its M <= 16 kernel: always at one and two rows,
-        # never at 3+ rows on weights of 96 MiB and more (their single-launch kernel has no quantising variant), and
-        # at 3+ rows on the other weights unless fp8_gemm streams the activations through LDS (long K, 16+ groups)
+        # one call up to 131072 activation elements: always at one and two rows; from three rows up only where
+        # fp8_gemm takes its M <= 16 kernel (never on weights of 96 MiB and more, nor where it streams the activations)
         fused = ops.linear_fp8_fused(m, n, k)
         if m <= 2:
             assert fused == (m * k <= 131072), name
         else:
             assert not (fused and (m * k > 131072 or n * k >= 96 << 20)), name
-            if name == "wkv_a":
-                assert fused, name                          # 7168 -> 576 (9 groups of 64 rows): the M <= 16 kernel
         x = workloads.activations(m, k, seed=m + n % 7, outliers=True).cuda()
         w8, ws = workloads.weight(n, k, seed=3)
         w8, ws = w8.cuda(), ws.cuda()
@@ -360,7 +359,20 @@ def test_fused_linear_equals_act_quant_then_gemm(K, m, fmt):
         for code in (_lib.BF16, _lib.F32):
             two = torch.ops.dsv3fp8.fp8_gemm(a, a_s, w8, ws, code)
             one = torch.ops.dsv3fp8.linear_fp8(x, w8, ws, code_fmt, code)
-            assert one.dtype == two.dtype and torch.equal(one, two), (name, code)
+            assert one.dtype == two.dtype
+            if torch.equal(one, two):
+                continue
+            assert m <= 2, (name, code)                     # (another kernel behind fp8_gemm: sums in another order)
+            rms = two.float().pow(2).mean().sqrt().item()
+            tol = 1e-3 * rms if code == _lib.F32 else 2.0 ** -7 * two.float().abs().max().item()
+            assert (one.float() - two.float()).abs().max().item() <= tol, (name, code)
+    # three rows and more where fp8_gemm itself takes the M <= 16 kernel (K below 512): one call, the same bits
+    x = workloads.activations(8, 256, seed=4).cuda()
+    w8, ws = workloads.weight(4096, 256, seed=5)
+    a, a_s = K.act_quant(x, 128, fmt)
+    assert ops.linear_fp8_fused(8, 4096, 256)
+    assert torch.equal(torch.ops.dsv3fp8.linear_fp8(x, w8.cuda(), ws.cuda(), code_fmt, _lib.F32),
+                       torch.ops.dsv3fp8.fp8_gemm(a, a_s, w8.cuda(), ws.cuda(), _lib.F32))
     # rows above the fused kernel's range take the two calls inside the op
     x = workloads.activations(40, 512, seed=1).cuda()
     w8, ws = workloads.weight(256, 512, seed=2)
@@ -480,11 +492,11 @@ def test_fused_linear_non_finite_activations(K, fmt):
     the scale): rows that hold one come out as NaN in the one call and in the two calls alike, the other rows bit-equal."""
     from dsv3fp8 import workloads, ops, _lib
     code_fmt = _lib.SCALE_FMT_UE8M0 if fmt == "ue8m0" else _lib.SCALE_FMT_NONE
-    k, n = 7168, 576
+    k, n = 384, 576                             # (four rows run as one call where K is below 512)
     x = workloads.activations(4, k, seed=9)
     x[0, 100] = float("nan")
-    x[1, 3000] = float("inf")
-    x[2, 7000] = float("-inf"); x[2, 5] = float("nan")
+    x[1, 300] = float("inf")
+    x[2, 383] = float("-inf"); x[2, 5] = float("nan")
     assert ops.linear_fp8_fused(4, n, k)
     w8, ws = workloads.weight(n, k, seed=3)
     xc, w8, ws = x.cuda(), w8.cuda(), ws.cuda()
