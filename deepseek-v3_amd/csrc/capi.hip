@@ -252,6 +252,31 @@ int dsv3_fp8_gemm_grouped_pow2(const void* a, const float* a_s, const int32_t* a
                                     m, n, k, tile_group, tile_row0, tile_rows, num_tiles, stream, true);
 }
 
+int dsv3_fp8_gemm_grouped_swiglu_fused(int64_t m, int64_t a_num_rows, int64_t inter, int64_t k) {
+    return m > 0 && a_num_rows >= 0 && inter > 0 && k > 0 && k % 128 == 0 && m <= 0x7fffffff && 2 * inter <= 0x7fffffff &&
+           k <= 0x7fffffff && grouped_swiglu_supported(m, a_num_rows, inter, k);
+}
+
+int dsv3_fp8_gemm_grouped_swiglu(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
+                                 const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
+                                 void* y, float* s, int64_t m, int64_t inter, int64_t k,
+                                 const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
+                                 int64_t num_tiles, int block_size, int scale_fmt, void* stream) {
+    if (scale_fmt != DSV3_SCALE_FMT_NONE && scale_fmt != DSV3_SCALE_FMT_UE8M0) return DSV3_ERR_BAD_DTYPE;
+    if (block_size != 128) return DSV3_ERR_BAD_BLOCK;
+    if (m < 0 || inter < 0 || k < 0 || a_num_rows < 0 || num_tiles < 0 || b_group_stride < 0 || bs_group_stride < 0)
+        return DSV3_ERR_BAD_SHAPE;
+    if (k % 128 != 0 || k == 0 || inter % 128 != 0) return DSV3_ERR_BAD_SHAPE;
+    if (m == 0 || inter == 0 || num_tiles == 0) return DSV3_OK;
+    if (!dsv3_fp8_gemm_grouped_swiglu_fused(m, a_num_rows, inter, k)) return DSV3_ERR_BAD_SHAPE;   // ask ..._fused first
+    if (!a || !a_s || !b || !b_s || !y || !s || !tile_group || !tile_row0 || !tile_rows) return DSV3_ERR_NULL_POINTER;
+    if (!aligned(a, 16) || !aligned(b, 16) || b_group_stride % 16 != 0 || !aligned(a_s, 4) || !aligned(b_s, 4) ||
+        !aligned(y, 16) || !aligned(s, 4))
+        return DSV3_ERR_MISALIGNED;
+    return launch_grouped_swiglu(a, a_s, a_rows, b, b_s, y, s, m, inter, k, num_tiles, tile_group, tile_row0, tile_rows,
+                                 b_group_stride, bs_group_stride, scale_fmt, (hipStream_t)stream);
+}
+
 int dsv3_swiglu_quant(const void* h, int h_dtype, void* y, float* s, int64_t rows, int64_t inter,
                       int block_size, int scale_fmt, void* stream) {
     if (h_dtype != DSV3_BF16) return DSV3_ERR_BAD_DTYPE;

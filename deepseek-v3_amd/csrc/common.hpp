@@ -84,6 +84,28 @@ __device__ __forceinline__ float block_quotient(float x, float sc, float r, bool
     return x / sc;
 }
 
+// A binary32 value rounded to bf16 and widened again.
+__device__ __forceinline__ float round_bf16(float v) { return bf16lo_to_f32(pack_bf16(v, 0.f) & 0xffffu); }
+
+// silu(x1) * x3 as the reference's bf16 tensor operations round it (inference/model.py:633): F.silu on a bf16 tensor
+// is x / (1 + exp(-x)) in binary32 rounded to bf16, then the bf16 product.  exp(-x) goes through the hardware's 2^t:
+// after the rounding to bf16 the result equals the one with expf() for every bf16 x.  FAST (the caller guarantees
+// |x1| < 64): the denominator is a normal number far from overflow and a reciprocal with one correction step (and x's
+// sign for the zeros) rounds to the same bf16 as the IEEE division for every such x.  (Both checked on the device over
+// all 65536 bf16 values; x * rcp(1 + e) without the correction differs for a few inputs, and the corrected form fails
+// at x = -87.5 where the reciprocal is subnormal.)
+template <bool FAST> __device__ __forceinline__ float swiglu_bf16(float x1, float x3) {
+    const float d = 1.0f + __builtin_amdgcn_exp2f(-x1 * 1.44269504088896340736f);
+    float sl;
+    if (FAST) {
+        const float r = __builtin_amdgcn_rcpf(d), q0 = x1 * r;
+        sl = __builtin_copysignf(__builtin_fmaf(__builtin_fmaf(-q0, d, x1), r, q0), x1);
+    } else {
+        sl = x1 / d;
+    }
+    return round_bf16(round_bf16(sl) * x3);
+}
+
 // Output element writers: one binary32 -> C element of dsv3_dtype T.
 template <int DT> struct OutT;
 template <> struct OutT<DSV3_BF16> { typedef uint16_t type; static constexpr int bytes = 2; };
@@ -145,6 +167,11 @@ template <int CD, bool P2 = false>
 int launch_grouped(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s, void* c,
                    int64_t m, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group, const int* tile_row0,
                    const int* tile_rows, int64_t b_stride, int64_t bs_stride, hipStream_t stream);
+bool grouped_swiglu_supported(int64_t m, int64_t a_num_rows, int64_t inter, int64_t k);
+int launch_grouped_swiglu(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s,
+                          void* y, float* s, int64_t m, int64_t inter, int64_t k, int64_t num_tiles,
+                          const int* tile_group, const int* tile_row0, const int* tile_rows, int64_t b_stride,
+                          int64_t bs_stride, int scale_fmt, hipStream_t stream);
 int launch_grouped_skinny(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s, void* c,
                           int c_dtype, int64_t n, int64_t k, int64_t num_tiles, const int* tile_group,
                           const int* tile_row0, const int* tile_rows, int64_t b_stride, int64_t bs_stride,

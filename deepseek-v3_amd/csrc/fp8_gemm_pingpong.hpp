@@ -75,7 +75,7 @@ constexpr int LDS_BYTES = lds_bytes<4>();               // 136 KiB (100 KiB for 
 // results; the caller sends everything else down the one-tile path.
 constexpr int PS_STAGING = 8 * 2048;
 
-template <int CD, bool P2, bool G = false, int SM = 4, bool PS = false>
+template <int CD, bool P2, bool G = false, int SM = 4, bool PS = false, bool SG = false>
 __device__ __forceinline__ void tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -88,6 +88,7 @@ __device__ __forceinline__ void tile(
     constexpr int LDS_A = GEO::LDS_A, LDS_B = GEO::LDS_B, LDS_SC = GEO::LDS_SC, NM2 = GEO::NM2;
     static_assert(!G || SM == 4, "grouped slots run the 256-row tile");
     static_assert(!PS || (!G && SM == 4 && CD != DSV3_F32), "persistent mode: dense 256-row tiles with 16-bit results");
+    static_assert(!SG || (G && !P2 && CD == DSV3_BF16), "SwiGLU mode: grouped, binary32 scales, bf16 intermediate");
 
     // ---- workgroup -> tile: a contiguous run of tiles per XCD, walked in bands of GROUP_M tile rows; in grouped
     // mode the row tiles are dealt round-robin over the XCDs and the column tiles of a row tile stay on one XCD
@@ -107,6 +108,7 @@ __device__ __forceinline__ void tile(
         n0_ = (tn_first + in_band / band_rows) * BN;
     };
     int m0, n0, rows_here;
+    int tn_idx = 0;                     // (SwiGLU mode: the column tile)
     if (G) {
         const int x = wg % 8, idx = wg / 8;
         const int tm = (idx / tiles_n) * 8 + x, tn = idx - (idx / tiles_n) * tiles_n;
@@ -114,6 +116,7 @@ __device__ __forceinline__ void tile(
         m0 = g.tile_row0[tm];
         rows_here = g.tile_rows[tm];
         n0 = (tn_first + tn) * BN;
+        tn_idx = tn_first + tn;
         b += (size_t)expert * g.b_stride;
         b_s += (size_t)expert * g.bs_stride;
     } else {
@@ -176,7 +179,7 @@ __device__ __forceinline__ void tile(
     const uint32_t lds0 = lds_addr_of(lds);
     auto plan = [&](bool from_b, int q, uint32_t& src, uint32_t& dst0, uint32_t& dst1) {
         const int r = q * 8 + (lane >> 3), ch = (lane & 7) ^ swz(r);
-        src = (from_b ? (uint32_t)min(n0_ld + r, N - 1) : a_row(r)) * (uint32_t)K + ch * 16;
+        src = (from_b ? (uint32_t)(SG ? sg_weight_row(r, tn_idx, N / 2) : min(n0_ld + r, N - 1)) : a_row(r)) * (uint32_t)K + ch * 16;
         dst0 = lds0 + (from_b ? LDS_B : LDS_A) + q * 1024;
         dst1 = dst0 + (from_b ? B_STAGE : A_STAGE);
     };
@@ -217,8 +220,9 @@ __device__ __forceinline__ void tile(
     // per row, a one-line copy in the other three blocks to keep the counts) was built and was not faster.
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
-    const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT
-                                      : (uint32_t)min((PS ? 0 : n0 / 128) + (wave == 4 ? min(lane, 1) : 0), nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
+    const int b_scale_row = SG ? sg_scale_row(wave == 4 ? min(lane, 1) : 0, tn_idx, N / 2)
+                               : min((PS ? 0 : n0 / 128) + (wave == 4 ? min(lane, 1) : 0), nb_last);
+    const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT : (uint32_t)b_scale_row * (uint32_t)KBT) + (uint32_t)kb0;
     auto issue_scales = [&](int kb, int slot, bool tail = true) {
         if constexpr (PS) {
             const bool nx = tail && kb >= KB;
@@ -459,6 +463,10 @@ __device__ __forceinline__ void tile(
     // ---- epilogue: lane holds c[m][n .. n + 3] for every (i, j); see fp8_gemm_prefill.hip for the LDS route
     constexpr int WN = 128, SN = 8;
     auto sub_row = [&](int j) { return wm * WM + j * 16; };
+    if constexpr (SG) {
+        swiglu_store<SM>(acc, lds, wm, grp, lane, sub_row, m0, rows_here, tn_idx, N / 2, g);
+        return;
+    }
     const bool lds_epilogue = CD != DSV3_F32 && (N % 8) == 0 && ldc == N;
     const bool f32_lds_epilogue = CD == DSV3_F32 && (N % 4) == 0 && (ldc % 4) == 0;
     const bool vec_ok = (N % 4) == 0 && (ldc % 4) == 0;

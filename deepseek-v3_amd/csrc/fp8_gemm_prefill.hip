@@ -79,13 +79,97 @@ struct GroupTable {
     const int* a_rows;       // [rows of c] or nullptr
     int64_t b_stride;        // bytes between consecutive groups' weights
     int64_t bs_stride;       // floats between consecutive groups' weight scales
+    // SwiGLU mode (SG): the tile's results do not leave as c but as act_quant(silu(h1) * h3), see swiglu_store
+    uint8_t* sg_y;           // [rows of c, N / 2] e4m3
+    float* sg_s;             // [rows of c, N / 256] scales
+    int sg_ue8m0;            // scale format of the re-quantisation
 };
+
+// SwiGLU mode of the grouped kernels (inference/model.py:633 feeding the Linear of :631 -> inference/kernel.py:23-35):
+// a group's weight is w1 stacked over w3 ([2 * inter, K]); a column tile takes the matching 128 rows of both as its
+// two column halves -- rows tn * 128 .. + 127 of w1 for the first m-wavefront column, the same rows of w3 for the
+// second -- so that after the K loop wavefront (wm, 0) holds h1 and wavefront (wm, 1) h3 of the same 64 x 128 outputs.
+// Weight row behind row r (0 .. 255) of column tile tn, and the scale row of a column half:
+__device__ __forceinline__ int sg_weight_row(int r, int tn, int inter) { return (r < 128 ? 0 : inter - 128) + tn * 128 + r; }
+__device__ __forceinline__ int sg_scale_row(int half, int tn, int inter) { return (half ? inter / 128 : 0) + tn; }
+
+// Epilogue of SwiGLU mode.  h3 crosses from wavefront (wm, 1) to (wm, 0) through LDS in the accumulators' own
+// layout (lane l of the one writes what lane l of the other reads: 512 contiguous bytes per 16 x 16 tile, no bank
+// conflicts); the first wavefront then forms g = bf16(bf16(silu(bf16 h1)) * bf16 h3) with the arithmetic of
+// dsv3_swiglu_quant, reduces the row maximum over its 32 values and the three other lanes that hold the row, and
+// writes 128 e4m3 bytes and one scale per row: the 128 columns of a tile are exactly one quantisation block.
+// The result is what dsv3_fp8_gemm_grouped followed by dsv3_swiglu_quant produces, bit for bit; it saves that launch
+// and three quarters of the bytes the GEMM writes.  acc[i][j]: column sub-tile i (16 columns), row sub-tile j.
+template <int SM, typename SubRow>
+__device__ __forceinline__ void swiglu_store(v4f (&acc)[8][SM], uint8_t* lds, int wm, int wn, int lane, SubRow sub_row,
+                                             int m0, int rows_here, int tn, int inter, const GroupTable& g) {
+    const int fr = lane & 15, fq = lane >> 4;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // every wavefront is done with the LDS stages
+    v2u* xch = (v2u*)(lds + wm * (SM * 8 * 512));
+    if (wn == 1) {
+#pragma unroll
+        for (int j = 0; j < SM; ++j)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                xch[(j * 8 + i) * 64 + lane] = v2u{ pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3]) };
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (wn == 1) return;
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        if (sub_row(j) >= rows_here) continue;                         // (uniform) a sub-tile of padding rows
+        float x1[8][4], big = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { x1[i][e] = round_bf16(acc[i][j][e]); big = fmaxf(big, fabsf(x1[i][e])); }
+        float gv[8][4];
+        const bool fast = __all(big < 64.f);                            // (false for NaN as well)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const v2u h3 = xch[(j * 8 + i) * 64 + lane];
+            const float x3[4] = { bf16lo_to_f32(h3[0]), bf16hi_to_f32(h3[0]), bf16lo_to_f32(h3[1]), bf16hi_to_f32(h3[1]) };
+#pragma unroll
+            for (int e = 0; e < 4; ++e) gv[i][e] = fast ? swiglu_bf16<true>(x1[i][e], x3[e]) : swiglu_bf16<false>(x1[i][e], x3[e]);
+        }
+        uint32_t abits = 0u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) abits = umax_u32(abits, abs_bits(gv[i][e]));
+        abits = umax_u32(abits, (uint32_t)__shfl_xor((int)abits, 16));  // the row's other three lanes
+        abits = umax_u32(abits, (uint32_t)__shfl_xor((int)abits, 32));
+        const float sc = block_scale(abits, g.sg_ue8m0 != 0);
+        const bool finite = __all(block_is_finite(abits));              // uniform, so that only one quotient is evaluated
+        const float rcp = 1.0f / sc;
+        // the sub-tile's 16 rows x 128 bytes pass through the part of the exchange area this wavefront has just read
+        // (16-byte chunks xor-ed with the row), so that a store instruction writes 8 whole rows instead of 16-byte pieces
+        uint8_t* stg = (uint8_t*)(xch + j * 8 * 64);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float q[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) q[e] = finite ? block_quotient(gv[i][e], sc, rcp, true) : block_quotient(gv[i][e], sc, rcp, false);
+            *(uint32_t*)(stg + fr * 128 + ((i ^ (fr & 7)) * 16) + fq * 4) = pack_fp8x4(q[0], q[1], q[2], q[3]);
+        }
+        const int r0 = sub_row(j);
+        if (fq == 0 && r0 + fr < rows_here) g.sg_s[(size_t)(m0 + r0 + fr) * (size_t)(inter / 128) + tn] = sc;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int rr = p * 8 + (lane >> 3), ch = lane & 7;
+            const v4u v = *(const v4u*)(stg + rr * 128 + ((ch ^ (rr & 7)) * 16));
+            if (r0 + rr < rows_here)
+                *(v4u*)(g.sg_y + (size_t)(m0 + r0 + rr) * (size_t)inter + tn * 128 + ch * 16) = v;
+        }
+    }
+}
 
 // One workgroup's tile (grouped mode: tile slot) from start to end; the kernels below are thin wrappers.
 // P2: every scale is a power of two (act_quant's ue8m0 format and checkpoints whose block scales are stored that
 // way).  The block scales then ride in the MFMA's E8M0 scale operands and the products of all K blocks accumulate
 // inside the matrix core: no fold, no vector-ALU work in the K loop.
-template <int CD, bool G, int TM, int S, int SB = S, bool P2 = false>
+template <int CD, bool G, int TM, int S, int SB = S, bool P2 = false, bool SG = false>
 __device__ __forceinline__ void prefill_tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -96,6 +180,7 @@ __device__ __forceinline__ void prefill_tile(
     constexpr int SS = C::SS;
     constexpr int WM = C::WM, SM = C::SM, A_LOADS = C::A_LOADS, B_LOADS = C::B_LOADS;
     constexpr int A_STAGE = C::A_STAGE, B_STAGE = C::B_STAGE, LDS_A = C::LDS_A, LDS_B = C::LDS_B, LDS_SC = C::LDS_SC;
+    static_assert(!SG || (G && !P2 && CD == DSV3_BF16), "SwiGLU mode: grouped, binary32 scales, bf16 intermediate");
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     // ---- workgroup -> tile.  Consecutive workgroup ids go to consecutive XCDs (8 of them, each with its own L2).
@@ -104,6 +189,7 @@ __device__ __forceinline__ void prefill_tile(
     // contiguous split would leave the XCDs that get the unused tail idle -- and keeps the column tiles of a row
     // tile on one XCD (they share the gathered rows of a).
     int m0, n0, rows_here;              // first row of the tile in c, first column, valid rows
+    int tn_idx = 0;                     // (SwiGLU mode: the column tile)
     if (G) {
         const int x = wg % 8, idx = wg / 8;
         const int tm = (idx / tiles_n) * 8 + x, tn = idx - (idx / tiles_n) * tiles_n;
@@ -113,6 +199,7 @@ __device__ __forceinline__ void prefill_tile(
         m0 = g.tile_row0[tm];
         rows_here = g.tile_rows[tm];
         n0 = (tn_first + tn) * BN;
+        tn_idx = tn_first + tn;
         b += (size_t)grp * g.b_stride;
         b_s += (size_t)grp * g.bs_stride;
     } else {
@@ -175,7 +262,7 @@ __device__ __forceinline__ void prefill_tile(
 #pragma unroll
     for (int t = A_LOADS; t < A_LOADS + B_LOADS; ++t) {
         const int row = ((t - A_LOADS) * 8 + wave) * 8 + (lane >> 3);
-        src_off[t] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + (((lane & 7) ^ swz(row)) * 16);
+        src_off[t] = (uint32_t)(SG ? sg_weight_row(row, tn_idx, N / 2) : min(n0 + row, N - 1)) * (uint32_t)K + (((lane & 7) ^ swz(row)) * 16);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -210,8 +297,9 @@ __device__ __forceinline__ void prefill_tile(
     // instruction instead of 64.
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
-    const uint32_t sc_off = (wave < 4 ? a_scale_row * (uint32_t)KBT
-                                      : (uint32_t)min(n0 / 128 + (wave == 4 ? min(lane, 1) : 0), nb_last) * (uint32_t)KBT) + (uint32_t)kb0;
+    const int b_scale_row = SG ? sg_scale_row(wave == 4 ? min(lane, 1) : 0, tn_idx, N / 2)
+                               : min(n0 / 128 + (wave == 4 ? min(lane, 1) : 0), nb_last);
+    const uint32_t sc_off = (wave < 4 ? a_scale_row * (uint32_t)KBT : (uint32_t)b_scale_row * (uint32_t)KBT) + (uint32_t)kb0;
     auto issue_scales = [&](int kb, int stage) {
         __builtin_amdgcn_global_load_lds((gptr_t)(sc_base + sc_off + (uint32_t)kb),
                                          (lptr_t)(lds + LDS_SC + stage * SC_STAGE + wave * 256), 4, 0, 0);
@@ -490,10 +578,16 @@ __device__ __forceinline__ void prefill_tile(
     else if (ja_live == 1)  pipeline(std::integral_constant<int, 1>{});
     else {
         pipeline(std::integral_constant<int, 0>{});
+        if (SG) { wg_barrier(); wg_barrier(); return; }         // the two barriers of swiglu_store
         if (lds_epilogue || f32_lds_epilogue) wg_barrier();     // the barrier the other wavefronts take before they reuse the LDS stages
         return;
     }
 #undef DSV3_SGB
+    if constexpr (SG) {
+        static_assert(SN == 8, "swiglu_store: eight column sub-tiles per wavefront");
+        swiglu_store<SM>(acc, lds, wm, wn, lane, sub_row, m0, rows_here, tn_idx, N / 2, g);
+        return;
+    }
 
     // ---- epilogue: lane holds c[m][n .. n+3] for every (i, j)
     const bool vec_ok = (N % 4) == 0 && (ldc % 4) == 0;
@@ -611,7 +705,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 // straight from HBM, and a second block of prefetch is what hides that), one with fewer the 128-row
 // configuration with three stages of both.  The choice is uniform over the workgroup and needs no host knowledge of
 // the group sizes: a layer with a few rows per expert and one with hundreds go through the same launch.
-template <int CD, bool P2 = false>
+template <int CD, bool P2 = false, bool SG = false>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -622,12 +716,12 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
     const int rows = g.tile_rows[tm];
     if (rows > 192) {
         if (g.tile_group[tm] < 0) return;
-        pingpong::tile<CD, P2, true>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x, g);
+        pingpong::tile<CD, P2, true, 4, false, SG>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x, g);
     }
     else if (rows > 128)
-        prefill_tile<CD, true, 192, 2, 3, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+        prefill_tile<CD, true, 192, 2, 3, P2, SG>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
     else
-        prefill_tile<CD, true, 128, 3, 3, P2>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+        prefill_tile<CD, true, 128, 3, 3, P2, SG>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
 }
 
 // Dense GEMM whose last column tiles run as 128-row tiles: the first tiles_m * tn_tall workgroups compute 256-row
@@ -947,7 +1041,7 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
     if (m <= skinny_max)
         return launch_grouped_skinny(a, a_s, a_rows, b, b_s, c, CD, n, k, num_tiles, tile_group, tile_row0, tile_rows,
                                      b_stride, bs_stride, m < num_tiles ? m : num_tiles, stream);
-    GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride};
+    GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride, nullptr, nullptr, 0};
     constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES;               // the largest of the three configurations
     static_assert(LDS_BYTES >= pingpong::LDS_BYTES && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES, "LDS of the grouped kernel");
     const int64_t tn = (n + BN - 1) / BN;
@@ -960,6 +1054,36 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
                        (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)num_tiles,
                        (int)tn, 0, (int)(k / 128), (int)n, g);
+    return launch_status();
+}
+
+// The first GEMM of a SwiGLU block with the activation and the re-quantisation in its epilogue (SwiGLU mode above): b
+// holds w1 over w3 per group ([2 * inter, k]), y / s receive act_quant(silu(a w1^T) * (a w3^T)).  Only the tile kernels
+// have this mode: launches of few rows (the weight-streaming kernel's) are refused and take the two separate calls.
+bool grouped_swiglu_supported(int64_t m, int64_t a_num_rows, int64_t inter, int64_t k) {
+    static const int skinny_max = getenv("DSV3_GROUPED_SKINNY_MAX") ? atoi(getenv("DSV3_GROUPED_SKINNY_MAX")) : 320;
+    return m > skinny_max && inter >= 128 && inter % 128 == 0 && grouped_supported(a_num_rows, 2 * inter, k) &&
+           m * inter < (1ll << 32);
+}
+
+int launch_grouped_swiglu(const void* a, const float* a_s, const int* a_rows, const void* b, const float* b_s,
+                          void* y, float* s, int64_t m, int64_t inter, int64_t k, int64_t num_tiles,
+                          const int* tile_group, const int* tile_row0, const int* tile_rows, int64_t b_stride,
+                          int64_t bs_stride, int scale_fmt, hipStream_t stream) {
+    using namespace prefill;
+    GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride, (uint8_t*)y, s,
+                 scale_fmt == DSV3_SCALE_FMT_UE8M0 ? 1 : 0};
+    constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES;
+    const int64_t tn = inter / 128;
+    if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    if (num_tiles * tn == 0) return DSV3_OK;
+    auto kern = fp8_gemm_grouped_kernel<DSV3_BF16, false, true>;
+    static LdsGrant grant;
+    if (!grant.ensure((const void*)kern, LDS_BYTES)) return DSV3_ERR_LAUNCH;
+    const int64_t grid = (num_tiles + 7) / 8 * 8 * tn;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
+                       (const uint8_t*)b, b_s, (uint16_t*)nullptr, (int)m, (int)(2 * inter), (int)k, (int)num_tiles,
+                       (int)tn, 0, (int)(k / 128), (int)(2 * inter), g);
     return launch_status();
 }
 

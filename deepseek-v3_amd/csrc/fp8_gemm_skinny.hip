@@ -185,36 +185,29 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
         // the 8 lanes that hold the chunks of one (row, K block) are consecutive and aligned: amax by DPP
 #pragma unroll
         for (int i = 0; i < kSlabChunks; ++i) {
-            float f[16];
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    f[8 * h + 2 * e] = bf16lo_to_f32(raw[i][h][e]);
-                    f[8 * h + 2 * e + 1] = bf16hi_to_f32(raw[i][h][e]);
-                }
+            // (the 16 values are widened twice, for the maximum and for the quotients, instead of being kept: with the
+            // weight ring live this section must stay inside the register budget)
+            auto widen = [&](int e) { return (e & 1) ? bf16hi_to_f32(raw[i][e >> 3][(e >> 1) & 3]) : bf16lo_to_f32(raw[i][e >> 3][(e >> 1) & 3]); };
             uint32_t abits = 0u;                 // non-finite values reach the scale as in act_quant
 #pragma unroll
-            for (int e = 0; e < 16; ++e) abits = umax_u32(abits, abs_bits(f[e]));
+            for (int e = 0; e < 16; ++e) abits = umax_u32(abits, abs_bits(widen(e)));
             abits = dpp_umax<0xB1>(abits);       // quad_perm [1,0,3,2]
             abits = dpp_umax<0x4E>(abits);       // quad_perm [2,3,0,1]
             abits = dpp_umax<0x141>(abits);      // row_half_mirror
             const float sc = block_scale(abits, ue8m0 != 0);
-            float q[16];
-            if (block_is_finite(abits)) {        // x / sc, correctly rounded for bf16 x with |x| <= amax (as act_quant)
-                const float r = 1.0f / sc;
+            const bool fast = block_is_finite(abits);
+            const float r = 1.0f / sc;
+            v4i o;
 #pragma unroll
-                for (int e = 0; e < 16; ++e) q[e] = block_quotient(f[e], sc, r, true);
-            } else {
+            for (int g = 0; g < 4; ++g) {        // x / sc, correctly rounded for bf16 x with |x| <= amax (as act_quant)
+                float q[4];
 #pragma unroll
-                for (int e = 0; e < 16; ++e) q[e] = block_quotient(f[e], sc, 0.f, false);
+                for (int e = 0; e < 4; ++e) q[e] = fast ? block_quotient(widen(4 * g + e), sc, r, true) : block_quotient(widen(4 * g + e), sc, r, false);
+                o[g] = (int)pack_fp8x4(q[0], q[1], q[2], q[3]);
             }
             const int c = tid + i * (int)blockDim.x;
             if (c < chunks) {
                 const int ch = c & 7, R = c >> 3;
-                v4i o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (int)pack_fp8x4(q[4 * e], q[4 * e + 1], q[4 * e + 2], q[4 * e + 3]);
                 *(v4i*)(act + R * 128 + ((ch ^ swz(R)) * 16)) = o;
                 if (ch == 0) act_s[R] = sc * stage_q[i];
             }

@@ -283,15 +283,14 @@ Plan make_plan(int64_t m, int64_t n, int64_t k) {
     return p;
 }
 
-// 3 to 16 rows on a weight of 96 MiB or more with 8192 rows or more: the dense GEMM runs as one group of the grouped
-// weight-streaming kernel -- 32-row strips of such a weight fill the chip, one launch, no partial sums in memory
-// (7168 -> 36864 at 8 rows 51 against 70 us).  One and two rows stay with the M <= 16 kernel, which quantises bf16
-// activations itself for linear() there.
+// 3 to 16 rows on a weight of 96 MiB or more for which the activation-streaming kernel has no plan: the dense GEMM runs
+// as one group of the grouped weight-streaming kernel -- 32-row strips of such a weight fill the chip, one launch, no
+// partial sums in memory.
 bool single_group_stream(int64_t m, int64_t n, int64_t k) {
     if (m < 3 || m > 16 || n * k < (96ll << 20) || !skinny_single_supported(m, n, k)) return false;
-    // weights of fewer than 8192 rows: the activation-streaming kernel with two workgroups per compute unit
-    // (16384 -> 7168 at 4 / 8 / 16 rows: 22.4 / 22.7 / 23.8 against 25.6 / 26.7 / 29.6 us)
-    return !(n < 8192 && stream_supported(m, n, k));
+    // wherever the activation-streaming kernel has a plan it is faster (16384 -> 7168 at 4 / 8 / 16 rows: 22.2 / 22.5 /
+    // 23.5 against 25.6 / 26.7 / 29.6 us; 7168 -> 18432: 22 / 22 / 22.8 against 28.5 / 31 / 36.5 us)
+    return !stream_supported(m, n, k);
 }
 
 // DSV3_GEMM_FORCE=tile|prefill|stream|skinny pins the kernel choice where the named kernel supports the shape (tuning /
@@ -310,15 +309,16 @@ int forced_kernel() {
 }
 
 // Which problems go to the large-M kernel (K range cut into slices when the tiles do not fill the chip): every M
-// above 64, and M = 9 .. 64 when the weight is large (>= 96 MiB) and has 8192 rows or more.  There it runs at a flat
-// 32-34 us per 117-132 MB from 9 to 64 rows.  Large weights of fewer rows go to the activation-streaming kernel
-// (16384 -> 7168 at 16 / 32 / 64 rows 23.8 / 27.3 / 32.7 against 33 / 31.6 / 34.6 us); for the smaller decode weights
-// the streaming and tile kernels are faster anyway.
+// above 64, and M = 33 .. 64 when the weight is large (>= 96 MiB) and has 8192 rows or more (7168 -> 36864 at 64 rows:
+// 65 against 66-76 us).  There it runs at a flat 32-34 us per 117-132 MB from 9 to 64 rows.  Everything else the
+// activation-streaming kernel has a plan for goes there (16384 -> 7168 at 16 / 32 / 64 rows 23.5 / 24.5 / 29.5 against
+// 33 / 31.6 / 34.6 us; 7168 -> 18432 at 16 / 32 rows 22.8 / 25.3 against 36.5 / 30.7 us); for the smaller decode
+// weights the streaming and tile kernels are faster anyway.
 bool to_large_m_kernel(int64_t m, int64_t n, int64_t k) {
     if (!prefill_supported(m, n, k)) return false;
     if (m > 64) return true;
     if (m <= 8 || n * k < (96ll << 20)) return false;
-    return !(n < 8192 && stream_supported(m, n, k));
+    return !((n < 8192 || m <= 32) && stream_supported(m, n, k));
 }
 
 template <int CD>

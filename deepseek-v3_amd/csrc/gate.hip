@@ -50,7 +50,6 @@ __device__ __forceinline__ Best wave_argmax(Best x) {
 __device__ __forceinline__ Best better(Best a, Best b) {
     return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
 }
-__device__ __forceinline__ float round_bf16(float x) { return bf16lo_to_f32(pack_bf16(x, 0.f) & 0xffffu); }
 
 constexpr int kTokensPerWg = 4;
 

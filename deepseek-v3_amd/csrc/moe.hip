@@ -16,8 +16,6 @@ namespace {
 
 constexpr int kThreads = 256;
 
-__device__ __forceinline__ float round_bf16(float v) { return bf16lo_to_f32(pack_bf16(v, 0.f) & 0xffffu); }
-
 // h: [rows, 2*inter] bf16 (h1 | h3 side by side), y: [rows, inter] e4m3, s: [rows, inter/128].
 // A lane owns 8 consecutive output columns; the 16 lanes of a DPP row own one 128-wide scale block.
 template <bool UE8M0>
@@ -31,13 +29,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_quant_kernel(
     const int col = (int)(cc - row * chunks_per_row);
     const v4u a = __builtin_nontemporal_load(h + row * 2 * chunks_per_row + col);
     const v4u b = __builtin_nontemporal_load(h + row * 2 * chunks_per_row + chunks_per_row + col);
-    // F.silu on a bf16 tensor: x / (1 + exp(-x)) in binary32, rounded to bf16; then the bf16 product with h3.
-    // exp(-x) goes through the hardware's 2^t: after the rounding to bf16 the result equals the one with expf() for
-    // every bf16 x.  The division is the IEEE one unless every |x| of the wavefront is below 64; then the
-    // denominator is a normal number far from overflow and a reciprocal with one correction step (and x's sign for
-    // the zeros) rounds to the same bf16 for every such x.  (Both checked on the device over all 65536 bf16 values;
-    // x * rcp(1 + e) without the correction differs for a few inputs, and the corrected form fails at x = -87.5
-    // where the reciprocal is subnormal.)
+    // silu(h1) * h3 with the roundings of the reference's bf16 tensors (swiglu_bf16); the IEEE division unless every
+    // |x| of the wavefront is below 64
     float x1[8], x3[8], g[8], big = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -47,18 +40,10 @@ __global__ __launch_bounds__(kThreads) void swiglu_quant_kernel(
     }
     if (__all(big < 64.f)) {            // (false for NaN as well)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float d = 1.0f + __builtin_amdgcn_exp2f(-x1[i] * 1.44269504088896340736f);
-            const float r = __builtin_amdgcn_rcpf(d), q0 = x1[i] * r;
-            const float q = __builtin_copysignf(__builtin_fmaf(__builtin_fmaf(-q0, d, x1[i]), r, q0), x1[i]);
-            g[i] = live ? round_bf16(round_bf16(q) * x3[i]) : 0.f;
-        }
+        for (int i = 0; i < 8; ++i) g[i] = live ? swiglu_bf16<true>(x1[i], x3[i]) : 0.f;
     } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float sl = round_bf16(x1[i] / (1.0f + __builtin_amdgcn_exp2f(-x1[i] * 1.44269504088896340736f)));
-            g[i] = live ? round_bf16(sl * x3[i]) : 0.f;
-        }
+        for (int i = 0; i < 8; ++i) g[i] = live ? swiglu_bf16<false>(x1[i], x3[i]) : 0.f;
     }
     uint32_t abits = 0u;             // non-finite values reach the scale as in act_quant
 #pragma unroll

@@ -45,6 +45,10 @@ EXPORTS = {
     "dsv3_fp8_gemm_grouped_pow2": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64,
                                            c_void_p, c_int, c_int64, c_int64, c_int64,
                                            c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
+    "dsv3_fp8_gemm_grouped_swiglu_fused": (c_int, [c_int64, c_int64, c_int64, c_int64]),
+    "dsv3_fp8_gemm_grouped_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64,
+                                             c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                             c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "dsv3_swiglu_quant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]),
     "dsv3_moe_combine": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int64, c_int, c_int64, c_void_p]),

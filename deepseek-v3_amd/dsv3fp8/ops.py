@@ -30,6 +30,8 @@ _libdef.define("group_tiles(Tensor counts, int max_tiles) -> (Tensor, Tensor, Te
 _libdef.define("moe_route(Tensor indices, Tensor weights, int experts, bool shared_group) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)")
 _libdef.define("fp8_gemm_grouped(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b, Tensor b_s, int rows, "
                "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int out_dtype) -> Tensor")
+_libdef.define("fp8_gemm_grouped_swiglu(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b, Tensor b_s, int rows, "
+               "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int scale_fmt) -> (Tensor, Tensor)")
 _libdef.define("fp8_gemm_grouped_pow2(Tensor a, Tensor a_s, Tensor? a_rows, Tensor b, Tensor b_s, int rows, "
                "Tensor tile_group, Tensor tile_row0, Tensor tile_rows, int out_dtype) -> Tensor")
 _libdef.define("swiglu_quant(Tensor h, int block_size, int scale_fmt) -> (Tensor, Tensor)")
@@ -250,6 +252,42 @@ def _fp8_gemm_grouped_meta(a, a_s, a_rows, b, b_s, rows, tile_group, tile_row0, 
     return a.new_empty(rows, b.size(1), dtype=_CODE_DTYPE[out_dtype])
 
 
+def grouped_swiglu_fused(rows: int, a_num_rows: int, inter: int, k: int) -> bool:
+    """Whether the first grouped GEMM of a SwiGLU block can carry the activation and the re-quantisation in its
+    epilogue (dsv3_fp8_gemm_grouped_swiglu) for a launch of this size."""
+    return bool(_lib.lib.dsv3_fp8_gemm_grouped_swiglu_fused(rows, a_num_rows, inter, k))
+
+
+def _fp8_gemm_grouped_swiglu_dev(a, a_s, a_rows, b, b_s, rows: int, tile_group, tile_row0, tile_rows, scale_fmt: int):
+    """fp8_gemm_grouped over b = [w1 ; w3] per group followed by swiglu_quant, fused where the library implements it
+    (the same bits either way); returns (y [rows, inter] e4m3, s [rows, inter / 128])."""
+    k, inter = a.size(1), b.size(1) // 2
+    if not grouped_swiglu_fused(rows, a.size(0), inter, k):
+        h = _fp8_gemm_grouped_dev(a, a_s, a_rows, b, b_s, rows, tile_group, tile_row0, tile_rows, _lib.BF16)
+        return _swiglu_quant_dev(h, 128, scale_fmt)
+    assert a.dim() == 2 and b.dim() == 3 and b_s.dim() == 3 and a.is_contiguous() and b.is_contiguous()
+    assert a_s.is_contiguous() and b_s.is_contiguous() and b.size(0) == b_s.size(0) and b.size(2) == k
+    for t in (tile_group, tile_row0, tile_rows):
+        assert t.dtype == torch.int32 and t.is_contiguous() and t.numel() == tile_group.numel()
+    if a_rows is not None:
+        assert a_rows.dtype == torch.int32 and a_rows.is_contiguous() and a_rows.numel() == rows
+    y = a.new_empty(rows, inter, dtype=FP8)
+    s = a.new_empty(rows, inter // 128, dtype=torch.float32)
+    with torch.cuda.device(a.device):
+        rc = _lib.lib.dsv3_fp8_gemm_grouped_swiglu(
+            a.data_ptr(), a_s.data_ptr(), a_rows.data_ptr() if a_rows is not None else None, a.size(0),
+            b.data_ptr(), b_s.data_ptr(), b.stride(0), b_s.stride(0), y.data_ptr(), s.data_ptr(), rows, inter, k,
+            tile_group.data_ptr(), tile_row0.data_ptr(), tile_rows.data_ptr(), tile_group.numel(), 128, scale_fmt,
+            _stream(a))
+    _lib.check(rc, "dsv3_fp8_gemm_grouped_swiglu")
+    return y, s
+
+
+def _fp8_gemm_grouped_swiglu_meta(a, a_s, a_rows, b, b_s, rows, tile_group, tile_row0, tile_rows, scale_fmt):
+    inter = b.size(1) // 2
+    return a.new_empty(rows, inter, dtype=FP8), a.new_empty(rows, inter // 128, dtype=torch.float32)
+
+
 def _swiglu_quant_dev(h: torch.Tensor, block_size: int, scale_fmt: int):
     assert h.dim() == 2 and h.is_contiguous() and h.size(1) % 2 == 0
     rows, inter = h.size(0), h.size(1) // 2
@@ -337,6 +375,7 @@ for _name, _dev, _meta in (("wkv_b_absorb", _wkv_b_absorb_dev, _wkv_b_absorb_met
                            ("moe_route", _moe_route_dev, _moe_route_meta),
                            ("fp8_gemm_grouped", _fp8_gemm_grouped_dev, _fp8_gemm_grouped_meta),
                            ("fp8_gemm_grouped_pow2", _fp8_gemm_grouped_pow2_dev, _fp8_gemm_grouped_meta),
+                           ("fp8_gemm_grouped_swiglu", _fp8_gemm_grouped_swiglu_dev, _fp8_gemm_grouped_swiglu_meta),
                            ("swiglu_quant", _swiglu_quant_dev, _swiglu_quant_meta),
                            ("moe_combine", _moe_combine_dev, _moe_combine_meta)):
     _libimpl.impl(_name, _dev, "CUDA")

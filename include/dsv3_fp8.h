@@ -13,7 +13,8 @@
  * Around them, each documented at its declaration: dsv3_linear_fp8 (the two calls of linear() as one launch for
  * few rows), dsv3_fp8_gemm_pow2 / dsv3_fp8_gemm_grouped_pow2 (power-of-two scales), dsv3_weight_quant (the inverse
  * of weight_dequant), the mixture-of-experts functions (dsv3_gate_route, dsv3_moe_route, dsv3_group_tiles,
- * dsv3_fp8_gemm_grouped, dsv3_swiglu_quant, dsv3_moe_combine) and dsv3_wkv_b_absorb (attention).
+ * dsv3_fp8_gemm_grouped, dsv3_fp8_gemm_grouped_swiglu, dsv3_swiglu_quant, dsv3_moe_combine) and
+ * dsv3_wkv_b_absorb (attention).
  *
  * Conventions
  *   - every pointer is a device pointer into memory the caller owns; the library
@@ -262,6 +263,26 @@ int dsv3_fp8_gemm_grouped_pow2(const void* a, const float* a_s, const int32_t* a
                                void* c, int c_dtype, int64_t m, int64_t n, int64_t k,
                                const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
                                int64_t num_tiles, void* stream);
+
+/*
+ * The first grouped GEMM of a SwiGLU expert block with the activation and the re-quantisation in its epilogue
+ * (inference/model.py:633: w2(silu(w1 x) * w3 x); the act_quant is that of w2's linear(), inference/model.py:159):
+ *     h = dsv3_fp8_gemm_grouped(a, ..., b = [w1 ; w3] per group) as bf16;  (y, s) = dsv3_swiglu_quant(h)
+ * in one launch, bit for bit: a column tile multiplies with the matching 128 rows of w1 and of w3, so that it
+ * holds both factors of its 128 outputs -- one quantisation block -- and writes e4m3 bytes and scales instead of
+ * 16-bit sums (a quarter of the bytes, and the launch in between is gone).
+ * b: per group [2 * inter, k] (w1 over w3), b_s: per group [2 * inter / 128, k / 128]; y: [m, inter] e4m3,
+ * s: [m, inter / 128]; the other arguments as dsv3_fp8_gemm_grouped.  block_size must be 128 and inter a multiple
+ * of it.  Only the tile kernel has this epilogue: dsv3_fp8_gemm_grouped_swiglu_fused(m, a_num_rows, inter, k) says
+ * whether a launch qualifies (more rows in all than the weight-streaming kernel takes); the entry point returns
+ * DSV3_ERR_BAD_SHAPE otherwise and the caller issues the two separate calls.
+ */
+int dsv3_fp8_gemm_grouped_swiglu_fused(int64_t m, int64_t a_num_rows, int64_t inter, int64_t k);
+int dsv3_fp8_gemm_grouped_swiglu(const void* a, const float* a_s, const int32_t* a_rows, int64_t a_num_rows,
+                                 const void* b, const float* b_s, int64_t b_group_stride, int64_t bs_group_stride,
+                                 void* y, float* s, int64_t m, int64_t inter, int64_t k,
+                                 const int32_t* tile_group, const int32_t* tile_row0, const int32_t* tile_rows,
+                                 int64_t num_tiles, int block_size, int scale_fmt, void* stream);
 
 /*
  * silu(h1) * h3 followed by act_quant, in one pass (inference/model.py:633 feeding the act_quant of w2's

@@ -154,6 +154,26 @@ def test_grouped_validation(L):
     assert call(m=0, a=None, tg=None) == 0 and call(nt=0) == 0
 
 
+def test_grouped_swiglu_validation(L):
+    f, fused = L.lib.dsv3_fp8_gemm_grouped_swiglu, L.lib.dsv3_fp8_gemm_grouped_swiglu_fused
+    assert fused(4096, 4096, 2048, 7168) and fused(321, 100, 128, 128)
+    assert not fused(320, 4096, 2048, 7168)          # few rows in all: the weight-streaming kernel, two calls
+    assert not fused(4096, 4096, 2000, 7168) and not fused(4096, 4096, 2048, 7100) and not fused(0, 0, 128, 128)
+    ok = dict(a=A16, a_s=A16, a_rows=None, an=4096, b=A16, b_s=A16, bst=256 * 128, sst=2, y=A16, s=A16,
+              m=4096, inter=128, k=128, tg=A16, t0=A16, tr=A16, nt=40, blk=128, fmt=0, st=None)
+
+    def call(**kw):
+        v = {**ok, **kw}
+        return f(*[v[key] for key in ("a", "a_s", "a_rows", "an", "b", "b_s", "bst", "sst", "y", "s", "m", "inter", "k",
+                                      "tg", "t0", "tr", "nt", "blk", "fmt", "st")])
+    assert call(a=None) == 1 and call(y=None) == 1 and call(s=None) == 1 and call(tr=None) == 1
+    assert call(k=100) == 2 and call(inter=100) == 2 and call(m=-1) == 2
+    assert call(m=100) == 2                          # below the tile kernel's range: ask ..._fused first
+    assert call(blk=64) == 3 and call(fmt=5) == 5
+    assert call(a=A16 + 8) == 4 and call(y=A16 + 2) == 4 and call(bst=100) == 4
+    assert call(m=0) == 0 and call(nt=0) == 0
+
+
 def test_group_tiles_validation(L):
     f = L.lib.dsv3_group_tiles
     assert f(None, 4, 8, A16, A16, A16, None) == 1

@@ -506,3 +506,46 @@ def test_fused_linear_non_finite_activations(K, fmt):
     assert bool(torch.isnan(two[:3]).all()) and bool(torch.isfinite(two[3]).all())
     assert torch.equal(torch.isnan(one), torch.isnan(two))
     assert torch.equal(one[3], two[3])
+
+
+_RING_CASES = [(1, 16384, 7168), (2, 16384, 7168), (1, 32768, 2048), (2, 32768, 1000)]
+
+
+def _ring_outputs():
+    """fp8_gemm and the one-call linear on shapes whose M <= 16 kernel runs its ring variant (every wavefront's K range
+    two ring rounds or more): the weight loads and their counted waits are written out by hand there."""
+    import dsv3fp8 as K
+    from dsv3fp8 import workloads, ops, _lib
+    out = {}
+    for m, k, n in _RING_CASES:
+        x = workloads.activations(m, k, seed=m + k % 13).cuda()
+        w8, ws = workloads.weight(n, k, seed=n % 17)
+        w8, ws = w8.cuda(), ws.cuda()
+        a, a_s = K.act_quant(x)
+        out[f"gemm_{m}_{k}_{n}"] = torch.ops.dsv3fp8.fp8_gemm(a, a_s, w8, ws, _lib.F32).cpu()
+        assert ops.linear_fp8_fused(m, n, k)
+        out[f"linear_{m}_{k}_{n}"] = torch.ops.dsv3fp8.linear_fp8(x, w8, ws, _lib.SCALE_FMT_NONE, _lib.F32).cpu()
+    return out
+
+
+def test_ring_variant_equals_batch_variant(K, tmp_path):
+    """The ring variant of the M <= 16 kernel (loads and waits in inline assembly, a slot refilled as soon as it has been
+    multiplied) against the batch variant of the same kernel (compiler-scheduled loads; DSV3_SKINNY_NORING=1, read once
+    per process, hence the second process), with and without the in-kernel quantiser: bit for bit."""
+    import os, subprocess, sys
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    ring = _ring_outputs()
+    dst = tmp_path / "batch.pt"
+    code = ("import sys, torch\n"
+            f"sys.path[:0] = [{str(root)!r}, {str(root / 'deepseek-v3_amd')!r}]\n"
+            "from tests.test_gpu_fp8_gemm import _ring_outputs\n"
+            f"torch.save(_ring_outputs(), {str(dst)!r})\n")
+    env = dict(os.environ, DSV3_SKINNY_NORING="1")
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    batch = torch.load(dst, weights_only=True)
+    assert set(batch) == set(ring)
+    for key, v in ring.items():
+        assert torch.equal(v, batch[key]), key
+        assert torch.isfinite(v).all() and v.abs().max() > 0

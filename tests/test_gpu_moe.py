@@ -87,6 +87,47 @@ def test_fp8_gemm_grouped_vs_oracle(K, counts, n, k, gather):
         row += c
 
 
+@pytest.mark.parametrize("fmt", [None, "ue8m0"])
+@pytest.mark.parametrize("counts,inter,k,gather", [
+    ([128, 97, 161, 0, 300, 131, 200, 256, 3, 193], 256, 512, True),     # every tile configuration: <= 128, 129-192, > 192 rows
+    ([500], 128, 128, False),                                           # one column tile, one K block
+    ([40, 255, 130, 64], 384, 1152, True),                              # odd number of K blocks, three column tiles
+])
+def test_grouped_gemm_with_swiglu_epilogue_equals_the_two_calls(K, counts, inter, k, gather, fmt):
+    """dsv3_fp8_gemm_grouped_swiglu (silu(h1) * h3 and its act_quant in the epilogue of the w1 | w3 GEMM) against
+    dsv3_fp8_gemm_grouped followed by dsv3_swiglu_quant: bytes and scales bit for bit, including rows whose group
+    fills only part of a tile.  The two-call chain is held against the oracle elsewhere."""
+    from dsv3fp8 import ops, _lib
+    code_fmt = _lib.SCALE_FMT_UE8M0 if fmt == "ue8m0" else _lib.SCALE_FMT_NONE
+    xq, xs, w, a_rows = _grouped_case(counts, 2 * inter, k, 500 + inter, gather)
+    rows = sum(counts)
+    assert ops.grouped_swiglu_fused(rows, xq.size(0), inter, k)
+    R, tg, t0, tr = _tables(counts, rows // ops.grouped_tile_rows() + len(counts))
+    b = torch.stack([wi[0].view(torch.uint8) for wi in w]).view(FP8).cuda()
+    b_s = torch.stack([wi[1] for wi in w]).cuda()
+    args = (xq.cuda(), xs.cuda(), a_rows.cuda() if gather else None, b, b_s, rows, tg, t0, tr)
+    h = torch.ops.dsv3fp8.fp8_gemm_grouped(*args, ops.dtype_code(torch.bfloat16))
+    y2, s2 = torch.ops.dsv3fp8.swiglu_quant(h, 128, code_fmt)
+    y = torch.full((rows, inter), 0x7F, dtype=torch.uint8, device="cuda").view(FP8)     # poisoned outputs
+    y1, s1 = torch.ops.dsv3fp8.fp8_gemm_grouped_swiglu(*args, code_fmt)
+    assert y1.shape == y2.shape == (rows, inter) and s1.shape == s2.shape == (rows, inter // 128)
+    assert torch.equal(s1, s2)
+    assert torch.equal(y1.view(torch.uint8), y2.view(torch.uint8))
+    assert bool(torch.isfinite(s1).all()) and int((y1.view(torch.uint8) & 0x7F).max()) == 0x7E
+    del y
+    # few rows in all: the op falls back to the two calls (the weight-streaming kernel has no such epilogue)
+    small = [3, 0, 9]
+    xq, xs, w, _ = _grouped_case(small, 2 * inter, k, 600, False)
+    assert not ops.grouped_swiglu_fused(sum(small), xq.size(0), inter, k)
+    R, tg, t0, tr = _tables(small, len(small) + 1)
+    b = torch.stack([wi[0].view(torch.uint8) for wi in w]).view(FP8).cuda()
+    b_s = torch.stack([wi[1] for wi in w]).cuda()
+    args = (xq.cuda(), xs.cuda(), None, b, b_s, sum(small), tg, t0, tr)
+    y1, s1 = torch.ops.dsv3fp8.fp8_gemm_grouped_swiglu(*args, code_fmt)
+    y2, s2 = torch.ops.dsv3fp8.swiglu_quant(torch.ops.dsv3fp8.fp8_gemm_grouped(*args, ops.dtype_code(torch.bfloat16)), 128, code_fmt)
+    assert torch.equal(s1, s2) and torch.equal(y1.view(torch.uint8), y2.view(torch.uint8))
+
+
 def test_fp8_gemm_grouped_seeded_tables(K):
     """Twelve seeded tables mixing empty, tiny, 129-192-row, 193-256-row and multi-tile groups (every tile
     configuration of the grouped kernel, and the weight-streaming kernel when the total is small)."""
@@ -280,6 +321,9 @@ def test_moe_grouped_matches_expert_loop_and_oracle(K, tokens):
             y_grouped = moe(x.cuda())                   # 300 tokens: the shared expert rides along as group 8
             assert moe._stacked is not None and moe.experts[3].w1.weight.data_ptr() == moe._stacked[0][3].data_ptr()
             assert moe._shared_stacked and moe.shared_experts.w2.weight.data_ptr() == moe._stacked[2][8].data_ptr()
+            moe.fuse_swiglu_epilogue = True             # SwiGLU + act_quant in the first GEMM's epilogue: the same bits
+            assert torch.equal(moe(x.cuda()), y_grouped)
+            del moe.fuse_swiglu_epilogue
             moe.fold_shared_max_tokens = 0              # the shared expert as three dense linears instead
             y_unfolded = moe(x.cuda())
             del moe.fold_shared_max_tokens
