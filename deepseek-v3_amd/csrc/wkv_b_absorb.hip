@@ -368,6 +368,182 @@ __global__ __launch_bounds__(256) void absorb_v_staged_kernel(AbsorbArgs p) {
     __builtin_amdgcn_s_waitcnt(0x0f70);     // the clamped refills of the last iterations still write LDS
 }
 
+
+// Up to 256 tokens the conversion of the weight slab is the longest step of a wavefront that does it alone (a
+// 128 x 128 slab is 256 values per lane before the first MFMA can start).  The kernels below give a slab to a
+// workgroup of four wavefronts: each converts a quarter of it and leaves its MFMA operand fragments in LDS (one
+// 16-byte piece per lane and fragment, lanes in order: no bank conflicts either way), and after one barrier every
+// wavefront reads the whole slab's fragments back and takes every fourth 16-token sub-tile.  An output element is
+// still formed by one wavefront over the whole K range in the same order, so the results are those of the kernels
+// above bit for bit.
+template <int KS, int PF>
+__global__ __launch_bounds__(256) void absorb_q_shared_kernel(AbsorbArgs p) {
+    __shared__ v4u frag[KS * 8 * 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slab = blockIdx.y, h = blockIdx.x, i = lane & 15, g = lane >> 4;
+    const int c0 = slab * 128;
+    const int64_t row0 = (int64_t)h * p.head_rows;
+    const int stride = gridDim.z * 4;
+    const int ms0 = blockIdx.z * 4 + wave;
+
+    const uint16_t* xh = p.x + (int64_t)h * p.x_hs + g * 8;
+    const int64_t last = p.tokens - 1;
+    auto load_b = [&](int ms, v4u (&b)[KS]) {
+        ms = ms < p.subtiles ? ms : p.subtiles - 1;
+        int64_t tok = (int64_t)ms * 16 + i;
+        tok = tok < last ? tok : last;
+        const uint16_t* src = xh + tok * p.x_ts;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) b[s] = *(const v4u*)(src + s * 32);
+    };
+    v4u ring[PF][KS];                                      // PF sub-tiles' activations in flight, the first during the conversion
+#pragma unroll
+    for (int j = 0; j < PF; ++j) load_b(ms0 + j * stride, ring[j]);
+
+    for (int s = wave; s < KS; s += 4) {
+        const int64_t r = row0 + s * 32 + g * 8;           // 8 rows r .. r+7 lie in one scale block
+        const float sc = p.ws[(r >> 7) * p.ws_cols + slab];
+        v2u raw[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) raw[e] = *(const v2u*)(p.w + (r + e) * p.w_cols + c0 + i * 8);
+        v4u a[8];
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+            float f0[8], f1[8];
+            cvt8(raw[2 * e2], f0);
+            cvt8(raw[2 * e2 + 1], f1);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) a[t][e2] = pack_bf16(f0[t] * sc, f1[t] * sc);
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) frag[(s * 8 + t) * 64 + lane] = a[t];
+    }
+    __syncthreads();
+    if (ms0 >= p.subtiles) return;
+    v4u A[KS][8];
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) A[s][t] = frag[(s * 8 + t) * 64 + lane];
+
+    for (int base = ms0; base < p.subtiles; base += PF * stride)
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+        const int ms = base + j * stride;
+        if (ms >= p.subtiles) break;
+        v4u b[KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) b[s] = ring[j][s];
+        load_b(ms + PF * stride, ring[j]);
+        v4f acc[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc[t] = mfma_bf16(b[s], A[s][t], acc[t]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int64_t tok = (int64_t)ms * 16 + g * 4 + j;
+            tok = tok < last ? tok : last;
+            v4u o;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) o[q] = pack_bf16(acc[2 * q][j], acc[2 * q + 1][j]);
+            *(v4u*)(p.y + (tok * p.heads + h) * p.n_out + c0 + i * 8) = o;
+        }
+    }
+}
+
+// Side V for up to 256 tokens, C == 512 and v == 128: the K range, not the features, is split over the wavefronts.
+// A wavefront that owns a feature slab needs every byte of a token's 1 KiB activation row, so the four slabs of a
+// head read each row four times (through the L1 at best, through the fabric when they sit on different XCDs), in
+// scattered 16-byte pieces; with few tokens that, and a 16 KiB slab to convert per wavefront, is the whole time.
+// Here a workgroup of eight wavefronts owns a head: wavefront (kb, dh) holds K block kb (128 values) of feature
+// half dh (64 features) -- an 8 KiB slab, 64 registers of MFMA operands, half the conversion -- and reads only its
+// quarter of each activation row, so every activation byte is read by two wavefronts of one CU and no more.  The four
+// K partial sums of an output meet in LDS: every wavefront leaves its four 16 x 16 partial tiles there and, after one
+// barrier, adds up (in K order, whichever wavefront does it) the tile whose number equals its kb.  Two LDS buffers
+// alternate so that a sub-tile needs one barrier.  Feature map: MFMA row i of sub-tile t is feature
+// dh*64 + 16*(i/4) + 4*t + i%4, so the lane (token i%16, group g) that reduces tile t ends with the four consecutive
+// features dh*64 + 16*g + 4*t + [0, 4).  blockIdx.x is the head: the workgroups of a head (gridDim.z token groups)
+// have the same index mod 8 and so share one XCD's L2 for the weight.
+template <int PF>
+__global__ __launch_bounds__(512) void absorb_v_ksplit_kernel(AbsorbArgs p) {
+    __shared__ v4f part[2][8][4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int kb = wave & 3, dh = wave >> 2;
+    const int h = blockIdx.x, i = lane & 15, g = lane >> 4;
+    const int64_t row0 = (int64_t)h * p.head_rows + p.nope + dh * 64;
+    const int stride = gridDim.z;
+
+    const uint16_t* xh = p.x + (int64_t)h * p.x_hs + kb * 128 + g * 32;
+    const int64_t last = p.tokens - 1;
+    auto load_b = [&](int ms, v4u (&b)[4]) {
+        ms = ms < p.subtiles ? ms : p.subtiles - 1;
+        int64_t tok = (int64_t)ms * 16 + i;
+        tok = tok < last ? tok : last;
+        const uint16_t* src = xh + tok * p.x_ts;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) b[s] = *(const v4u*)(src + s * 8);
+    };
+    v4u ring[PF][4];                                       // PF sub-tiles' activations in flight, the first during the conversion
+#pragma unroll
+    for (int j = 0; j < PF; ++j) load_b(blockIdx.z + j * stride, ring[j]);
+
+    v4u A[4][4];
+    {
+        v4u raw[4][2];
+        float sc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int64_t r = row0 + (i >> 2) * 16 + t * 4 + (i & 3);
+            sc[t] = p.ws[(r >> 7) * p.ws_cols + kb];
+            const v4u* src = (const v4u*)(p.w + r * p.w_cols + kb * 128 + g * 32);
+            raw[t][0] = src[0];
+            raw[t][1] = src[1];
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                float f[8];
+                cvt8(v2u{raw[t][s >> 1][2 * (s & 1)], raw[t][s >> 1][2 * (s & 1) + 1]}, f);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) A[t][s][q] = pack_bf16(f[2 * q] * sc[t], f[2 * q + 1] * sc[t]);
+            }
+    }
+
+    int buf = 0;
+    for (int base = blockIdx.z; base < p.subtiles; base += PF * stride)
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+        const int ms = base + j * stride;
+        if (ms >= p.subtiles) break;                       // (the same for the whole workgroup)
+        v4u b[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) b[s] = ring[j][s];
+        load_b(ms + PF * stride, ring[j]);
+        v4f acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[t] = mfma_bf16(A[t][s], b[s], acc[t]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) part[buf][wave][t][lane] = acc[t];
+        __syncthreads();
+        // tile kb of this feature half, summed over the four K blocks in K order
+        v4f r = part[buf][dh * 4 + 0][kb][lane];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) r += part[buf][dh * 4 + w][kb][lane];
+        int64_t tok = (int64_t)ms * 16 + i;
+        tok = tok < last ? tok : last;            // clamped rows rewrite the last token's values
+        *(v2u*)(p.y + (tok * p.heads + h) * p.n_out + dh * 64 + g * 16 + kb * 4) = v2u{ pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]) };
+        buf ^= 1;
+    }
+}
+
 }  // namespace
 
 bool wkv_b_absorb_supported(int side, int nope, int v, int64_t kv_rank) {
@@ -386,6 +562,29 @@ int launch_wkv_b_absorb(const void* x, int64_t x_ts, int64_t x_hs, const void* w
     const bool q = side == DSV3_ABSORB_Q;
     p.n_out = q ? (int)kv_rank : v;
     p.slabs = q ? (int)(kv_rank / 128) : v / 32;
+    if (!q && kv_rank == 512 && v == 128 && p.subtiles >= 3 && p.subtiles <= 8) {
+        // 33 .. 128 tokens of side V: a head per workgroup, K split over its wavefronts; one workgroup per CU
+        int gz = 256 / (heads > 0 ? heads : 1);
+        gz = gz < 1 ? 1 : gz;
+        gz = gz > p.subtiles ? p.subtiles : gz;
+        hipLaunchKernelGGL(absorb_v_ksplit_kernel<1>, dim3(heads, 1, gz), dim3(512), 0, st, p);
+        return launch_status();
+    }
+    if (q && p.subtiles <= 16) {
+        // up to 256 tokens of side Q: a slab per workgroup, its sub-tiles dealt over (gridDim.z, wavefront); the
+        // head is blockIdx.x, so that the workgroups of a head share one XCD's L2
+        int gz = (p.subtiles + 3) / 4;
+        const int cap = 512 / (p.slabs * heads > 0 ? p.slabs * heads : 1);
+        gz = gz > cap ? cap : gz;
+        gz = gz < 1 ? 1 : gz;
+        const dim3 grid(heads, p.slabs, gz), block(256);
+        const bool one = (p.subtiles + 4 * gz - 1) / (4 * gz) <= 1;      // sub-tiles per wavefront
+        if (nope == 128 && one) hipLaunchKernelGGL((absorb_q_shared_kernel<4, 1>), grid, block, 0, st, p);
+        else if (nope == 128) hipLaunchKernelGGL((absorb_q_shared_kernel<4, 2>), grid, block, 0, st, p);
+        else if (one) hipLaunchKernelGGL((absorb_q_shared_kernel<2, 1>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((absorb_q_shared_kernel<2, 2>), grid, block, 0, st, p);
+        return launch_status();
+    }
     // few tokens: one wavefront per workgroup spreads the weight reads over every CU; many tokens: the wavefronts
     // of a workgroup take different slabs of the same head and share the activation reads
     const int waves = p.subtiles > 4 ? 4 : 1;

@@ -43,7 +43,7 @@ def _check(y, x, w8, s, side, nope, v):
     assert (err <= bound).all(), (err / bound).max()
 
 
-@pytest.mark.parametrize("tokens", [1, 5, 16, 17, 64, 100, 333])
+@pytest.mark.parametrize("tokens", [1, 5, 16, 17, 33, 64, 100, 128, 200, 256, 333])
 @pytest.mark.parametrize("side", [Q, V])
 def test_absorb_671b_shape(K, tokens, side):
     heads, nope, v, c = 128, 128, 128, 512
@@ -87,6 +87,9 @@ def test_absorb_dequantises_bit_exactly(K):
     eye = torch.eye(c, dtype=torch.bfloat16).unsqueeze(1).expand(c, heads, c).contiguous()
     y = _absorb(eye.cuda(), w8.cuda(), s.cuda(), V, nope, v).cpu()          # y[c, h, d] = W[h, nope + d, c]
     assert torch.equal(y.float(), wd[:, nope:, :].permute(2, 0, 1))
+    for lo, hi in ((200, 328), (0, 40)):            # 128 and 40 tokens: the kernel that splits K over its wavefronts
+        y = _absorb(eye[lo:hi].contiguous().cuda(), w8.cuda(), s.cuda(), V, nope, v).cpu()
+        assert torch.equal(y.float(), wd[:, nope:, lo:hi].permute(2, 0, 1))
 
     wn = w8.view(torch.uint8).clone().view(heads, nope + v, c)
     wn[1, 5, 7] = 0x7F
