@@ -334,6 +334,34 @@ def decode_trace(K, W, launches_per_cell: int = 60):
     print(json.dumps({"decode_trace": {"launches_per_cell": launches_per_cell, "cells": order}}), flush=True)
 
 
+def grouped_rows_sweep(K, W, rows_per_group=(16, 64, 96, 128, 160, 192, 256), launches: int = 6):
+    """For `rocprofv3 --kernel-trace` / `--pmc GRBM_GUI_ACTIVE`: the grouped GEMM at the MoE layer's w1|w3 shape
+    (256 groups, 7168 -> 4096, one weight of 29 MB per group, all streamed from HBM) with the SAME number of rows
+    in every group, one row count after the other, as plain launches.  Every group is one tile slot, so a compute
+    unit runs 16 tiles of 56 K blocks per launch and the time per K block is launch time / (16 * 56).  Prints one
+    JSON line with the launch order and HIP-event times so that the trace's rows can be cut into row counts."""
+    groups, n, k = 256, 4096, 7168
+    w8, sc = W.weight(n, k, 40, "cuda")
+    w = w8.unsqueeze(0).repeat(groups, 1, 1)                   # distinct storage per group: 7.5 GB
+    s = sc.unsqueeze(0).repeat(groups, 1, 1).contiguous()
+    from dsv3fp8 import ops as _ops
+    g = torch.ops.dsv3fp8.fp8_gemm_grouped
+    code = _ops.dtype_code(torch.bfloat16)
+    out = []
+    for r in rows_per_group:
+        m = groups * r
+        a, a_s = K.act_quant(W.activations(m, k, r, "cuda"))
+        counts = torch.full((groups,), r, dtype=torch.int32, device="cuda")
+        tg, t0, tr = torch.ops.dsv3fp8.group_tiles(counts, groups + 8)
+        fn = lambda: g(a, a_s, None, w, s, m, tg, t0, tr, code)
+        ms = time_loop(fn, launches - 2, 2)
+        out.append({"rows_per_group": r, "launches": launches, "us": round(ms * 1e3, 1),
+                    "us_per_k_block": round(ms * 1e3 / (16 * (k // 128)), 3),
+                    "weight_GBps": round(groups * n * k / ms / 1e6, 1)})
+        del a, a_s
+    print(json.dumps({"grouped_rows_sweep": {"shape": "256 groups x (rows, 7168) -> 4096", "cells": out}}), flush=True)
+
+
 def decode_roofline(dec: dict, ceil: dict) -> dict:
     """The metric's second half in one block: the decode sweep (M = 1, 8, 32, 64 over the MLA projections) as HBM
     fractions of its algorithmic bytes, against the 8 TB/s peak and against this GPU's measured read stream."""
@@ -591,6 +619,9 @@ def main():
     ap.add_argument("--decode-trace", action="store_true",
                     help="profiling aid: run only the decode sweep as plain launches (see decode_trace) and print "
                          "the cell order")
+    ap.add_argument("--grouped-rows-sweep", action="store_true",
+                    help="profiling aid: run only the grouped GEMM with equal row counts per group (see "
+                         "grouped_rows_sweep)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known HBM traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled")
@@ -607,6 +638,9 @@ def main():
     torch.cuda.set_device(0)
     if args.decode_trace:
         decode_trace(K, W)
+        return
+    if args.grouped_rows_sweep:
+        grouped_rows_sweep(K, W)
         return
     if args.only_absorb:
         if args.copy_calibration:
