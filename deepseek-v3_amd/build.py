@@ -26,11 +26,19 @@ HIPCC_FLAGS = [
 ]
 
 
-# Kernels whose weight loads and counted s_waitcnt are written as inline assembly: the compiler does not know that a
-# register named by such a load is not valid until the wait, so a spill or a copy of it in between would read the
-# register before the data has landed.  Their register budgets are sized so that nothing spills; the build fails
-# if that ever stops being true.
+# The decode kernels of these files must not use scratch memory, for two reasons.  Some of them issue their global
+# loads and count the outstanding ones by hand (inline asm global_load + s_waitcnt vmcnt(n)): the register named by
+# such a load is not valid until the wait, so a spill or a copy of it in between would read the register before the
+# data has landed.  And a kernel that uses scratch at all costs a launch about 3 us more on this hardware (measured:
+# linear() at one row 7.4 -> 10.4 us when a rewrite of the in-kernel quantiser spilled nine registers) -- as much as
+# the whole quantisation such a launch is meant to save.  The build fails if a kernel of these files reports scratch
+# or spills; the one exception is listed with its reason.
 NO_SPILL_SOURCES = {"fp8_gemm_skinny.hip", "fp8_gemm_stream.hip"}
+SCRATCH_ALLOWED = {
+    # the quantising variant with four strips per wavefront (a plan for very wide weights at one or two rows that none
+    # of the 671B projections takes): compiler-counted waits, 20 bytes per lane
+    "skinny_kernelILi1ELi4ELi2ELb1ELb0E": 24,
+}
 
 
 def check_no_spills(name: str, remarks: str) -> None:
@@ -42,11 +50,12 @@ def check_no_spills(name: str, remarks: str) -> None:
             kernel = m.group(1)
             continue
         m = re.search(r"(VGPRs Spill|SGPRs Spill|ScratchSize \[bytes/lane\]): (\d+)", line)
-        # (the M <= 16 kernel writes its loads out only in its ring variant: last template argument true)
-        hand_waited = kernel and ("stream_kernel" in kernel or re.search(r"skinny_kernelI(Li\d+E){3}Lb[01]ELb1E", kernel))
-        if m and hand_waited and int(m.group(2)) != 0:
-            raise RuntimeError(f"{name}: {kernel} reports {m.group(1)} = {m.group(2)}; the hand-counted waits of "
-                               f"this kernel require that nothing spills (lower its register use or its occupancy target)")
+        if not (m and kernel and "_kernel" in kernel):
+            continue
+        allowed = max([v for k, v in SCRATCH_ALLOWED.items() if k in kernel], default=0)
+        if int(m.group(2)) > allowed:
+            raise RuntimeError(f"{name}: {kernel} reports {m.group(1)} = {m.group(2)} (allowed: {allowed}); the decode "
+                               f"kernels must not spill (lower the kernel's register use or its occupancy target)")
 
 
 def _hipcc() -> str:

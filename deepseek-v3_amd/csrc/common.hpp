@@ -61,6 +61,11 @@ __device__ __forceinline__ v2f fp8x2_hi_to_f32(uint32_t p) { return __builtin_am
 // rounded up to a power of two for the ue8m0 format (non-finite scales pass through unchanged).
 __device__ __forceinline__ uint32_t umax_u32(uint32_t a, uint32_t b) { return a > b ? a : b; }
 __device__ __forceinline__ uint32_t abs_bits(float f) { return f32_as_u32(f) & 0x7fffffffu; }
+// unsigned maximum of the two 16-bit halves of a and b (v_pk_max_u16)
+__device__ __forceinline__ uint32_t pk_umax_u16(uint32_t a, uint32_t b) {
+    typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2us, a), __builtin_bit_cast(v2us, b)));
+}
 template <int CTRL> __device__ __forceinline__ uint32_t dpp_umax(uint32_t v) {
     return umax_u32(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true));
 }

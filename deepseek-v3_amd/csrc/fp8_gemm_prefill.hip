@@ -145,13 +145,17 @@ __device__ __forceinline__ void swiglu_store(v4f (&acc)[8][SM], uint8_t* lds, in
         // the sub-tile's 16 rows x 128 bytes pass through the part of the exchange area this wavefront has just read
         // (16-byte chunks xor-ed with the row), so that a store instruction writes 8 whole rows instead of 16-byte pieces
         uint8_t* stg = (uint8_t*)(xch + j * 8 * 64);
+        auto quantise = [&](auto fast_tag) {
+            constexpr bool FAST = decltype(fast_tag)::value;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float q[4];
+            for (int i = 0; i < 8; ++i) {
+                float q[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) q[e] = finite ? block_quotient(gv[i][e], sc, rcp, true) : block_quotient(gv[i][e], sc, rcp, false);
-            *(uint32_t*)(stg + fr * 128 + ((i ^ (fr & 7)) * 16) + fq * 4) = pack_fp8x4(q[0], q[1], q[2], q[3]);
-        }
+                for (int e = 0; e < 4; ++e) q[e] = block_quotient(gv[i][e], sc, rcp, FAST);
+                *(uint32_t*)(stg + fr * 128 + ((i ^ (fr & 7)) * 16) + fq * 4) = pack_fp8x4(q[0], q[1], q[2], q[3]);
+            }
+        };
+        if (finite) quantise(std::true_type{}); else quantise(std::false_type{});
         const int r0 = sub_row(j);
         if (fq == 0 && r0 + fr < rows_here) g.sg_s[(size_t)(m0 + r0 + fr) * (size_t)(inter / 128) + tn] = sc;
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");

@@ -188,9 +188,12 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
             // (the 16 values are widened twice, for the maximum and for the quotients, instead of being kept: with the
             // weight ring live this section must stay inside the register budget)
             auto widen = [&](int e) { return (e & 1) ? bf16hi_to_f32(raw[i][e >> 3][(e >> 1) & 3]) : bf16lo_to_f32(raw[i][e >> 3][(e >> 1) & 3]); };
-            uint32_t abits = 0u;                 // non-finite values reach the scale as in act_quant
+            // largest |x| as a bit pattern (non-finite values reach the scale as in act_quant), two bf16 patterns per
+            // instruction: the sixteen values are not widened for it
+            uint32_t m2 = 0u;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) abits = umax_u32(abits, abs_bits(widen(e)));
+            for (int e = 0; e < 8; ++e) m2 = pk_umax_u16(m2, raw[i][e >> 2][e & 3] & 0x7fff7fffu);
+            uint32_t abits = umax_u32(m2 & 0xffffu, m2 >> 16) << 16;
             abits = dpp_umax<0xB1>(abits);       // quad_perm [1,0,3,2]
             abits = dpp_umax<0x4E>(abits);       // quad_perm [2,3,0,1]
             abits = dpp_umax<0x141>(abits);      // row_half_mirror
@@ -198,11 +201,17 @@ __global__ __launch_bounds__(kMaxWaves * kWave) __attribute__((amdgpu_waves_per_
             const bool fast = block_is_finite(abits);
             const float r = 1.0f / sc;
             v4i o;
+            // x / sc, correctly rounded for bf16 x with |x| <= amax (as act_quant).  In a block with a non-finite value
+            // the quotient needs no division either: sc = inf gives r = 0 and x * 0 is the IEEE x / inf (+-0 for finite
+            // x, NaN for infinite x), sc = NaN gives NaN; only the correction step must be left out there.
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {        // x / sc, correctly rounded for bf16 x with |x| <= amax (as act_quant)
+            for (int g = 0; g < 4; ++g) {
                 float q[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) q[e] = fast ? block_quotient(widen(4 * g + e), sc, r, true) : block_quotient(widen(4 * g + e), sc, r, false);
+                for (int e = 0; e < 4; ++e) {
+                    const float x = widen(4 * g + e), q0 = x * r;
+                    q[e] = fast ? block_quotient(x, sc, r, true) : q0;
+                }
                 o[g] = (int)pack_fp8x4(q[0], q[1], q[2], q[3]);
             }
             const int c = tid + i * (int)blockDim.x;

@@ -20,9 +20,10 @@ reference checkout).  All arithmetic is IEEE binary32 on the CPU:
 Pinning (see tests/test_oracle_*.py): the conversions and all three kernels are
 checked against the independent plain-C restatement in ``dsv3_oracle.c`` and
 against closed-form known answers; ``wkv_b_absorb`` against a scalar triple loop,
-one-hot inputs that read single dequantised weights and exact integer cases; nothing here is "parity unpinned" except the
-choice among equal scores in ``gate`` (torch.topk leaves ties unspecified; the
-workloads are generated without ties).
+one-hot inputs that read single dequantised weights and exact integer cases.  "Parity unpinned": the choice among
+equal scores in ``gate`` (torch.topk leaves ties unspecified; the workloads are generated without ties), and what
+``act_quant`` does with a NaN or an infinity in a block -- this restatement follows torch's ``amax`` (the NaN reaches
+the scale, in both scale formats), and no file of the reference says whether its Triton maximum does the same.
 """
 from __future__ import annotations
 
