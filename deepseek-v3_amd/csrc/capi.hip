@@ -103,8 +103,10 @@ static int fp8_gemm_validate(const void* a, const float* a_s, const void* b, con
                              void* workspace, size_t workspace_bytes, bool check_workspace = true) {
     if (!valid_dtype(c_dtype)) return DSV3_ERR_BAD_DTYPE;
     if (m < 0 || n < 0 || k < 0) return DSV3_ERR_BAD_SHAPE;
-    if (k % 128 != 0) return DSV3_ERR_BAD_SHAPE;
     if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
+    // (K need not be a multiple of 128: the last block is then masked, as in the reference's kernel; m is a grid
+    // dimension of that fallback)
+    if (k % 128 != 0 && m > 65535) return DSV3_ERR_BAD_SHAPE;
     if (m == 0 || n == 0) return DSV3_OK;
     if (!c) return DSV3_ERR_NULL_POINTER;
     if (k > 0 && (!a || !a_s || !b || !b_s)) return DSV3_ERR_NULL_POINTER;

@@ -286,6 +286,36 @@ Plan make_plan(int64_t m, int64_t n, int64_t k) {
 // 3 to 16 rows on a weight of 96 MiB or more for which the activation-streaming kernel has no plan: the dense GEMM runs
 // as one group of the grouped weight-streaming kernel -- 32-row strips of such a weight fill the chip, one launch, no
 // partial sums in memory.
+// K not a multiple of 128 (inference/kernel.py:145, 158-159: the reference's kernel masks the last, partial K block;
+// its act_quant cannot produce such an operand, kernel.py:52, so nothing on the model's path gets here).  A plain
+// kernel for completeness, not for speed: rows of a and b are not 16-byte aligned then, so everything is read bytewise.
+// One thread per output element; a workgroup owns one row of a and 256 columns, stages the row's K block in LDS as
+// binary32 and walks the K blocks in the reference's order: (dot * a_s) * b_s, accumulated in binary32.  The scale
+// tensors have ceil(K / 128) columns.
+template <int CD>
+__global__ __launch_bounds__(256) void fp8_gemm_any_k_kernel(
+        const uint8_t* __restrict__ a, const float* __restrict__ a_s,
+        const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+        typename OutT<CD>::type* __restrict__ c, int M, int N, int K) {
+    __shared__ float arow[128];
+    const int m = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
+    const int KB = (K + 127) / 128;
+    const uint8_t* brow = b + (size_t)min(n, N - 1) * K;
+    float acc = 0.f;
+    for (int kb = 0; kb < KB; ++kb) {
+        const int len = min(128, K - kb * 128);
+        __syncthreads();
+        if ((int)threadIdx.x < len)
+            arow[threadIdx.x] = __builtin_amdgcn_cvt_f32_fp8((int)a[(size_t)m * K + kb * 128 + threadIdx.x], 0);
+        __syncthreads();
+        float dot = 0.f;
+        for (int t = 0; t < len; ++t)
+            dot = __builtin_fmaf(arow[t], __builtin_amdgcn_cvt_f32_fp8((int)brow[kb * 128 + t], 0), dot);
+        acc += (dot * a_s[(size_t)m * KB + kb]) * b_s[(size_t)(min(n, N - 1) / 128) * KB + kb];
+    }
+    if (n < N) c[(size_t)m * N + n] = cvt_out<CD>(acc);
+}
+
 bool single_group_stream(int64_t m, int64_t n, int64_t k) {
     if (m < 3 || m > 16 || n * k < (96ll << 20) || !skinny_single_supported(m, n, k)) return false;
     // wherever the activation-streaming kernel has a plan it is faster (16384 -> 7168 at 4 / 8 / 16 rows: 22.2 / 22.5 /
@@ -328,6 +358,11 @@ int launch_typed(const void* a, const float* a_s, const void* b, const float* b_
         const int64_t mn0 = m * n;
         hipLaunchKernelGGL((splitk_reduce_kernel<CD>), dim3(splitk_reduce_grid(mn0)), dim3(256), 0, st,
                            (const float*)nullptr, (typename OutT<CD>::type*)c, mn0, 0);
+        return launch_status();
+    }
+    if (k % 128 != 0) {
+        hipLaunchKernelGGL((fp8_gemm_any_k_kernel<CD>), dim3((unsigned)((n + 255) / 256), (unsigned)m), dim3(256), 0, st,
+                           (const uint8_t*)a, a_s, (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k);
         return launch_status();
     }
     const int force = forced_kernel();

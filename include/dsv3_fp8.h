@@ -134,11 +134,12 @@ int dsv3_weight_quant(const void* w, int w_dtype, void* y, float* s,
  * fp8_gemm (inference/kernel.py:145-172):
  *     c[i,j] = c_dtype( sum_kb ( sum_{t<128} a[i,128kb+t] * b[j,128kb+t] )
  *                                * a_s[i,kb] * b_s[j/128,kb] )
- * a: [m,k] fp8, a_s: [m,k/128] binary32, b: [n,k] fp8 (the weight, out x in),
- * b_s: [ceil(n/128), k/128] binary32, c: [m,n] of c_dtype.  Products and sums
+ * a: [m,k] fp8, a_s: [m,ceil(k/128)] binary32, b: [n,k] fp8 (the weight, out x in),
+ * b_s: [ceil(n/128), ceil(k/128)] binary32, c: [m,n] of c_dtype.  Products and sums
  * are binary32; the order of additions differs from the reference's.
- * k must be a multiple of 128 (guaranteed by act_quant, inference/kernel.py:52);
- * any m, n >= 0.  a and b must be 16-byte aligned.
+ * Any m, n >= 0.  a and b must be 16-byte aligned.  The kernels are written for k a multiple of 128, which is what
+ * act_quant produces (inference/kernel.py:52); any other k runs a plain fallback kernel that masks the last,
+ * partial block as the reference's kernel does (kernel.py:145, 158-159; m <= 65535 there, no workspace).
  * `workspace` must hold at least dsv3_fp8_gemm_workspace_bytes(m,n,k) bytes
  * (256-byte aligned) when that is non-zero; its contents on entry are ignored
  * and are undefined on return.  Calls sharing a workspace must be ordered on

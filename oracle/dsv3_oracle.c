@@ -134,14 +134,14 @@ void oracle_weight_dequant(const uint8_t* x, const float* s, uint16_t* y,
  * binary32 and a double holds the sum of 128 of them without rounding); the
  * per-block result is rounded to binary32 once, scaled in binary32 in the
  * reference's order (dot*a_s)*b_s and accumulated in binary32.
- * a: [m,k] bytes, b: [n,k] bytes, a_s: [m,k/128], b_s: [ceil(n/128), k/128],
+ * a: [m,k] bytes, b: [n,k] bytes, a_s: [m,ceil(k/128)], b_s: [ceil(n/128), ceil(k/128)],
  * c32: [m,n] binary32, c16: [m,n] bf16 bits (either may be NULL).
  */
 void oracle_fp8_gemm(const uint8_t* a, const float* a_s, const uint8_t* b, const float* b_s,
                      float* c32, uint16_t* c16, int64_t m, int64_t n, int64_t k) {
     float lut[256];
     for (int i = 0; i < 256; ++i) lut[i] = oracle_e4m3_to_f32((uint8_t)i);
-    int64_t kb_n = k / 128;
+    int64_t kb_n = (k + 127) / 128;           /* a last block of fewer than 128 values is masked (kernel.py:145, 158-159) */
     for (int64_t i = 0; i < m; ++i)
         for (int64_t j = 0; j < n; ++j) {
             float acc = 0.f;
@@ -149,7 +149,8 @@ void oracle_fp8_gemm(const uint8_t* a, const float* a_s, const uint8_t* b, const
                 double dot = 0.0;
                 const uint8_t* ap = a + i * k + kb * 128;
                 const uint8_t* bp = b + j * k + kb * 128;
-                for (int t = 0; t < 128; ++t) dot += (double)lut[ap[t]] * (double)lut[bp[t]];
+                const int len = (int)(k - kb * 128 < 128 ? k - kb * 128 : 128);
+                for (int t = 0; t < len; ++t) dot += (double)lut[ap[t]] * (double)lut[bp[t]];
                 volatile float d = (float)dot;
                 volatile float d1 = d * a_s[i * kb_n + kb];
                 volatile float d2 = d1 * b_s[(j / 128) * kb_n + kb];

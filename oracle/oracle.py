@@ -88,14 +88,15 @@ def fp8_gemm_f32(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch
     k = a.size(-1)
     m = a.numel() // k
     n = b.size(0)
-    assert k % BLOCK == 0
     af = a.reshape(m, k).float()
     bf = b.float()
     asf = a_s.reshape(m, -1).float()
     nb = torch.arange(n) // BLOCK
     acc = torch.zeros(m, n, dtype=torch.float32)
-    for kb in range(k // BLOCK):
-        sl = slice(kb * BLOCK, (kb + 1) * BLOCK)
+    # a last block of fewer than 128 values is masked, i.e. zero-filled (kernel.py:145, 158-159): its scales are
+    # column ceil(k / 128) - 1 of both scale tensors
+    for kb in range(-(-k // BLOCK)):
+        sl = slice(kb * BLOCK, min((kb + 1) * BLOCK, k))
         dot = af[:, sl] @ bf[:, sl].t()
         acc += dot * asf[:, kb, None] * b_s[nb, kb][None, :]
     return acc.view(*a.shape[:-1], n)

@@ -84,7 +84,7 @@ def test_fp8_gemm_validation(L, entry):
     ws = L.lib.dsv3_fp8_gemm_workspace_bytes
     assert f(None, A16, A16, A16, A16, L.BF16, 4, 128, 128, None, 0, None) == 1
     assert f(A16, A16, A16, A16, None, L.BF16, 4, 128, 128, None, 0, None) == 1
-    assert f(A16, A16, A16, A16, A16, L.BF16, 4, 128, 100, None, 0, None) == 2    # K % 128
+    assert f(A16, A16, A16, A16, A16, L.BF16, 70000, 128, 100, None, 0, None) == 2    # K % 128 != 0 is served by a fallback whose grid takes m <= 65535
     assert f(A16, A16, A16, A16, A16, L.BF16, -4, 128, 128, None, 0, None) == 2
     assert f(A16 + 8, A16, A16, A16, A16, L.BF16, 4, 128, 128, None, 0, None) == 4
     assert f(A16, A16, A16, A16, A16, 3, 4, 128, 128, None, 0, None) == 5
@@ -106,7 +106,7 @@ def test_fp8_gemm_static_reports_argument_errors_before_the_size_limit(L):
     assert f(A16, A16, A16, A16, A16, 3, *big, None) == 5                 # bad dtype code
     assert f(None, A16, A16, A16, A16, L.BF16, *big, None) == 1
     assert f(A16 + 8, A16, A16, A16, A16, L.BF16, *big, None) == 4
-    assert f(A16, A16, A16, A16, A16, L.BF16, 9, 129280, 7168 + 64, None) == 2   # K % 128
+    assert f(A16, A16, A16, A16, A16, L.BF16, 70000, 129280, 7168 + 64, None) == 2   # K % 128 != 0 with more rows than its fallback takes
     assert f(A16, A16, A16, A16, A16, L.BF16, -9, 129280, 7168, None) == 2
     assert f(None, None, None, None, None, L.BF16, 0, 129280, 7168, None) == 0   # nothing to do
 

@@ -127,6 +127,31 @@ def test_ragged_n(K, n):
         _check(K, x, w8, ws)
 
 
+@pytest.mark.parametrize("mnk", [(3, 5, 1), (2, 130, 127), (4, 7, 129), (70, 200, 300), (1, 576, 7168 + 64),
+                                 (5, 1000, 200)])
+def test_k_not_a_multiple_of_128(K, mnk):
+    """The reference's kernel masks a last, partial K block (inference/kernel.py:145, 158-159; its act_quant cannot
+    produce one, kernel.py:52): scale tensors of ceil(k / 128) columns, the tail zero-filled.  Against the oracle, and
+    against the same problem padded with zero bytes to the next multiple of 128, which runs the regular kernels."""
+    m, n, k = mnk
+    g = torch.Generator().manual_seed(k)
+    kb = -(-k // 128)
+    a = torch.randn(m, k, generator=g).to(torch.float8_e4m3fn)
+    b = (torch.randn(n, k, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    a_s = torch.rand(m, kb, generator=g) * 0.1 + 0.01
+    b_s = torch.rand(-(-n // 128), kb, generator=g) * 0.1 + 0.01
+    ref = oracle.fp8_gemm_f32(a, a_s, b, b_s)
+    c32, c16 = _gemm_both(K, a.cuda(), a_s.cuda(), b.cuda(), b_s.cuda())
+    rms = ref.pow(2).mean().sqrt().item()
+    assert (c32.cpu() - ref).abs().max().item() <= TOL * rms
+    assert torch.equal(c16.cpu().view(torch.int16), c32.cpu().to(torch.bfloat16).view(torch.int16))
+    kp = kb * 128
+    ap = torch.zeros(m, kp, dtype=torch.uint8); ap[:, :k] = a.view(torch.uint8)
+    bp = torch.zeros(n, kp, dtype=torch.uint8); bp[:, :k] = b.view(torch.uint8)
+    padded = K.fp8_gemm_f32(ap.view(torch.float8_e4m3fn).cuda(), a_s.cuda(), bp.view(torch.float8_e4m3fn).cuda(), b_s.cuda())
+    assert (c32 - padded).abs().max().item() <= 1e-3 * rms          # two binary32 summation orders of the same products
+
+
 def test_ragged_n_equals_prefix_of_padded(K):
     """N=576 must equal the first 576 columns of the N=640 problem built from the same rows."""
     from dsv3fp8 import workloads

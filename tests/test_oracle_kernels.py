@@ -259,6 +259,47 @@ def test_fp8_gemm_ragged_n_is_a_prefix():
     assert torch.equal(full[:, :576], part)
 
 
+def _ragged_k_problem(m, n, k, seed):
+    """fp8 operands with a K that is not a multiple of 128 and scale tensors of ceil(k / 128) columns (act_quant cannot
+    produce such a pair, kernel.py:52; fp8_gemm's own kernel masks the tail, kernel.py:145, 158-159)."""
+    g = torch.Generator().manual_seed(seed)
+    kb = -(-k // 128)
+    a = torch.randn(m, k, generator=g).to(FP8)
+    b = (torch.randn(n, k, generator=g) * 0.5).to(FP8)
+    a_s = torch.rand(m, kb, generator=g) * 0.1 + 0.01
+    b_s = torch.rand(-(-n // 128), kb, generator=g) * 0.1 + 0.01
+    return a, a_s, b, b_s
+
+
+@pytest.mark.parametrize("mnk", [(3, 5, 1), (2, 130, 127), (4, 7, 129), (3, 200, 300), (1, 16, 7168 + 64)])
+def test_fp8_gemm_masked_k_tail_equals_zero_padding(coracle, mnk):
+    """A masked tail is a zero-filled tail: the result must equal, bit for bit, that of the operands padded with zero
+    bytes to the next multiple of 128 (same scales) -- in the torch restatement and in the C one."""
+    m, n, k = mnk
+    a, a_s, b, b_s = _ragged_k_problem(m, n, k, seed=k)
+    kp = -(-k // 128) * 128
+    ap = torch.zeros(m, kp, dtype=torch.uint8); ap[:, :k] = a.view(torch.uint8)
+    bp = torch.zeros(n, kp, dtype=torch.uint8); bp[:, :k] = b.view(torch.uint8)
+    got = oracle.fp8_gemm_f32(a, a_s, b, b_s)
+    assert torch.equal(got, oracle.fp8_gemm_f32(ap.view(FP8), a_s, bp.view(FP8), b_s))
+    c32, _ = c_fp8_gemm(coracle, a, a_s, b, b_s)
+    c32p, _ = c_fp8_gemm(coracle, ap.view(FP8), a_s, bp.view(FP8), b_s)
+    assert torch.equal(c32, c32p)
+    rms = c32.pow(2).mean().sqrt()
+    assert (got - c32).abs().max() <= 2e-6 * rms + 1e-30
+
+
+def test_fp8_gemm_masked_k_tail_brute_force():
+    a, a_s, b, b_s = _ragged_k_problem(2, 3, 200, seed=2)
+    ref = oracle.fp8_gemm_f32(a, a_s, b, b_s).double()
+    af, bf = a.double(), b.double()
+    for i in range(2):
+        for j in range(3):
+            acc = sum(af[i, t].item() * bf[j, t].item() for t in range(128)) * a_s[i, 0].item() * b_s[0, 0].item()
+            acc += sum(af[i, t].item() * bf[j, t].item() for t in range(128, 200)) * a_s[i, 1].item() * b_s[0, 1].item()
+            assert abs(ref[i, j].item() - acc) <= 1e-5 * max(1.0, abs(acc))
+
+
 def test_fp8_gemm_close_to_unquantised_product():
     g = torch.Generator().manual_seed(6)
     x = torch.randn(8, 1024, generator=g).bfloat16()
