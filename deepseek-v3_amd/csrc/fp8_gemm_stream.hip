@@ -5,7 +5,7 @@
 // 128-row block of weight scales; a workgroup's strips may lie in two) and walk
 // the workgroup's K range; their weights go straight from global memory into the MFMA register layout through a
 // ring of NPF K blocks whose loads and waits are written out explicitly (inline asm), so that exactly NPF-1
-// blocks stay in flight behind the one being multiplied.  The fifth wavefront is the PRODUCER: it copies the
+// blocks stay in flight behind the one being multiplied.  One more wavefront is the PRODUCER: it copies the
 // activations the consumers share (chunks of KC K blocks x 16*MT rows, plus their scales and the weight scales of
 // those K blocks) into a ring of LDS buffers with global_load_lds, AHEAD chunks ahead of the one the consumers
 // read, so that a chunk's trip from L2 is hidden behind the chunks before it (with one chunk in flight at a time
@@ -24,7 +24,7 @@ namespace stream {
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-constexpr int kMaxConsumers = 8;          // consumer wavefronts per workgroup: 4 or 8, chosen per launch (blockDim.x / 64 - 1)
+constexpr int kMaxConsumers = 8;          // consumer wavefronts per workgroup: 2 .. 8, chosen per launch (blockDim.x / 64 - 1)
 constexpr int kThreads = (kMaxConsumers + 1) * kWave;
 
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }

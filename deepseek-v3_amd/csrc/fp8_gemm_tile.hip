@@ -283,9 +283,6 @@ Plan make_plan(int64_t m, int64_t n, int64_t k) {
     return p;
 }
 
-// 3 to 16 rows on a weight of 96 MiB or more for which the activation-streaming kernel has no plan: the dense GEMM runs
-// as one group of the grouped weight-streaming kernel -- 32-row strips of such a weight fill the chip, one launch, no
-// partial sums in memory.
 // K not a multiple of 128 (inference/kernel.py:145, 158-159: the reference's kernel masks the last, partial K block;
 // its act_quant cannot produce such an operand, kernel.py:52, so nothing on the model's path gets here).  A plain
 // kernel for completeness, not for speed: rows of a and b are not 16-byte aligned then, so everything is read bytewise.
@@ -316,6 +313,9 @@ __global__ __launch_bounds__(256) void fp8_gemm_any_k_kernel(
     if (n < N) c[(size_t)m * N + n] = cvt_out<CD>(acc);
 }
 
+// 3 to 16 rows on a weight of 96 MiB or more for which the activation-streaming kernel has no plan: the dense GEMM runs
+// as one group of the grouped weight-streaming kernel -- 32-row strips of such a weight fill the chip, one launch, no
+// partial sums in memory.
 bool single_group_stream(int64_t m, int64_t n, int64_t k) {
     if (m < 3 || m > 16 || n * k < (96ll << 20) || !skinny_single_supported(m, n, k)) return false;
     // wherever the activation-streaming kernel has a plan it is faster (16384 -> 7168 at 4 / 8 / 16 rows: 22.2 / 22.5 /
