@@ -64,6 +64,7 @@ template <int SM> struct Geo {
 constexpr int SC_SLOT = 2048, SC_SLOTS = 2;
 template <int SM> constexpr int lds_bytes() { return Geo<SM>::LDS_SC + SC_SLOTS * SC_SLOT; }
 constexpr int LDS_BYTES = lds_bytes<4>();               // 136 KiB (100 KiB for the 128-row tile)
+constexpr int LDS_BYTES_SCB = LDS_BYTES + 3 * 4096;     // with scale batches: two buffers and the area of the copies nobody reads
 
 // PS (persistent): the workgroup computes tiles wg, wg + wg_stride, ... one after the other and treats their K blocks
 // as one stream -- the last two blocks of a tile request the first copies of the next tile where a single tile
@@ -75,7 +76,8 @@ constexpr int LDS_BYTES = lds_bytes<4>();               // 136 KiB (100 KiB for 
 // results; the caller sends everything else down the one-tile path.
 constexpr int PS_STAGING = 8 * 2048;
 
-template <int CD, bool P2, bool G = false, int SM = 4, bool PS = false, bool SG = false>
+// SCB (grouped mode): the activation scales are copied four K blocks at a time, see issue_scales.
+template <int CD, bool P2, bool G = false, int SM = 4, bool PS = false, bool SG = false, bool SCB = false>
 __device__ __forceinline__ void tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -223,7 +225,26 @@ __device__ __forceinline__ void tile(
     const int b_scale_row = SG ? sg_scale_row(wave == 4 ? min(lane, 1) : 0, tn_idx, N / 2)
                                : min((PS ? 0 : n0 / 128) + (wave == 4 ? min(lane, 1) : 0), nb_last);
     const uint32_t sc_off = (wave < 4 ? a_row(wave * 64 + lane) * (uint32_t)KBT : (uint32_t)b_scale_row * (uint32_t)KBT) + (uint32_t)kb0;
+    // Grouped mode streams its weights from HBM, and there the 256 lines per K block of the activation scales cost a
+    // tenth of a 256-row slot's time (with one line per copy, results aside: 2.24 -> 2.00 us per K block).  When a row
+    // of a_s is a whole number of 16-byte pieces, wavefronts 0-3 therefore copy the scales of FOUR K blocks at a time
+    // (16 bytes per row, into one of two 4 KiB buffers behind the slots) in the block that would have requested the
+    // first of them, and a one-line copy nobody reads in the other three, which keeps the counted waits as they are.
+    // (sc_one_line: a 16-byte aligned address of a_s that every lane may read.)
+    constexpr int LDS_SCB = LDS_SC + SC_SLOTS * SC_SLOT, SCB_BYTES = 256 * 16;
+    constexpr bool batched = SCB;                       // (the caller has checked: KBT % 4 == 0, a_s 16-byte aligned)
+    static_assert(!SCB || (G && !PS), "scale batches: grouped mode");
+    const uint32_t sc_one_line = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc_off);
     auto issue_scales = [&](int kb, int slot, bool tail = true) {
+        if constexpr (batched) if (wave < 4) {
+            // (no branch: one in the middle of a phase splits the region the phases' instruction order is pinned in, and
+            // the register allocation with it.  The copy that is not needed reads one line and lands in a dump area.)
+            const bool real = (kb & 3) == 0;
+            const uint32_t off = real ? sc_off * 4u : sc_one_line * 4u;
+            const uint32_t dst = lds_addr_of(lds + LDS_SCB) + (real ? ((kb >> 2) & 1) * SCB_BYTES : 2 * SCB_BYTES) + wave * 1024;
+            copy16(sc_base + (uint32_t)(real ? kb : 0), off, dst);
+            return;
+        }
         if constexpr (PS) {
             const bool nx = tail && kb >= KB;
             copy4((nx ? nxt.sc : cur.sc) + (uint32_t)(nx ? kb - KB : kb), sc_off * 4u, lds_addr_of(lds + LDS_SC + slot * SC_SLOT + wave * 256));
@@ -237,6 +258,7 @@ __device__ __forceinline__ void tile(
     const uint8_t* a_rd = lds + LDS_A + (wm * WM + fr) * 128;           // + j * 2048 + stage * A_STAGE
     const uint8_t* b_rd = lds + LDS_B + (grp * 128 + fr) * 128;         // + i * 2048 + stage * B_STAGE
     const uint8_t* sa_rd = lds + LDS_SC + (wm * WM + fr) * 4;           // + j * 64 + slot * SC_SLOT
+    const uint8_t* sab_rd = lds + LDS_SCB + (wm * WM + fr) * 16;        // (batched) + j * 256 + buffer + 4 (kb & 3)
     const uint8_t* sb_rd = lds + LDS_SC + (256 + grp) * 4;
 
     v4f acc[8][SM];
@@ -374,9 +396,12 @@ __device__ __forceinline__ void tile(
             }
             {
                 const float bs = *(const float*)(sb_rd + ST * SC_SLOT);
+                const uint8_t* sab_kb = sab_rd + (((kb >> 2) & 1) * SCB_BYTES + (kb & 3) * 4);
 #pragma unroll
                 for (int j = 0; j < SM; ++j) {
-                    const float as = *(const float*)(sa_rd + j * 64 + ST * SC_SLOT);
+                    float as;
+                    if constexpr (batched) as = *(const float*)(sab_kb + j * 256);
+                    else as = *(const float*)(sa_rd + j * 64 + ST * SC_SLOT);
                     if (P2) ea[j] = (int)(f32_as_u32(as) >> 23);
                     else sc[ST][j] = as * bs;
                 }

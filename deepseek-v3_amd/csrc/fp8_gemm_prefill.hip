@@ -709,7 +709,10 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 // straight from HBM, and a second block of prefetch is what hides that), one with fewer the 128-row
 // configuration with three stages of both.  The choice is uniform over the workgroup and needs no host knowledge of
 // the group sizes: a layer with a few rows per expert and one with hundreds go through the same launch.
-template <int CD, bool P2 = false, bool SG = false>
+// SCB: a row of a_s is a whole number of 16-byte pieces (K a multiple of 512, a_s 16-byte aligned), so that the slots of
+// more than 192 rows copy their activation scales four K blocks at a time (the smaller slots keep one line per row and
+// K block: with the batch addresses their configurations no longer fit the register file).
+template <int CD, bool P2 = false, bool SG = false, bool SCB = false>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -720,7 +723,7 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
     const int rows = g.tile_rows[tm];
     if (rows > 192) {
         if (g.tile_group[tm] < 0) return;
-        pingpong::tile<CD, P2, true, 4, false, SG>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x, g);
+        pingpong::tile<CD, P2, true, 4, false, SG, SCB>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x, g);
     }
     else if (rows > 128)
         prefill_tile<CD, true, 192, 2, 3, P2, SG>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
@@ -810,6 +813,8 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
     return launch_status();
 }
 constexpr int kGroupedTileRows = 256;     // slot height of the grouped kernel's tile table
+// whether a row of a_s (K / 128 binary32 values) is a whole number of aligned 16-byte pieces
+inline bool scale_batches_ok(const float* a_s, int64_t k) { return (k / 128) % 4 == 0 && ((uintptr_t)a_s & 15) == 0; }
 constexpr int64_t kCUs = 256;
 inline int env_tile_rows() { static const int v = [] { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }(); return v; }
 }  // namespace
@@ -1047,18 +1052,21 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
                                      b_stride, bs_stride, m < num_tiles ? m : num_tiles, stream);
     GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride, nullptr, nullptr, 0};
     constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES;               // the largest of the three configurations
-    static_assert(LDS_BYTES >= pingpong::LDS_BYTES && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES, "LDS of the grouped kernel");
+    static_assert(LDS_BYTES >= pingpong::LDS_BYTES_SCB && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES, "LDS of the grouped kernel");
     const int64_t tn = (n + BN - 1) / BN;
     if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (num_tiles * tn == 0) return DSV3_OK;
-    auto kern = fp8_gemm_grouped_kernel<CD, P2>;
-    static LdsGrant grant;
-    if (!grant.ensure((const void*)kern, LDS_BYTES)) return DSV3_ERR_LAUNCH;
     const int64_t grid = (num_tiles + 7) / 8 * 8 * tn;                  // row tiles are dealt over the 8 XCDs
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
-                       (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)num_tiles,
-                       (int)tn, 0, (int)(k / 128), (int)n, g);
-    return launch_status();
+    auto launch = [&](auto kern, LdsGrant& grant) {
+        if (!grant.ensure((const void*)kern, LDS_BYTES)) return (int)DSV3_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
+                           (const uint8_t*)b, b_s, (typename OutT<CD>::type*)c, (int)m, (int)n, (int)k, (int)num_tiles,
+                           (int)tn, 0, (int)(k / 128), (int)n, g);
+        return launch_status();
+    };
+    static LdsGrant grant, grant_scb;
+    if (scale_batches_ok(a_s, k)) return launch(fp8_gemm_grouped_kernel<CD, P2, false, true>, grant_scb);
+    return launch(fp8_gemm_grouped_kernel<CD, P2>, grant);
 }
 
 // The first GEMM of a SwiGLU block with the activation and the re-quantisation in its epilogue (SwiGLU mode above): b
@@ -1081,14 +1089,17 @@ int launch_grouped_swiglu(const void* a, const float* a_s, const int* a_rows, co
     const int64_t tn = inter / 128;
     if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (num_tiles * tn == 0) return DSV3_OK;
-    auto kern = fp8_gemm_grouped_kernel<DSV3_BF16, false, true>;
-    static LdsGrant grant;
-    if (!grant.ensure((const void*)kern, LDS_BYTES)) return DSV3_ERR_LAUNCH;
     const int64_t grid = (num_tiles + 7) / 8 * 8 * tn;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
-                       (const uint8_t*)b, b_s, (uint16_t*)nullptr, (int)m, (int)(2 * inter), (int)k, (int)num_tiles,
-                       (int)tn, 0, (int)(k / 128), (int)(2 * inter), g);
-    return launch_status();
+    auto launch = [&](auto kern, LdsGrant& grant) {
+        if (!grant.ensure((const void*)kern, LDS_BYTES)) return (int)DSV3_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, stream, (const uint8_t*)a, a_s,
+                           (const uint8_t*)b, b_s, (uint16_t*)nullptr, (int)m, (int)(2 * inter), (int)k, (int)num_tiles,
+                           (int)tn, 0, (int)(k / 128), (int)(2 * inter), g);
+        return launch_status();
+    };
+    static LdsGrant grant, grant_scb;
+    if (scale_batches_ok(a_s, k)) return launch(fp8_gemm_grouped_kernel<DSV3_BF16, false, true, true>, grant_scb);
+    return launch(fp8_gemm_grouped_kernel<DSV3_BF16, false, true>, grant);
 }
 
 #define DSV3_INST(CD) \

@@ -57,6 +57,7 @@ def _grouped_case(counts, n, k, seed, gather):
     ([129, 64], 576, 256, False),            # ragged n: 576 = 2 tiles + 64, 5 scale rows
     ([40] * 6, 256, 1152, True),             # odd number of K blocks
     ([145, 177, 200, 241, 17], 512, 384, True),   # 256-row slots with 10, 12, 13 and 16 live sub-tiles, then a small one
+    ([300, 7, 250, 193], 256, 1536, True),   # 256-row slots, 12 K blocks: activation scales in three batches of four blocks
     ([1] * 9, 4096, 7168, True),             # one token of the MoE layer: the weight-streaming kernel (up to 320 rows in all)
     ([2, 0, 1, 5, 0, 3], 7168, 2048, False), # ... its second GEMM shape, ragged group sizes, no gather
     ([20, 3, 13], 200, 640, True),           # ... a slot of more than 16 rows (two passes), n not a multiple of 32
@@ -85,6 +86,25 @@ def test_fp8_gemm_grouped_vs_oracle(K, counts, n, k, gather):
         err = (out32[row:row + c].cpu() - ref).abs().max().item()
         assert err <= 1e-2 * ref.pow(2).mean().sqrt().item(), (gi, err)     # tolerance of the fp32 output
         row += c
+
+
+def test_fp8_gemm_grouped_scale_batches_need_aligned_scales(K):
+    """A row of a_s that is a whole number of 16-byte pieces lets the 256-row slots copy the scales of four K blocks
+    at a time; the same a_s four bytes further on in memory takes the one-line copies.  Same bits either way."""
+    from dsv3fp8 import ops
+    counts, n, k = [300, 250, 40], 256, 1024
+    xq, xs, w, a_rows = _grouped_case(counts, n, k, 13, True)
+    rows = sum(counts)
+    R, tg, t0, tr = _tables(counts, rows // ops.grouped_tile_rows() + len(counts))
+    b = torch.stack([wi[0].view(torch.uint8) for wi in w]).view(FP8).cuda()
+    b_s = torch.stack([wi[1] for wi in w]).cuda()
+    xs_al = xs.cuda()
+    xs_off = torch.empty(xs.numel() + 1, dtype=torch.float32, device="cuda")[1:].view_as(xs)
+    xs_off.copy_(xs_al)
+    assert xs_al.data_ptr() % 16 == 0 and xs_off.data_ptr() % 16 == 4
+    outs = [torch.ops.dsv3fp8.fp8_gemm_grouped(xq.cuda(), s, a_rows.cuda(), b, b_s, rows, tg, t0, tr,
+                                               ops.dtype_code(torch.float32)) for s in (xs_al, xs_off)]
+    assert torch.equal(outs[0], outs[1])
 
 
 @pytest.mark.parametrize("fmt", [None, "ue8m0"])
