@@ -44,7 +44,11 @@ template <int TM, int S, int SB = S> struct Cfg {                    // S: activ
     static constexpr int LDS_A = 0, LDS_B = S * A_STAGE;              // [A stages | B stages | scale slots]
     static constexpr int LDS_SC = S * A_STAGE + SB * B_STAGE;
     static constexpr int LDS_BYTES = LDS_SC + SS * SC_STAGE;
-    static_assert(LDS_BYTES <= 160 * 1024, "LDS of a gfx950 compute unit");
+    // grouped mode with scale batches (SCB) keeps, in place of the slots, two buffers of the scales of four K blocks --
+    // 16 bytes per tile row, then the 64 x 16 bytes that wavefront 4 copies (lanes 0 and 1: b_s) -- and 1 KiB that
+    // takes the copies nobody reads
+    static constexpr int SCB_BUF = TM * 16 + 1024, LDS_DUMP = LDS_SC + 2 * SCB_BUF, LDS_BYTES_SCB = LDS_DUMP + 1024;
+    static_assert(LDS_BYTES <= 160 * 1024 && LDS_BYTES_SCB <= 160 * 1024, "LDS of a gfx950 compute unit");
     static_assert(SB >= S, "the weights are the operand that comes from HBM");
 };
 
@@ -173,7 +177,9 @@ __device__ __forceinline__ void swiglu_store(v4f (&acc)[8][SM], uint8_t* lds, in
 // P2: every scale is a power of two (act_quant's ue8m0 format and checkpoints whose block scales are stored that
 // way).  The block scales then ride in the MFMA's E8M0 scale operands and the products of all K blocks accumulate
 // inside the matrix core: no fold, no vector-ALU work in the K loop.
-template <int CD, bool G, int TM, int S, int SB = S, bool P2 = false, bool SG = false>
+// SCB (grouped mode; K a multiple of 512, a_s and b_s 16-byte aligned): the scales are copied four K blocks at a time,
+// see issue_scales.
+template <int CD, bool G, int TM, int S, int SB = S, bool P2 = false, bool SG = false, bool SCB = false>
 __device__ __forceinline__ void prefill_tile(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
         const uint8_t* __restrict__ b, const float* __restrict__ b_s,
@@ -304,12 +310,35 @@ __device__ __forceinline__ void prefill_tile(
     const int b_scale_row = SG ? sg_scale_row(wave == 4 ? min(lane, 1) : 0, tn_idx, N / 2)
                                : min(n0 / 128 + (wave == 4 ? min(lane, 1) : 0), nb_last);
     const uint32_t sc_off = (wave < 4 ? a_scale_row * (uint32_t)KBT : (uint32_t)b_scale_row * (uint32_t)KBT) + (uint32_t)kb0;
+    // SCB.  A group's weights stream from HBM, and there the lines of the activation scales -- one per row and K block,
+    // 4 bytes used of each -- cost 6 % of a 128-row slot's time.  With SCB every wavefront copies 16 bytes per lane, the
+    // scales of FOUR K blocks, into one of two buffers in the block that would have requested the first of them, and one
+    // line that nobody reads (sc_one_line: a 16-byte aligned address every lane may read) in the other three, which
+    // keeps the counted waits as they are.  No branch on the block number or the wavefront: the addresses are selected
+    // (a branch in the middle of a block splits the region its instruction order is pinned in, and that costs spills).
+    static_assert(!SCB || G, "scale batches: grouped mode");
+    constexpr int SCB_BUF = C::SCB_BUF, LDS_DUMP = C::LDS_DUMP;
+    const bool sc_live = wave < TM / 64 || wave == 4;
+    const int sc_dst = LDS_SC + (wave < TM / 64 ? wave * 1024 : TM * 16);
+    const uint32_t sc_one_line = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc_off);
     auto issue_scales = [&](int kb, int stage) {
-        __builtin_amdgcn_global_load_lds((gptr_t)(sc_base + sc_off + (uint32_t)kb),
-                                         (lptr_t)(lds + LDS_SC + stage * SC_STAGE + wave * 256), 4, 0, 0);
+        if constexpr (SCB) {
+            const bool real = sc_live && (kb & 3) == 0;
+            __builtin_amdgcn_global_load_lds((gptr_t)(sc_base + (real ? sc_off + (uint32_t)kb : sc_one_line)),
+                                             (lptr_t)(lds + (real ? sc_dst + ((kb >> 2) & 1) * SCB_BUF : LDS_DUMP)), 16, 0, 0);
+        } else
+            __builtin_amdgcn_global_load_lds((gptr_t)(sc_base + sc_off + (uint32_t)kb),
+                                             (lptr_t)(lds + LDS_SC + stage * SC_STAGE + wave * 256), 4, 0, 0);
     };
-    auto lds_as = [&](int j, int stage) { return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (sub_row(j) + fr) * 4); };
-    auto lds_bs = [&](int stage) { return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (256 + wn) * 4); };
+    // the scales of K block kb (whose slot is `stage`): a_s of the lane's row of sub-tile j, b_s of the wavefront's columns
+    auto lds_as = [&](int j, int stage, int kb) {
+        if constexpr (SCB) return *(const float*)(lds + LDS_SC + ((kb >> 2) & 1) * SCB_BUF + (kb & 3) * 4 + (sub_row(j) + fr) * 16);
+        else return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (sub_row(j) + fr) * 4);
+    };
+    auto lds_bs = [&](int stage, int kb) {
+        if constexpr (SCB) return *(const float*)(lds + LDS_SC + ((kb >> 2) & 1) * SCB_BUF + (kb & 3) * 4 + TM * 16 + wn * 16);
+        else return *(const float*)(lds + LDS_SC + stage * SC_STAGE + (256 + wn) * 4);
+    };
 
     v4f acc[SN][SM];
 #pragma unroll
@@ -398,9 +427,9 @@ __device__ __forceinline__ void prefill_tile(
         // the activations' (B operand, the lane's row)
         int eb, ea[JA], eb_nxt, ea_nxt[JA];
         auto e8m0 = [](float x) { return (int)(f32_as_u32(x) >> 23); };
-        eb_nxt = e8m0(lds_bs(0));
+        eb_nxt = e8m0(lds_bs(0, 0));
 #pragma unroll
-        for (int j = 0; j < JA; ++j) ea_nxt[j] = e8m0(lds_as(j, 0));
+        for (int j = 0; j < JA; ++j) ea_nxt[j] = e8m0(lds_as(j, 0, 0));
         v8i nf0, nf1, mf[JA];
         {
             const uint8_t* as_base = lds + a_rd;
@@ -427,9 +456,9 @@ __device__ __forceinline__ void prefill_tile(
                 if (i == kSync) {
                     __builtin_amdgcn_s_waitcnt(kWaitSync);
                     wg_barrier();
-                    eb_nxt = e8m0(lds_bs(ss_next));
+                    eb_nxt = e8m0(lds_bs(ss_next, kb + 1));
 #pragma unroll
-                    for (int j = 0; j < JA; ++j) ea_nxt[j] = e8m0(lds_as(j, ss_next));
+                    for (int j = 0; j < JA; ++j) ea_nxt[j] = e8m0(lds_as(j, ss_next, kb + 1));
                     issue_scales(kb_a, ahead_s(st_s));
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -468,9 +497,9 @@ __device__ __forceinline__ void prefill_tile(
         } else {
         float sc[JA], sc_nxt[JA];
         {
-            const float bs = lds_bs(0);
+            const float bs = lds_bs(0, 0);
 #pragma unroll
-            for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, 0) * bs;
+            for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, 0, 0) * bs;
 #pragma unroll
             for (int j = 0; j < JA; ++j) sc[j] = 0.f;
         }
@@ -511,9 +540,9 @@ __device__ __forceinline__ void prefill_tile(
                     __builtin_amdgcn_s_waitcnt(kWaitSync);
                     wg_barrier();
                     {
-                        const float bs = lds_bs(ss_next);
+                        const float bs = lds_bs(ss_next, kb + 1);
 #pragma unroll
-                        for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, ss_next) * bs;
+                        for (int j = 0; j < JA; ++j) sc_nxt[j] = lds_as(j, ss_next, kb + 1) * bs;
                     }
                     issue_scales(kb_a, ahead_s(st_s));
                     __builtin_amdgcn_sched_barrier(0);
@@ -709,9 +738,8 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_prefill_kernel(
 // straight from HBM, and a second block of prefetch is what hides that), one with fewer the 128-row
 // configuration with three stages of both.  The choice is uniform over the workgroup and needs no host knowledge of
 // the group sizes: a layer with a few rows per expert and one with hundreds go through the same launch.
-// SCB: a row of a_s is a whole number of 16-byte pieces (K a multiple of 512, a_s 16-byte aligned), so that the slots of
-// more than 192 rows copy their activation scales four K blocks at a time (the smaller slots keep one line per row and
-// K block: with the batch addresses their configurations no longer fit the register file).
+// SCB: the rows of a_s and b_s are whole numbers of aligned 16-byte pieces (K a multiple of 512), so that the tiles
+// copy their scales four K blocks at a time.
 template <int CD, bool P2 = false, bool SG = false, bool SCB = false>
 __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
         const uint8_t* __restrict__ a, const float* __restrict__ a_s,
@@ -726,9 +754,9 @@ __global__ __launch_bounds__(THREADS, 1) void fp8_gemm_grouped_kernel(
         pingpong::tile<CD, P2, true, 4, false, SG, SCB>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, blockIdx.x, g);
     }
     else if (rows > 128)
-        prefill_tile<CD, true, 192, 2, 3, P2, SG>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+        prefill_tile<CD, true, 192, 2, 3, P2, SG, SCB>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
     else
-        prefill_tile<CD, true, 128, 3, 3, P2, SG>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
+        prefill_tile<CD, true, 128, 3, 3, P2, SG, SCB>(a, a_s, b, b_s, c, M, N, K, tiles_m, tiles_n, tn_first, kb_per_split, ldc, g, blockIdx.x);
 }
 
 // Dense GEMM whose last column tiles run as 128-row tiles: the first tiles_m * tn_tall workgroups compute 256-row
@@ -813,8 +841,10 @@ int launch_kernel(const void* a, const float* a_s, const void* b, const float* b
     return launch_status();
 }
 constexpr int kGroupedTileRows = 256;     // slot height of the grouped kernel's tile table
-// whether a row of a_s (K / 128 binary32 values) is a whole number of aligned 16-byte pieces
-inline bool scale_batches_ok(const float* a_s, int64_t k) { return (k / 128) % 4 == 0 && ((uintptr_t)a_s & 15) == 0; }
+// whether the rows of a_s and of every group's b_s (K / 128 binary32 values each) are whole numbers of aligned 16-byte pieces
+inline bool scale_batches_ok(const float* a_s, const float* b_s, int64_t bs_stride, int64_t k) {
+    return (k / 128) % 4 == 0 && (((uintptr_t)a_s | (uintptr_t)b_s) & 15) == 0 && bs_stride % 4 == 0;
+}
 constexpr int64_t kCUs = 256;
 inline int env_tile_rows() { static const int v = [] { const char* e = getenv("DSV3_PREFILL_TILE"); return e ? atoi(e) : 0; }(); return v; }
 }  // namespace
@@ -1051,8 +1081,9 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
         return launch_grouped_skinny(a, a_s, a_rows, b, b_s, c, CD, n, k, num_tiles, tile_group, tile_row0, tile_rows,
                                      b_stride, bs_stride, m < num_tiles ? m : num_tiles, stream);
     GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride, nullptr, nullptr, 0};
-    constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES;               // the largest of the three configurations
-    static_assert(LDS_BYTES >= pingpong::LDS_BYTES_SCB && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES, "LDS of the grouped kernel");
+    constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES_SCB;           // the largest of the three configurations
+    static_assert(LDS_BYTES >= pingpong::LDS_BYTES_SCB && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES_SCB &&
+                  LDS_BYTES >= Cfg<192, 2, 3>::LDS_BYTES && LDS_BYTES >= Cfg<128, 3>::LDS_BYTES, "LDS of the grouped kernel");
     const int64_t tn = (n + BN - 1) / BN;
     if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (num_tiles * tn == 0) return DSV3_OK;
@@ -1065,7 +1096,7 @@ int launch_grouped(const void* a, const float* a_s, const int* a_rows, const voi
         return launch_status();
     };
     static LdsGrant grant, grant_scb;
-    if (scale_batches_ok(a_s, k)) return launch(fp8_gemm_grouped_kernel<CD, P2, false, true>, grant_scb);
+    if (scale_batches_ok(a_s, b_s, bs_stride, k)) return launch(fp8_gemm_grouped_kernel<CD, P2, false, true>, grant_scb);
     return launch(fp8_gemm_grouped_kernel<CD, P2>, grant);
 }
 
@@ -1085,7 +1116,7 @@ int launch_grouped_swiglu(const void* a, const float* a_s, const int* a_rows, co
     using namespace prefill;
     GroupTable g{tile_group, tile_row0, tile_rows, a_rows, b_stride, bs_stride, (uint8_t*)y, s,
                  scale_fmt == DSV3_SCALE_FMT_UE8M0 ? 1 : 0};
-    constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES;
+    constexpr int LDS_BYTES = Cfg<192, 2, 3>::LDS_BYTES_SCB;
     const int64_t tn = inter / 128;
     if ((num_tiles + 8) * tn > 0x7fffffff) return DSV3_ERR_BAD_SHAPE;
     if (num_tiles * tn == 0) return DSV3_OK;
@@ -1098,7 +1129,7 @@ int launch_grouped_swiglu(const void* a, const float* a_s, const int* a_rows, co
         return launch_status();
     };
     static LdsGrant grant, grant_scb;
-    if (scale_batches_ok(a_s, k)) return launch(fp8_gemm_grouped_kernel<DSV3_BF16, false, true, true>, grant_scb);
+    if (scale_batches_ok(a_s, b_s, bs_stride, k)) return launch(fp8_gemm_grouped_kernel<DSV3_BF16, false, true, true>, grant_scb);
     return launch(fp8_gemm_grouped_kernel<DSV3_BF16, false, true>, grant);
 }
 
