@@ -341,7 +341,7 @@ def test_moe_grouped_matches_expert_loop_and_oracle(K, tokens):
             y_grouped = moe(x.cuda())                   # 300 tokens: the shared expert rides along as group 8
             assert moe._stacked is not None and moe.experts[3].w1.weight.data_ptr() == moe._stacked[0][3].data_ptr()
             assert moe._shared_stacked and moe.shared_experts.w2.weight.data_ptr() == moe._stacked[2][8].data_ptr()
-            moe.fuse_swiglu_epilogue = True             # SwiGLU + act_quant in the first GEMM's epilogue: the same bits
+            moe.fuse_swiglu_epilogue = False            # SwiGLU + act_quant as a kernel of their own: the same bits
             assert torch.equal(moe(x.cuda()), y_grouped)
             del moe.fuse_swiglu_epilogue
             moe.fold_shared_max_tokens = 0              # the shared expert as three dense linears instead
