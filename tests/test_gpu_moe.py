@@ -57,7 +57,7 @@ def _grouped_case(counts, n, k, seed, gather):
     ([129, 64], 576, 256, False),            # ragged n: 576 = 2 tiles + 64, 5 scale rows
     ([40] * 6, 256, 1152, True),             # odd number of K blocks
     ([145, 177, 200, 241, 17], 512, 384, True),   # 256-row slots with 10, 12, 13 and 16 live sub-tiles, then a small one
-    ([300, 7, 250, 193], 256, 1536, True),   # 256-row slots, 12 K blocks: activation scales in three batches of four blocks
+    ([300, 7, 250, 193, 150, 100], 256, 1536, True),   # every tile configuration, 12 K blocks: scales in three batches of four blocks
     ([1] * 9, 4096, 7168, True),             # one token of the MoE layer: the weight-streaming kernel (up to 320 rows in all)
     ([2, 0, 1, 5, 0, 3], 7168, 2048, False), # ... its second GEMM shape, ragged group sizes, no gather
     ([20, 3, 13], 200, 640, True),           # ... a slot of more than 16 rows (two passes), n not a multiple of 32
@@ -186,7 +186,8 @@ def test_fp8_gemm_grouped_seeded_tables(K):
 
 
 @pytest.mark.parametrize("counts,n,k", [([5, 0, 300, 256, 1], 384, 512), ([145, 177, 200, 241, 17], 512, 384),
-                                        ([3, 2, 9], 256, 256)])
+                                        ([3, 2, 9], 256, 256),
+                                        ([300, 7, 150, 193, 100], 256, 1536)])   # scales in three batches of four K blocks
 def test_fp8_gemm_grouped_power_of_two_scales(K, counts, n, k):
     """Scales that are powers of two on both sides: the grouped tile kernel hands them to the matrix instruction
     (every tile configuration), a small launch takes the weight-streaming kernel as before."""
