@@ -218,8 +218,9 @@ __device__ __forceinline__ void tile(
     // every wavefront issues the same number of copies per block without asking the memory pipeline for more lines).
     // a_s[row, kb] sits 4 KBT bytes from a_s[row + 1, kb]: the 64 scales of a copy are 64 memory lines, a third of all
     // the lines a workgroup asks for, and they slow the phase after the one that requests them by 80-100 cycles (with
-    // one line per copy, results aside, a K block takes 2 % less).  Copying them for four K blocks at a time (16 bytes
-    // per row, a one-line copy in the other three blocks to keep the counts) was built and was not faster.
+    // one line per copy, results aside, a K block of a dense problem takes 2 % less).  Copying them for four K blocks at
+    // a time (16 bytes per row, a one-line copy in the other three blocks to keep the counts) was not faster there, where
+    // both operands come from the caches; in grouped mode it is (below).
     const int nb_last = (N - 1) / 128;
     const float* sc_base = wave < 4 ? a_s : b_s;
     const int b_scale_row = SG ? sg_scale_row(wave == 4 ? min(lane, 1) : 0, tn_idx, N / 2)

@@ -88,6 +88,40 @@ def test_fp8_gemm_grouped_vs_oracle(K, counts, n, k, gather):
         row += c
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_fp8_gemm_grouped_seeded_sweep(K, seed):
+    """Random group sizes (empty groups, one row, several slots per group), n and k: every tile configuration, launches
+    of the weight-streaming kernel (up to 320 rows in all), K ranges with and without whole batches of four scale
+    blocks, ragged n.  Every group against the oracle."""
+    from dsv3fp8 import ops
+    r = torch.Generator().manual_seed(100 + seed)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=r))
+    small = seed % 4 == 0                                     # a launch of the weight-streaming kernel
+    groups = pick(1, 7) if small else pick(3, 7)
+    top = (30, 140, 200, 420)[seed % 4]                       # ... then slots of every height
+    counts = [0 if pick(0, 5) == 0 else pick(1, top) for _ in range(groups)]
+    counts[0] = max(counts[0], 1 if small else 330)
+    n = 16 * pick(1, 40)
+    k = 512 * pick(1, 4) if seed & 2 else 128 * pick(1, 16)   # whole batches of four scale blocks, or any K
+    gather = bool(seed & 1)
+    xq, xs, w, a_rows = _grouped_case(counts, n, k, 200 + seed, gather)
+    rows = sum(counts)
+    R, tg, t0, tr = _tables(counts, rows // ops.grouped_tile_rows() + len(counts))
+    b = torch.stack([wi[0].view(torch.uint8) for wi in w]).view(FP8).cuda()
+    b_s = torch.stack([wi[1] for wi in w]).cuda()
+    out = torch.ops.dsv3fp8.fp8_gemm_grouped(xq.cuda(), xs.cuda(), a_rows.cuda() if gather else None, b, b_s, rows,
+                                             tg, t0, tr, ops.dtype_code(torch.float32)).cpu()
+    row = 0
+    for gi, c in enumerate(counts):
+        if c == 0:
+            continue
+        idx = a_rows[row:row + c].long() if gather else torch.arange(row, row + c)
+        ref = oracle.fp8_gemm_f32(xq[idx], xs[idx], w[gi][0], w[gi][1])
+        err = (out[row:row + c] - ref).abs().max().item()
+        assert err <= 1e-2 * ref.pow(2).mean().sqrt().item(), (counts, n, k, gi, err)     # tolerance of the fp32 output
+        row += c
+
+
 def test_fp8_gemm_grouped_scale_batches_need_aligned_scales(K):
     """A row of a_s that is a whole number of 16-byte pieces lets the 256-row slots copy the scales of four K blocks
     at a time; the same a_s four bytes further on in memory takes the one-line copies.  Same bits either way."""
