@@ -534,11 +534,12 @@ def moe_stages(moe, x, Mdl):
     out = t("grouped_w2", lambda: g(gq, gs, None, w2, s2, pairs, tile_group, tile_row0, tile_rows, code))
     z = t("shared_expert", lambda: moe.shared_experts(x, (xq, xs)).contiguous())
     t("moe_combine", lambda: torch.ops.dsv3fp8.moe_combine(out, rows, w_sorted, z))
-    st["sum"] = round(sum(st.values()), 1)
     # the first GEMM with the activation and the re-quantisation in its epilogue, which is what MoE.forward runs
-    # (MoE.fuse_swiglu_epilogue) in place of grouped_w1w3 + swiglu_quant; not in the sum
+    # (MoE.fuse_swiglu_epilogue) in place of grouped_w1w3 + swiglu_quant
     st["w1w3_with_swiglu_epilogue"] = round(time_loop(lambda: torch.ops.dsv3fp8.fp8_gemm_grouped_swiglu(
         xq, xs, a_rows, w13, s13, pairs, tile_group, tile_row0, tile_rows, 0), 10, 2) * 1e3, 1)
+    # the launches of one forward: the fused first GEMM counts, the two-call form beside it does not
+    st["sum"] = round(sum(v for k, v in st.items() if k not in ("grouped_w1w3", "swiglu_quant")), 1)
     return st
 
 
